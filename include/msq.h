@@ -1,0 +1,87 @@
+/* libmsq: MI355X (gfx950) quantized matvec / MoE kernels over raw GGUF blocks -- C ABI.
+ *
+ * Drop-in boundary for the "quant" operator module of MacSeek (reference: src/kernels/quant.hpp). Every entry point
+ * below names the reference function it replaces. Conventions carried over from the reference:
+ *   - functions only ENQUEUE work on the given stream (reference: "only encode; never commit/wait", quant.hpp:3);
+ *     `stream` is a hipStream_t passed as void* (NULL = the default stream). Dependent calls on one stream are
+ *     ordered by the stream, so the reference's explicit Enc::barrier() between them has no counterpart.
+ *   - weights are raw GGUF block rows: an [in -> out] matrix is rows = out rows of cols = in elements
+ *     (quant.hpp:4); weight bases need 4-byte alignment only, activations / outputs 16-byte alignment
+ *     (docs/modules/quant.md:27-30). Activations must be finite and inside the fp16 range (they are staged as
+ *     fp16 pairs for the block formats, as the reference does for its n > 1 paths).
+ *   - all buffers are caller-owned device memory; MsqBuffer mirrors ms::Buffer {buf, off, size}
+ *     (src/core/metal.hpp:11-18).
+ *   - misuse is reported, not aborted: functions return 0 on success or a negative MSQ_ERR_* code and leave a
+ *     message for msq_last_error(). The C++ shim (include/macseek_amd/quant.hpp) turns a non-zero status into the
+ *     reference's behaviour: print "macseek quant: ... unsupported" and abort() (src/kernels/quant.mm:34-37).
+ */
+#ifndef MSQ_H
+#define MSQ_H
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ggml type ids (reference: src/kernels/quant_types.hpp:9-11) */
+enum {
+  MSQ_T_F32 = 0, MSQ_T_F16 = 1, MSQ_T_Q8_0 = 8, MSQ_T_Q5_K = 13, MSQ_T_Q6_K = 14, MSQ_T_IQ2_XXS = 16,
+  MSQ_T_IQ1_S = 19, MSQ_T_IQ4_NL = 20, MSQ_T_BF16 = 30
+};
+
+enum {
+  MSQ_OK = 0,
+  MSQ_ERR_UNSUPPORTED = -1, /* type / shape / combination the kernels do not cover (reference: die()) */
+  MSQ_ERR_ARGUMENT = -2,    /* null buffer, size too small, count out of range */
+  MSQ_ERR_SCRATCH = -3,     /* caller scratch smaller than *_scratch_bytes() */
+  MSQ_ERR_HIP = -4          /* HIP runtime / launch error (text in msq_last_error) */
+};
+
+/* reference: ms::Buffer (src/core/metal.hpp:11-18): device allocation base, byte offset, usable bytes from off */
+typedef struct MsqBuffer { void* dev; size_t off; size_t size; } MsqBuffer;
+
+/* reference: ms::q::MvCfg (quant.hpp:12). Launch shape of the decode matvec, 0 = auto:
+ * nr = rows one wave computes per tile, rsg = row-waves per workgroup, ks = waves splitting K inside a workgroup.
+ * nr and rsg never change a row's summation order; ks does. */
+typedef struct MsqMvCfg { int nr, rsg, ks; } MsqMvCfg;
+
+/* Library / device bring-up (no reference counterpart: Metal pipelines are created lazily by ms::Device). Optional:
+ * every entry point initialises on first use. Returns MSQ_OK or MSQ_ERR_HIP. */
+int msq_init(void);
+/* Last error message of the calling thread ("" if none). */
+const char* msq_last_error(void);
+/* 1 when the library was built for, and runs on, a gfx950 device. */
+int msq_device_ok(void);
+
+/* reference: block_elems / block_bytes / row_bytes / type_name (src/kernels/quant_types.hpp:13-43) */
+int msq_block_elems(int qtype);
+size_t msq_block_bytes(int qtype);
+size_t msq_row_bytes(int qtype, int64_t cols);
+const char* msq_type_name(int qtype);
+
+/* reference: ms::q::matvec_supported (quant.hpp:14, quant.mm:68). Additionally true for IQ4_NL, for which the
+ * reference has no GPU matvec (quant.mm:22-29). */
+int msq_matvec_supported(int qtype);
+
+/* reference: ms::q::matvec_cfg (quant.hpp:16-18, quant.mm:97-105): the launch shape msq_matvec would use. Row
+ * chunks of one matrix that all pass this shape produce bit-identical rows. */
+int msq_matvec_cfg(int qtype, int rows, int cols, MsqMvCfg* out);
+
+/* reference: ms::q::encode_matvec (quant.hpp:29-30, quant.mm:70-95).
+ * y[rows] (+)= W[rows x cols] . x[cols]; groups > 1 = block-diagonal: rows split into `groups` equal row groups,
+ * group g reads x[g*cols .. g*cols + cols). cfg may be NULL. Errors (reference aborts): unsupported type,
+ * cols not a multiple of the block size (256 for K/IQ/dense types, 32 for Q8_0 / IQ4_NL), groups < 1,
+ * rows % groups != 0. */
+int msq_matvec(void* stream, int qtype, const MsqBuffer* W, int rows, int cols, const MsqBuffer* x,
+               const MsqBuffer* y, int accumulate, int groups, const MsqMvCfg* cfg);
+
+/* Whole-buffer dequantization to fp32, bit-exact with the reference's CPU dequantizer
+ * (reference: ref::dequant_row, tests/ref/dequant.cpp:34-120; GPU relative: q_deq_f16, quant_mm.metal:143-154).
+ * n_elems must be a multiple of the block size; out holds n_elems floats. */
+int msq_dequant(void* stream, int qtype, const MsqBuffer* W, int64_t n_elems, const MsqBuffer* out);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MSQ_H */

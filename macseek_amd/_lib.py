@@ -1,0 +1,73 @@
+"""ctypes binding of libmsq.so (the C ABI declared in include/msq.h). Fails loudly when the library is absent."""
+import ctypes as C
+import os
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+SO = os.path.join(HERE, "libmsq.so")
+
+
+class MsqBuffer(C.Structure):
+    _fields_ = [("dev", C.c_void_p), ("off", C.c_size_t), ("size", C.c_size_t)]
+
+
+class MsqMvCfg(C.Structure):
+    _fields_ = [("nr", C.c_int), ("rsg", C.c_int), ("ks", C.c_int)]
+
+
+class MsqExpertSlot(C.Structure):
+    _fields_ = [("gate", MsqBuffer), ("up", MsqBuffer), ("down", MsqBuffer)]
+
+
+MSQ_MAX_ROUTED = 6
+
+
+class MsqMoeDecodeArgs(C.Structure):
+    _fields_ = [("t_gate_up", C.c_int), ("t_down", C.c_int), ("n_routed", C.c_int),
+                ("slot", MsqExpertSlot * MSQ_MAX_ROUTED), ("weights", MsqBuffer), ("has_shared", C.c_int),
+                ("t_shared", C.c_int), ("shared", MsqExpertSlot), ("x", MsqBuffer), ("y", MsqBuffer),
+                ("scratch", MsqBuffer), ("gu_nr", C.c_int), ("gu_rsg", C.c_int), ("d_nr", C.c_int), ("d_rsg", C.c_int),
+                ("dim", C.c_int), ("inter", C.c_int)]
+
+
+class MsqMoePrefillArgs(C.Structure):
+    _fields_ = [("t_gate_up", C.c_int), ("t_down", C.c_int), ("n_tokens", C.c_int), ("n_exp", C.c_int),
+                ("slots", C.POINTER(MsqExpertSlot)), ("offs", C.POINTER(C.c_int)), ("tok", MsqBuffer), ("wt", MsqBuffer),
+                ("slot_of", MsqBuffer), ("k_per_token", C.c_int), ("has_shared", C.c_int), ("t_shared", C.c_int),
+                ("shared", MsqExpertSlot), ("X", MsqBuffer), ("Y", MsqBuffer), ("scratch", MsqBuffer),
+                ("path", C.c_int), ("shared_dense", C.c_int), ("dim", C.c_int), ("inter", C.c_int),
+                ("x_is_bf16", C.c_int)]
+
+
+_lib = None
+
+# name -> (restype, argtypes); every symbol include/msq.h declares
+_BP = C.POINTER(MsqBuffer)
+SIGNATURES = {
+    "msq_init": (C.c_int, []),
+    "msq_last_error": (C.c_char_p, []),
+    "msq_device_ok": (C.c_int, []),
+    "msq_block_elems": (C.c_int, [C.c_int]),
+    "msq_block_bytes": (C.c_size_t, [C.c_int]),
+    "msq_row_bytes": (C.c_size_t, [C.c_int, C.c_int64]),
+    "msq_type_name": (C.c_char_p, [C.c_int]),
+    "msq_matvec_supported": (C.c_int, [C.c_int]),
+    "msq_matvec_cfg": (C.c_int, [C.c_int, C.c_int, C.c_int, C.POINTER(MsqMvCfg)]),
+    "msq_matvec": (C.c_int, [C.c_void_p, C.c_int, _BP, C.c_int, C.c_int, _BP, _BP, C.c_int, C.c_int, C.POINTER(MsqMvCfg)]),
+    "msq_dequant": (C.c_int, [C.c_void_p, C.c_int, _BP, C.c_int64, _BP]),
+}
+
+
+def load():
+    """The loaded library. Raises if libmsq.so has not been built (python -m macseek_amd.build)."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(SO):
+            raise RuntimeError("macseek_amd: %s is missing; build it with `python -m macseek_amd.build` "
+                               "(there is no CPU fallback)" % SO)
+        L = C.CDLL(SO)
+        for name, (res, args) in SIGNATURES.items():
+            fn = getattr(L, name)  # AttributeError if the library does not export a declared symbol
+            fn.restype = res
+            fn.argtypes = args
+        _lib = L
+    return _lib

@@ -1,0 +1,468 @@
+// Device-side building blocks for gfx950 (wave64): codebook tables, unaligned block loads, DPP wave reduction and the
+// per-format block decoders used by the decode (n = 1) kernels.
+//
+// Block byte layouts and element order follow the GGUF formats as restated by the reference's CPU dequantizer
+// (tests/ref/dequant.cpp:34-120). Lane/unit mappings are this library's own: one lane owns a UNIT-column slice of a
+// row (32 columns for the block formats) and keeps the matching activations in registers as fp16 pairs, so a row
+// costs one packed dot (v_dot2_f32_f16) per two weights plus the decode.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "iq_codebooks.h"
+#include "msq_types.h"
+
+namespace msq {
+
+typedef _Float16 h2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 h8_t __attribute__((ext_vector_type(8)));
+typedef float f4_t __attribute__((ext_vector_type(4)));
+
+constexpr int kWave = 64;
+
+// ------------------------------------------------------------------------------------------------ constant tables
+// fp16 images of the codebooks, expanded at compile time from the base-3 packed form.
+struct TblIQ1S { uint32_t w[MSQ_IQ1S_GRID_N * 4]; };      // 8 halves (-1, 0, +1) per entry
+struct TblIQ2XXS { uint32_t w[MSQ_IQ2XXS_GRID_N * 4]; };  // 8 halves (8, 25, 43) per entry
+struct TblSign { uint32_t w[128 * 4]; };                  // 8 fp16 sign-bit masks per 7-bit sign index
+struct TblIQ4NL { uint32_t w[256]; };                     // byte -> {half(kv[lo nibble]), half(kv[hi nibble])}
+
+constexpr uint16_t half_of_small_int(int v) {  // exact fp16 bits of an integer |v| < 2048
+  if (v == 0) return 0;
+  const uint16_t s = v < 0 ? 0x8000 : 0;
+  unsigned a = v < 0 ? (unsigned)-v : (unsigned)v;
+  int e = 0;
+  while ((a >> (e + 1)) != 0) e++;
+  const unsigned man = (a << (10 - e)) & 0x3FFu;
+  return (uint16_t)(s | (unsigned)((e + 15) << 10) | man);
+}
+constexpr TblIQ1S make_iq1s() {
+  TblIQ1S t{};
+  constexpr uint16_t hv[3] = {0xBC00, 0x0000, 0x3C00};
+  for (int i = 0; i < MSQ_IQ1S_GRID_N; i++) {
+    unsigned c = msq_iq1s_code[i];
+    for (int j = 0; j < 4; j++) {
+      const uint32_t lo = hv[c % 3]; c /= 3;
+      const uint32_t hi = hv[c % 3]; c /= 3;
+      t.w[4 * i + j] = lo | (hi << 16);
+    }
+  }
+  return t;
+}
+constexpr TblIQ2XXS make_iq2xxs() {
+  TblIQ2XXS t{};
+  constexpr uint16_t hv[3] = {half_of_small_int(8), half_of_small_int(25), half_of_small_int(43)};
+  for (int i = 0; i < MSQ_IQ2XXS_GRID_N; i++) {
+    unsigned c = msq_iq2xxs_code[i];
+    for (int j = 0; j < 4; j++) {
+      const uint32_t lo = hv[c % 3]; c /= 3;
+      const uint32_t hi = hv[c % 3]; c /= 3;
+      t.w[4 * i + j] = lo | (hi << 16);
+    }
+  }
+  return t;
+}
+constexpr TblSign make_sign() {  // ksigns_iq2xs[i] = i | parity(i) << 7; bit j set => element j negative
+  TblSign t{};
+  for (int i = 0; i < 128; i++) {
+    int par = 0;
+    for (int b = 0; b < 7; b++) par ^= (i >> b) & 1;
+    const unsigned s = (unsigned)i | ((unsigned)par << 7);
+    for (int j = 0; j < 4; j++)
+      t.w[4 * i + j] = ((s >> (2 * j)) & 1 ? 0x8000u : 0u) | ((s >> (2 * j + 1)) & 1 ? 0x80000000u : 0u);
+  }
+  return t;
+}
+constexpr int kIQ4NLValues[16] = {-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113};
+constexpr TblIQ4NL make_iq4nl() {
+  TblIQ4NL t{};
+  for (int b = 0; b < 256; b++)
+    t.w[b] = (uint32_t)half_of_small_int(kIQ4NLValues[b & 15]) | ((uint32_t)half_of_small_int(kIQ4NLValues[b >> 4]) << 16);
+  return t;
+}
+
+__device__ __attribute__((aligned(16))) const TblIQ1S g_tbl_iq1s = make_iq1s();
+__device__ __attribute__((aligned(16))) const TblIQ2XXS g_tbl_iq2xxs = make_iq2xxs();
+__device__ __attribute__((aligned(16))) const TblSign g_tbl_sign = make_sign();
+__device__ __attribute__((aligned(16))) const TblIQ4NL g_tbl_iq4nl = make_iq4nl();
+
+// ------------------------------------------------------------------------------------------------ loads
+// GGUF blocks are only 2-byte aligned (34/50/66/210-byte blocks, matrices placed at 4-byte offsets); gfx950 global
+// loads accept any alignment, so wider-than-alignment loads are expressed through under-aligned types.
+typedef uint32_t __attribute__((aligned(2), may_alias)) u32_a2;
+struct __attribute__((packed, aligned(2))) u64_a2 { uint32_t x, y; };
+struct __attribute__((packed, aligned(2))) u128_a2 { uint32_t x, y, z, w; };
+
+__device__ __forceinline__ uint32_t ld8(const uint8_t* p) { return *p; }
+__device__ __forceinline__ uint32_t ld16(const uint8_t* p) { return *(const uint16_t*)p; }
+__device__ __forceinline__ uint32_t ld32(const uint8_t* p) { return *(const u32_a2*)p; }
+__device__ __forceinline__ u64_a2 ld64(const uint8_t* p) { return *(const u64_a2*)p; }
+__device__ __forceinline__ u128_a2 ld128(const uint8_t* p) { return *(const u128_a2*)p; }
+
+__device__ __forceinline__ float half_bits_to_float(uint32_t b) {
+  return (float)__builtin_bit_cast(_Float16, (uint16_t)b);
+}
+__device__ __forceinline__ float bf16_bits_to_float(uint32_t b) { return __builtin_bit_cast(float, b << 16); }
+__device__ __forceinline__ h2_t as_h2(uint32_t v) { return __builtin_bit_cast(h2_t, v); }
+__device__ __forceinline__ uint32_t pack_h2(float a, float b) {
+  h2_t v = {(_Float16)a, (_Float16)b};
+  return __builtin_bit_cast(uint32_t, v);
+}
+__device__ __forceinline__ float dot2(uint32_t w, uint32_t x, float acc) {
+  return __builtin_amdgcn_fdot2(as_h2(w), as_h2(x), acc, false);
+}
+// bytes b0,b1 (sel_lo) or b2,b3 (sel_hi) of q become the halves 1024 + b (0x6400 | b)
+__device__ __forceinline__ uint32_t bytes01_to_h2_1024(uint32_t q) { return __builtin_amdgcn_perm(0x64646464u, q, 0x04010400u); }
+__device__ __forceinline__ uint32_t bytes23_to_h2_1024(uint32_t q) { return __builtin_amdgcn_perm(0x64646464u, q, 0x04030402u); }
+
+// ------------------------------------------------------------------------------------------------ wave reduction
+template <int CTRL, int ROW_MASK = 0xF>
+__device__ __forceinline__ float dpp_add(float v) {
+  const int moved = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, ROW_MASK, 0xF, false);
+  return v + __builtin_bit_cast(float, moved);
+}
+// Sum over the 64 lanes of a wave; the total is returned in every lane (broadcast through a scalar register).
+__device__ __forceinline__ float wave_sum(float v) {
+  v = dpp_add<0xB1>(v);        // quad_perm [1,0,3,2]
+  v = dpp_add<0x4E>(v);        // quad_perm [2,3,0,1]
+  v = dpp_add<0x141>(v);       // row_half_mirror
+  v = dpp_add<0x140>(v);       // row_mirror: every lane of a 16-lane row holds the row sum
+  v = dpp_add<0x142, 0xA>(v);  // row_bcast15 into rows 1 and 3
+  v = dpp_add<0x143, 0xC>(v);  // row_bcast31 into rows 2 and 3: lane 63 holds the total
+  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
+}
+
+// ------------------------------------------------------------------------------------------------ LDS table copies
+__device__ __forceinline__ void copy_words16(uint32_t* dst, const uint32_t* src, int nwords, int tid, int nthreads) {
+  const uint4* s = (const uint4*)src;
+  uint4* d = (uint4*)dst;
+  for (int i = tid; i < nwords / 4; i += nthreads) d[i] = s[i];
+}
+
+// ------------------------------------------------------------------------------------------------ x slices
+// 32 consecutive activations -> 16 fp16 pairs (round to nearest even) + the sum of the rounded values
+struct X32 {
+  uint32_t v[16];
+  float sx;
+};
+__device__ __forceinline__ void load_x32_consecutive(const float* x, uint32_t* v, int n) {
+  const float4* p = (const float4*)x;
+#pragma unroll
+  for (int i = 0; i < n / 4; i++) {
+    const float4 f = p[i];
+    v[2 * i] = pack_h2(f.x, f.y);
+    v[2 * i + 1] = pack_h2(f.z, f.w);
+  }
+}
+__device__ __forceinline__ float sum_h2(const uint32_t* v, int n) {
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < n; i++) {
+    const h2_t h = as_h2(v[i]);
+    s += (float)h.x + (float)h.y;
+  }
+  return s;
+}
+
+// ================================================================================================ decoders (n = 1)
+// Interface of a decoder D:
+//   UNIT            columns one lane owns per unit
+//   LDS_WORDS       32-bit words of table the workgroup stages in LDS (0 = none)
+//   fill_lds()      cooperative table copy
+//   X / load_x()    the lane's activation slice for unit u of a row (x points at the row's first activation)
+//   Raw / load()    the raw block bytes of unit u of a weight row (global loads only, so callers can prefetch)
+//   dot()           sum over the unit's columns of weight * activation, fp32
+
+// ---- IQ1_S: {fp16 d; u8 qs[32]; u16 qh[8]}, 50 bytes / 256 weights; unit = one 32-weight sub-block
+struct DecIQ1S {
+  static constexpr int UNIT = 32, LDS_WORDS = MSQ_IQ1S_GRID_N * 4;
+  typedef X32 X;
+  struct Raw { uint32_t qs, qh, d; };
+  __device__ static void fill_lds(uint32_t* lds, int tid, int nt) { copy_words16(lds, g_tbl_iq1s.w, LDS_WORDS, tid, nt); }
+  __device__ static X load_x(const float* x, uint32_t u) {
+    X r;
+    load_x32_consecutive(x + 32u * u, r.v, 32);
+    r.sx = sum_h2(r.v, 16);
+    return r;
+  }
+  __device__ static Raw load(const uint8_t* row, uint32_t u) {
+    const uint8_t* b = row + (u >> 3) * 50u;
+    const uint32_t ib = u & 7u;
+    return {ld32(b + 2 + 4 * ib), ld16(b + 34 + 2 * ib), ld16(b)};
+  }
+  __device__ static float dot(const Raw& r, const X& x, const uint32_t* lds) {
+    const uint4* grid = (const uint4*)lds;
+    float acc = 0.f;
+#pragma unroll
+    for (int l = 0; l < 4; l++) {
+      const uint32_t idx = ((r.qs >> (8 * l)) & 0xFFu) | (((r.qh >> (3 * l)) & 7u) << 8);
+      const uint4 g = grid[idx];
+      acc = dot2(g.x, x.v[4 * l + 0], acc);
+      acc = dot2(g.y, x.v[4 * l + 1], acc);
+      acc = dot2(g.z, x.v[4 * l + 2], acc);
+      acc = dot2(g.w, x.v[4 * l + 3], acc);
+    }
+    const float dl = half_bits_to_float(r.d) * (float)(2u * ((r.qh >> 12) & 7u) + 1u);
+    const float delta = (r.qh & 0x8000u) ? -0.125f : 0.125f;
+    return dl * (acc + delta * x.sx);
+  }
+};
+
+// ---- IQ2_XXS: {fp16 d; u16 qs[32]}, 66 bytes / 256 weights; unit = one 32-weight sub-block (8 bytes)
+struct DecIQ2XXS {
+  static constexpr int UNIT = 32, LDS_WORDS = MSQ_IQ2XXS_GRID_N * 4 + 128 * 4;
+  typedef X32 X;
+  struct Raw { uint32_t a0, a1, d; };
+  __device__ static void fill_lds(uint32_t* lds, int tid, int nt) {
+    copy_words16(lds, g_tbl_iq2xxs.w, MSQ_IQ2XXS_GRID_N * 4, tid, nt);
+    copy_words16(lds + MSQ_IQ2XXS_GRID_N * 4, g_tbl_sign.w, 128 * 4, tid, nt);
+  }
+  __device__ static X load_x(const float* x, uint32_t u) {
+    X r;
+    load_x32_consecutive(x + 32u * u, r.v, 32);
+    r.sx = 0.f;
+    return r;
+  }
+  __device__ static Raw load(const uint8_t* row, uint32_t u) {
+    const uint8_t* b = row + (u >> 3) * 66u;
+    const u64_a2 a = ld64(b + 2 + 8 * (u & 7u));
+    return {a.x, a.y, ld16(b)};
+  }
+  __device__ static float dot(const Raw& r, const X& x, const uint32_t* lds) {
+    const uint4* grid = (const uint4*)lds;
+    const uint4* sign = (const uint4*)(lds + MSQ_IQ2XXS_GRID_N * 4);
+    float acc = 0.f;
+#pragma unroll
+    for (int l = 0; l < 4; l++) {
+      const uint4 g = grid[(r.a0 >> (8 * l)) & 0xFFu];
+      const uint4 s = sign[(r.a1 >> (7 * l)) & 127u];
+      acc = dot2(g.x ^ s.x, x.v[4 * l + 0], acc);
+      acc = dot2(g.y ^ s.y, x.v[4 * l + 1], acc);
+      acc = dot2(g.z ^ s.z, x.v[4 * l + 2], acc);
+      acc = dot2(g.w ^ s.w, x.v[4 * l + 3], acc);
+    }
+    const float db = half_bits_to_float(r.d) * (0.5f + (float)(r.a1 >> 28)) * 0.25f;
+    return db * acc;
+  }
+};
+
+// ---- Q8_0: {fp16 d; int8 qs[32]}, 34 bytes / 32 weights; unit = one block, activations kept in fp32
+struct DecQ8_0 {
+  static constexpr int UNIT = 32, LDS_WORDS = 0;
+  struct X { float v[32]; };
+  struct Raw { uint32_t q[8]; uint32_t d; };
+  __device__ static void fill_lds(uint32_t*, int, int) {}
+  __device__ static X load_x(const float* x, uint32_t u) {
+    X r;
+    const float4* p = (const float4*)(x + 32u * u);
+#pragma unroll
+    for (int i = 0; i < 8; i++) { const float4 f = p[i]; r.v[4 * i] = f.x; r.v[4 * i + 1] = f.y; r.v[4 * i + 2] = f.z; r.v[4 * i + 3] = f.w; }
+    return r;
+  }
+  __device__ static Raw load(const uint8_t* row, uint32_t u) {
+    const uint8_t* b = row + u * 34u;
+    const u128_a2 a = ld128(b + 2), c = ld128(b + 18);
+    return {{a.x, a.y, a.z, a.w, c.x, c.y, c.z, c.w}, ld16(b)};
+  }
+  __device__ static float dot(const Raw& r, const X& x, const uint32_t*) {
+    float acc = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+      const uint32_t q = r.q[i];
+      acc += (float)(int8_t)(q & 0xFF) * x.v[4 * i];
+      acc += (float)(int8_t)((q >> 8) & 0xFF) * x.v[4 * i + 1];
+      acc += (float)(int8_t)((q >> 16) & 0xFF) * x.v[4 * i + 2];
+      acc += (float)(int8_t)(q >> 24) * x.v[4 * i + 3];
+    }
+    return half_bits_to_float(r.d) * acc;
+  }
+};
+
+// ---- IQ4_NL: {fp16 d; u8 qs[16]}, 18 bytes / 32 weights; byte j holds columns j (low nibble) and j + 16 (high)
+struct DecIQ4NL {
+  static constexpr int UNIT = 32, LDS_WORDS = 256;
+  struct X { uint32_t v[16]; };  // pair j = (x[j], x[j + 16])
+  struct Raw { uint32_t q[4]; uint32_t d; };
+  __device__ static void fill_lds(uint32_t* lds, int tid, int nt) { copy_words16(lds, g_tbl_iq4nl.w, 256, tid, nt); }
+  __device__ static X load_x(const float* x, uint32_t u) {
+    X r;
+    const float4* p = (const float4*)(x + 32u * u);
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      const float4 a = p[i], b = p[i + 4];
+      r.v[4 * i] = pack_h2(a.x, b.x); r.v[4 * i + 1] = pack_h2(a.y, b.y);
+      r.v[4 * i + 2] = pack_h2(a.z, b.z); r.v[4 * i + 3] = pack_h2(a.w, b.w);
+    }
+    return r;
+  }
+  __device__ static Raw load(const uint8_t* row, uint32_t u) {
+    const uint8_t* b = row + u * 18u;
+    const u128_a2 a = ld128(b + 2);
+    return {{a.x, a.y, a.z, a.w}, ld16(b)};
+  }
+  __device__ static float dot(const Raw& r, const X& x, const uint32_t* lds) {
+    float acc = 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+#pragma unroll
+      for (int k = 0; k < 4; k++) acc = dot2(lds[(r.q[i] >> (8 * k)) & 0xFFu], x.v[4 * i + k], acc);
+    }
+    return half_bits_to_float(r.d) * acc;
+  }
+};
+
+// ---- Q6_K: {u8 ql[128]; u8 qh[64]; int8 sc[16]; fp16 d}, 210 bytes / 256 weights.
+// Unit j of a block (8 per block): half h = j >> 2, l0 = 8 * (j & 3); it owns the four 8-column runs
+// 128 h + 32 k + l0 .. + 7 (k = 0..3), which share the bytes ql[64 h + l0 ..], ql[64 h + 32 + l0 ..], qh[32 h + l0 ..].
+struct DecQ6K {
+  static constexpr int UNIT = 32, LDS_WORDS = 0;
+  struct X { uint32_t v[16]; float sx[4]; };
+  struct Raw { uint32_t qa[2], qb[2], qh[2], sc[2], d; };
+  __device__ static void fill_lds(uint32_t*, int, int) {}
+  __device__ static X load_x(const float* x, uint32_t u) {
+    X r;
+    const uint32_t j = u & 7u;
+    const float* base = x + 256u * (u >> 3) + 128u * (j >> 2) + 8u * (j & 3u);
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+      load_x32_consecutive(base + 32 * k, r.v + 4 * k, 8);
+      r.sx[k] = sum_h2(r.v + 4 * k, 4);
+    }
+    return r;
+  }
+  __device__ static Raw load(const uint8_t* row, uint32_t u) {
+    const uint8_t* b = row + (u >> 3) * 210u;
+    const uint32_t j = u & 7u, h = j >> 2, l0 = 8u * (j & 3u);
+    const u64_a2 a = ld64(b + 64 * h + l0), c = ld64(b + 64 * h + 32 + l0), q = ld64(b + 128 + 32 * h + l0);
+    const u64_a2 s = ld64(b + 192 + 8 * h);
+    return {{a.x, a.y}, {c.x, c.y}, {q.x, q.y}, {s.x, s.y}, ld16(b + 208)};
+  }
+  __device__ static float dot(const Raw& r, const X& x, const uint32_t*, uint32_t u) {
+    const uint32_t is = (u >> 1) & 1u;  // l0 / 16
+    const float d = half_bits_to_float(r.d);
+    float total = 0.f;
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+      float acc = 0.f;
+#pragma unroll
+      for (int w = 0; w < 2; w++) {
+        const uint32_t src = (k & 1) ? r.qb[w] : r.qa[w];
+        const uint32_t n = (src >> (4 * (k >> 1))) & 0x0F0F0F0Fu;
+        const uint32_t hb = ((r.qh[w] >> (2 * k)) & 0x03030303u) << 4;
+        const uint32_t q = n | hb;  // 4 bytes in 0..63
+        acc = dot2(bytes01_to_h2_1024(q), x.v[4 * k + 2 * w], acc);
+        acc = dot2(bytes23_to_h2_1024(q), x.v[4 * k + 2 * w + 1], acc);
+      }
+      // scale byte index 2k + is lies in word k >> 1
+      const int sc = (int)(int8_t)((r.sc[k >> 1] >> (8u * ((2u * k & 3u) + is))) & 0xFFu);
+      total += d * (float)sc * (acc - 1056.f * x.sx[k]);  // halves carry 1024 + q6; weight = q6 - 32
+    }
+    return total;
+  }
+};
+
+// ---- Q5_K: {fp16 d, dmin; u8 sc[12]; u8 qh[32]; u8 ql[128]}, 176 bytes / 256 weights.
+// Unit j of a block: 64-column group g = j >> 1, l0 = 16 * (j & 1); it owns columns 64 g + l0 .. + 15 (low nibbles,
+// scale index 2 g) and 64 g + 32 + l0 .. + 15 (high nibbles, scale index 2 g + 1).
+struct DecQ5K {
+  static constexpr int UNIT = 32, LDS_WORDS = 0;
+  struct X { uint32_t v[16]; float sx[2]; };
+  struct Raw { uint32_t ql[4], qh[4], pa, pb, pc, dd; };
+  __device__ static void fill_lds(uint32_t*, int, int) {}
+  __device__ static X load_x(const float* x, uint32_t u) {
+    X r;
+    const uint32_t j = u & 7u;
+    const float* base = x + 256u * (u >> 3) + 64u * (j >> 1) + 16u * (j & 1u);
+    load_x32_consecutive(base, r.v, 16);
+    load_x32_consecutive(base + 32, r.v + 8, 16);
+    r.sx[0] = sum_h2(r.v, 8);
+    r.sx[1] = sum_h2(r.v + 8, 8);
+    return r;
+  }
+  __device__ static Raw load(const uint8_t* row, uint32_t u) {
+    const uint8_t* b = row + (u >> 3) * 176u;
+    const uint32_t j = u & 7u, g = j >> 1, l0 = 16u * (j & 1u), is = 2u * g;
+    const u128_a2 l = ld128(b + 48 + 32 * g + l0), h = ld128(b + 16 + l0);
+    // scale bytes is, is+1 (pa), is+4, is+5 (pb) and, for the upper groups, is-4, is-3 (pc)
+    return {{l.x, l.y, l.z, l.w}, {h.x, h.y, h.z, h.w}, ld16(b + 4 + is), ld16(b + 8 + is),
+            ld16(b + (is >= 4 ? is : 4u)), ld32(b)};
+  }
+  __device__ static float dot(const Raw& r, const X& x, const uint32_t*, uint32_t u) {
+    const uint32_t g = (u & 7u) >> 1;
+    const float d = half_bits_to_float(r.dd & 0xFFFFu), dmin = half_bits_to_float(r.dd >> 16);
+    float total = 0.f;
+#pragma unroll
+    for (int run = 0; run < 2; run++) {
+      float acc = 0.f;
+#pragma unroll
+      for (int w = 0; w < 4; w++) {
+        const uint32_t n = (r.ql[w] >> (4 * run)) & 0x0F0F0F0Fu;
+        const uint32_t hb = ((r.qh[w] >> (2 * g + run)) & 0x01010101u) << 4;
+        const uint32_t q = n | hb;  // 4 bytes in 0..31
+        acc = dot2(bytes01_to_h2_1024(q), x.v[8 * run + 2 * w], acc);
+        acc = dot2(bytes23_to_h2_1024(q), x.v[8 * run + 2 * w + 1], acc);
+      }
+      const uint32_t a = (r.pa >> (8 * run)) & 0xFFu, bq = (r.pb >> (8 * run)) & 0xFFu, c = (r.pc >> (8 * run)) & 0xFFu;
+      uint32_t sc, mn;
+      if (g < 2) { sc = a & 63u; mn = bq & 63u; }
+      else { sc = (bq & 0xFu) | ((c >> 6) << 4); mn = (bq >> 4) | ((a >> 6) << 4); }
+      total += (d * (float)sc) * (acc - 1024.f * x.sx[run]) - (dmin * (float)mn) * x.sx[run];
+    }
+    return total;
+  }
+};
+
+// ---- dense rows (F32 / F16 / BF16): unit = 8 consecutive elements, fp32 activations
+template <int QT>
+struct DecDense {
+  static constexpr int UNIT = 8, LDS_WORDS = 0;
+  struct X { float v[8]; };
+  struct Raw { uint32_t w[QT == MSQ_F32 ? 8 : 4]; };
+  __device__ static void fill_lds(uint32_t*, int, int) {}
+  __device__ static X load_x(const float* x, uint32_t u) {
+    X r;
+    const float4 a = ((const float4*)(x + 8u * u))[0], b = ((const float4*)(x + 8u * u))[1];
+    r.v[0] = a.x; r.v[1] = a.y; r.v[2] = a.z; r.v[3] = a.w; r.v[4] = b.x; r.v[5] = b.y; r.v[6] = b.z; r.v[7] = b.w;
+    return r;
+  }
+  __device__ static Raw load(const uint8_t* row, uint32_t u) {
+    Raw r;
+    if constexpr (QT == MSQ_F32) {
+      const u128_a2 a = ld128(row + 32u * u), b = ld128(row + 32u * u + 16);
+      r.w[0] = a.x; r.w[1] = a.y; r.w[2] = a.z; r.w[3] = a.w; r.w[4] = b.x; r.w[5] = b.y; r.w[6] = b.z; r.w[7] = b.w;
+    } else {
+      const u128_a2 a = ld128(row + 16u * u);
+      r.w[0] = a.x; r.w[1] = a.y; r.w[2] = a.z; r.w[3] = a.w;
+    }
+    return r;
+  }
+  __device__ static float dot(const Raw& r, const X& x, const uint32_t*) {
+    float acc = 0.f;
+    if constexpr (QT == MSQ_F32) {
+#pragma unroll
+      for (int i = 0; i < 8; i++) acc += __builtin_bit_cast(float, r.w[i]) * x.v[i];
+    } else if constexpr (QT == MSQ_F16) {
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+        acc += half_bits_to_float(r.w[i] & 0xFFFFu) * x.v[2 * i];
+        acc += half_bits_to_float(r.w[i] >> 16) * x.v[2 * i + 1];
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+        acc += __builtin_bit_cast(float, r.w[i] << 16) * x.v[2 * i];
+        acc += __builtin_bit_cast(float, r.w[i] & 0xFFFF0000u) * x.v[2 * i + 1];
+      }
+    }
+    return acc;
+  }
+};
+
+// Uniform call: decoders whose dot() needs the unit index (sub-position inside the block) take it as 4th argument.
+template <class D>
+__device__ __forceinline__ float dec_dot(const typename D::Raw& r, const typename D::X& x, const uint32_t* lds, uint32_t u) {
+  if constexpr (requires { D::dot(r, x, lds, u); }) return D::dot(r, x, lds, u);
+  else return D::dot(r, x, lds);
+}
+
+}  // namespace msq

@@ -1,0 +1,42 @@
+// Host-side helpers shared by the C-ABI translation units: error reporting, buffer checks, device facts.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdarg.h>
+#include <stdio.h>
+#include <string.h>
+
+#include "../../include/msq.h"
+#include "msq_types.h"
+
+namespace msq {
+
+extern thread_local char g_err[512];
+
+inline int fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof g_err, fmt, ap);
+  va_end(ap);
+  return code;
+}
+// reference message shape: "macseek quant: <what> unsupported (type T rows R cols C)" (src/kernels/quant.mm:34-37)
+inline int unsupported(const char* what, int t, int rows, int cols) {
+  return fail(MSQ_ERR_UNSUPPORTED, "macseek quant: %s unsupported (type %s rows %d cols %d)", what, msq_type_name_of(t), rows, cols);
+}
+inline int hip_fail(hipError_t e, const char* where) {
+  return fail(MSQ_ERR_HIP, "macseek quant: HIP error in %s: %s", where, hipGetErrorString(e));
+}
+#define MSQ_HIP(expr)                                        \
+  do {                                                       \
+    hipError_t e_ = (expr);                                  \
+    if (e_ != hipSuccess) return ::msq::hip_fail(e_, #expr); \
+  } while (0)
+
+inline const uint8_t* bptr(const MsqBuffer* b) { return (const uint8_t*)b->dev + b->off; }
+inline uint8_t* bptr_mut(const MsqBuffer* b) { return (uint8_t*)b->dev + b->off; }
+inline bool buf_ok(const MsqBuffer* b, size_t need) { return b && b->dev && b->size >= need; }
+
+struct DeviceInfo { int ok, cus; };
+const DeviceInfo& device_info();  // cached facts of the current device (CU count, gfx950 check)
+
+}  // namespace msq

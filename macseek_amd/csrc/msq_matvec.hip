@@ -1,0 +1,175 @@
+// C ABI: library bring-up, geometry queries, decode matvec and dequantization (see include/msq.h).
+#include <algorithm>
+
+#include "msq_deq.cuh"
+#include "msq_host.h"
+#include "msq_mv.cuh"
+
+namespace msq {
+
+thread_local char g_err[512] = "";
+
+const DeviceInfo& device_info() {
+  static const DeviceInfo info = [] {
+    DeviceInfo d{0, 256};
+    int dev = 0;
+    hipDeviceProp_t p;
+    if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&p, dev) == hipSuccess) {
+      d.cus = p.multiProcessorCount > 0 ? p.multiProcessorCount : 256;
+      d.ok = strncmp(p.gcnArchName, "gfx950", 6) == 0;
+    }
+    return d;
+  }();
+  return info;
+}
+
+namespace {
+
+// Launch shape of the decode matvec. units = cols / UNIT columns-slices per row; a wave covers 64 * iters of them.
+struct MvShape { int iters, ks, rw, rpw, unit; };
+
+int mv_unit(int t) { return msq_type_block_elems(t) == 1 ? 8 : 32; }
+
+bool mv_shape(int t, int rows, int cols, int groups, const MsqMvCfg* cfg, MvShape* s) {
+  const int unit = mv_unit(t);
+  const int units = cols / unit;
+  int iters = 1;
+  while (iters < 4 && units > 64 * 16 * iters) iters *= 2;
+  int ks = (units + 64 * iters - 1) / (64 * iters);
+  if (cfg && cfg->ks > 0) {  // a wider K split than needed only adds idle waves; a narrower one needs more iters
+    ks = cfg->ks;
+    while (iters < 4 && units > 64 * ks * iters) iters *= 2;
+  }
+  if (ks > 16 || units > 64 * ks * iters) return false;
+  int rw = std::max(1, 8 / ks);
+  if (cfg && cfg->rsg > 0) rw = cfg->rsg;
+  if (rw * ks > 16) rw = std::max(1, 16 / ks);
+  const int rpg = rows / groups;
+  // rows per wave per tile: enough tiles to fill the chip a few times over, at most 8 rows per wave
+  int rpw = 8;
+  while (rpw > 1 && (long)rows / (rw * rpw) < 2048) rpw /= 2;
+  if (cfg && cfg->nr > 0) rpw = std::min(cfg->nr, 64);
+  if (groups > 1) {  // every tile must stay inside one block-diagonal group
+    while (rpw > 1 && rpg % (rw * rpw)) rpw /= 2;
+    while (rw > 1 && rpg % (rw * rpw)) rw /= 2;
+    if (rpg % (rw * rpw)) return false;
+  }
+  *s = {iters, ks, rw, rpw, unit};
+  return true;
+}
+
+template <class D>
+int launch_mv(hipStream_t st, const MvShape& s, MvArgs& a) {
+  const int threads = 64 * s.rw * s.ks;
+  const int tile_rows = s.rw * s.rpw;
+  a.units = a.cols / D::UNIT;
+  a.ks = s.ks;
+  a.rpw = s.rpw;
+  a.ntiles = (a.rows + tile_rows - 1) / tile_rows;
+  const size_t lds = (size_t)D::LDS_WORDS * 4 + (size_t)tile_rows * s.ks * 4;
+  // persistent workgroups: as many as can be resident, never more than there are tiles
+  const int wg_per_cu = std::max(1, std::min(2048 / threads, (int)((160 * 1024) / std::max<size_t>(lds, 1))));
+  const int grid = (int)std::min<long>(a.ntiles, (long)device_info().cus * wg_per_cu);
+  switch (s.iters) {
+    case 1: hipLaunchKernelGGL((mv_kernel<D, 1>), dim3(grid), dim3(threads), lds, st, a); break;
+    case 2: hipLaunchKernelGGL((mv_kernel<D, 2>), dim3(grid), dim3(threads), lds, st, a); break;
+    default: hipLaunchKernelGGL((mv_kernel<D, 4>), dim3(grid), dim3(threads), lds, st, a); break;
+  }
+  MSQ_HIP(hipGetLastError());
+  return MSQ_OK;
+}
+
+bool mv_type_ok(int t) {
+  switch (t) {
+    case MSQ_F32: case MSQ_F16: case MSQ_BF16: case MSQ_Q8_0: case MSQ_Q5_K: case MSQ_Q6_K: case MSQ_IQ1_S:
+    case MSQ_IQ2_XXS: case MSQ_IQ4_NL: return true;
+    default: return false;
+  }
+}
+// column granularity the kernels need: dense types use a virtual 256 block like the reference (quant.mm:31-32)
+int mv_col_multiple(int t) { return msq_type_block_elems(t) == 1 ? 256 : msq_type_block_elems(t); }
+
+}  // namespace
+}  // namespace msq
+
+using namespace msq;
+
+extern "C" {
+
+int msq_init(void) {
+  g_err[0] = 0;
+  const DeviceInfo& d = device_info();
+  if (!d.ok) return fail(MSQ_ERR_HIP, "macseek quant: no gfx950 device is current");
+  return MSQ_OK;
+}
+const char* msq_last_error(void) { return g_err; }
+int msq_device_ok(void) { return device_info().ok; }
+
+int msq_block_elems(int t) { return msq_type_block_elems(t); }
+size_t msq_block_bytes(int t) { return msq_type_block_bytes(t); }
+size_t msq_row_bytes(int t, int64_t cols) { return msq_type_row_bytes(t, cols); }
+const char* msq_type_name(int t) { return msq_type_name_of(t); }
+
+int msq_matvec_supported(int t) { return mv_type_ok(t) ? 1 : 0; }
+
+int msq_matvec_cfg(int t, int rows, int cols, MsqMvCfg* out) {
+  MvShape s;
+  if (!out) return fail(MSQ_ERR_ARGUMENT, "macseek quant: matvec_cfg: null output");
+  if (!mv_type_ok(t) || rows < 1 || cols < 1 || cols % mv_col_multiple(t) || !mv_shape(t, rows, cols, 1, nullptr, &s))
+    return unsupported("matvec_cfg", t, rows, cols);
+  out->nr = s.rpw; out->rsg = s.rw; out->ks = s.ks;
+  return MSQ_OK;
+}
+
+int msq_matvec(void* stream, int t, const MsqBuffer* W, int rows, int cols, const MsqBuffer* x, const MsqBuffer* y,
+               int accumulate, int groups, const MsqMvCfg* cfg) {
+  if (!mv_type_ok(t) || rows < 1 || cols < 1 || cols % mv_col_multiple(t) || groups < 1 || rows % groups)
+    return unsupported("matvec", t, rows, cols);
+  const size_t rb = msq_type_row_bytes(t, cols);
+  if (!buf_ok(W, rb * (size_t)rows) || !buf_ok(x, (size_t)cols * groups * 4) || !buf_ok(y, (size_t)rows * 4))
+    return fail(MSQ_ERR_ARGUMENT, "macseek quant: matvec: buffer missing or too small (type %s rows %d cols %d)",
+                msq_type_name_of(t), rows, cols);
+  MvShape s;
+  if (!mv_shape(t, rows, cols, groups, cfg, &s)) return unsupported("matvec launch shape", t, rows, cols);
+  MvArgs a{};
+  a.W = bptr(W); a.x = (const float*)bptr(x); a.y = (float*)bptr_mut(y);
+  a.rows = (uint32_t)rows; a.cols = (uint32_t)cols; a.row_bytes = (uint32_t)rb;
+  a.rows_per_group = (uint32_t)(rows / groups); a.x_group_stride = (uint32_t)cols; a.accumulate = accumulate ? 1u : 0u;
+  hipStream_t st = (hipStream_t)stream;
+  switch (t) {
+    case MSQ_IQ1_S: return launch_mv<DecIQ1S>(st, s, a);
+    case MSQ_IQ2_XXS: return launch_mv<DecIQ2XXS>(st, s, a);
+    case MSQ_Q8_0: return launch_mv<DecQ8_0>(st, s, a);
+    case MSQ_IQ4_NL: return launch_mv<DecIQ4NL>(st, s, a);
+    case MSQ_Q6_K: return launch_mv<DecQ6K>(st, s, a);
+    case MSQ_Q5_K: return launch_mv<DecQ5K>(st, s, a);
+    case MSQ_F32: return launch_mv<DecDense<MSQ_F32>>(st, s, a);
+    case MSQ_F16: return launch_mv<DecDense<MSQ_F16>>(st, s, a);
+    case MSQ_BF16: return launch_mv<DecDense<MSQ_BF16>>(st, s, a);
+  }
+  return unsupported("matvec", t, rows, cols);
+}
+
+int msq_dequant(void* stream, int t, const MsqBuffer* W, int64_t n, const MsqBuffer* out) {
+  const int be = msq_type_block_elems(t);
+  if (!be || n < 0 || n % be || n % 8) return unsupported("dequant", t, 0, (int)n);
+  if (n == 0) return MSQ_OK;
+  if (!buf_ok(W, msq_type_row_bytes(t, n)) || !buf_ok(out, (size_t)n * 4))
+    return fail(MSQ_ERR_ARGUMENT, "macseek quant: dequant: buffer missing or too small");
+  const uint8_t* src = bptr(W);
+  float* dst = (float*)bptr_mut(out);
+  const int64_t nchunks = n / 8;
+  const dim3 grid((unsigned)((nchunks + 255) / 256)), block(256);
+  hipStream_t st = (hipStream_t)stream;
+  switch (t) {
+#define MSQ_DEQ(T) case T: hipLaunchKernelGGL((dequant_kernel<T>), grid, block, 0, st, src, dst, nchunks); break;
+    MSQ_DEQ(MSQ_F32) MSQ_DEQ(MSQ_F16) MSQ_DEQ(MSQ_BF16) MSQ_DEQ(MSQ_Q8_0) MSQ_DEQ(MSQ_IQ4_NL) MSQ_DEQ(MSQ_IQ1_S)
+    MSQ_DEQ(MSQ_IQ2_XXS) MSQ_DEQ(MSQ_Q6_K) MSQ_DEQ(MSQ_Q5_K)
+#undef MSQ_DEQ
+    default: return unsupported("dequant", t, 0, (int)n);
+  }
+  MSQ_HIP(hipGetLastError());
+  return MSQ_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,123 @@
+"""Host-side mirror of the reference operator API (namespace ms::q, src/kernels/quant.hpp) over the C ABI.
+
+Names, argument order and meaning follow the reference: `encode_*` functions only enqueue work on the encoder's
+stream. Where the reference prints "macseek quant: ... unsupported" and aborts (src/kernels/quant.mm:34-37) these
+functions raise QuantError with the same message. There is no CPU fallback: without libmsq.so every call raises.
+"""
+import ctypes as C
+import enum
+
+from . import _lib
+from ._lib import MsqBuffer, MsqMvCfg
+
+
+class QType(enum.IntEnum):  # reference: src/kernels/quant_types.hpp:9-11 (ggml type ids)
+    F32 = 0
+    F16 = 1
+    Q8_0 = 8
+    Q5_K = 13
+    Q6_K = 14
+    IQ2_XXS = 16
+    IQ1_S = 19
+    IQ4_NL = 20
+    BF16 = 30
+
+
+class QuantError(RuntimeError):
+    def __init__(self, code, msg):
+        super().__init__(msg)
+        self.code = code
+
+
+def _check(rc):
+    if rc != 0:
+        raise QuantError(rc, _lib.load().msq_last_error().decode())
+
+
+def block_elems(t):
+    return _lib.load().msq_block_elems(int(t))
+
+
+def block_bytes(t):
+    return _lib.load().msq_block_bytes(int(t))
+
+
+def row_bytes(t, cols):
+    return _lib.load().msq_row_bytes(int(t), int(cols))
+
+
+def type_name(t):
+    return _lib.load().msq_type_name(int(t)).decode()
+
+
+class Buffer:
+    """reference: ms::Buffer (src/core/metal.hpp:11-18). A device allocation (kept alive through `owner`), a byte
+    offset and the usable size from that offset."""
+
+    __slots__ = ("dev", "off", "size", "owner")
+
+    def __init__(self, dev=0, off=0, size=0, owner=None):
+        self.dev, self.off, self.size, self.owner = int(dev), int(off), int(size), owner
+
+    @staticmethod
+    def of(tensor):
+        """View of a whole torch tensor (must live on the GPU and be contiguous)."""
+        assert tensor.is_contiguous()
+        return Buffer(tensor.data_ptr(), 0, tensor.numel() * tensor.element_size(), tensor)
+
+    def sub(self, o, s):
+        assert o + s <= self.size
+        return Buffer(self.dev, self.off + o, s, self.owner)
+
+    def c(self):
+        return MsqBuffer(self.dev, self.off, self.size)
+
+
+class MvCfg:  # reference: ms::q::MvCfg (quant.hpp:12)
+    def __init__(self, nr=0, rsg=0, ks=0):
+        self.nr, self.rsg, self.ks = nr, rsg, ks
+
+
+class Enc:
+    """reference: ms::Enc (src/core/metal.hpp:37-71) reduced to what the quant operators need: a stream to enqueue
+    on. barrier() is a no-op because a HIP stream is in-order; wait() blocks until the stream has drained."""
+
+    def __init__(self, stream=None):
+        import torch
+        self._torch = torch
+        self.stream = stream if stream is not None else torch.cuda.current_stream()
+
+    @property
+    def handle(self):
+        return C.c_void_p(self.stream.cuda_stream)
+
+    def barrier(self):
+        pass
+
+    def wait(self):
+        self.stream.synchronize()
+
+
+def _bp(b):
+    return C.byref(b.c()) if b is not None else None
+
+
+def matvec_supported(t):  # reference: quant.hpp:14
+    return bool(_lib.load().msq_matvec_supported(int(t)))
+
+
+def matvec_cfg(t, rows, cols):  # reference: quant.hpp:16-18
+    out = MsqMvCfg()
+    _check(_lib.load().msq_matvec_cfg(int(t), rows, cols, C.byref(out)))
+    return MvCfg(out.nr, out.rsg, out.ks)
+
+
+def encode_matvec(e, t, W, rows, cols, x, y, accumulate=False, groups=1, cfg=None):  # reference: quant.hpp:29-30
+    c = MsqMvCfg(cfg.nr, cfg.rsg, cfg.ks) if cfg is not None else None
+    _check(_lib.load().msq_matvec(e.handle, int(t), _bp(W), rows, cols, _bp(x), _bp(y), int(bool(accumulate)), groups,
+                                  C.byref(c) if c is not None else None))
+
+
+def encode_dequant(e, t, W, n_elems, out):
+    """Whole-buffer dequantization to fp32 (bit-exact with ref::dequant_row, tests/ref/dequant.cpp:34-120)."""
+    _check(_lib.load().msq_dequant(e.handle, int(t), _bp(W), n_elems, _bp(out)))
