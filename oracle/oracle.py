@@ -45,7 +45,7 @@ def load():
     L.orc_dequant_row.argtypes = [i32, vp, vp, i64]; L.orc_dequant_row.restype = i32
     L.orc_matvec.argtypes = [i32, vp, i32, i32, vp, i32, vp, vp, vp, i32]; L.orc_matvec.restype = i32
     L.orc_swiglu.argtypes = [C.c_double] * 3; L.orc_swiglu.restype = C.c_double
-    L.orc_moe_decode.argtypes = [i32] * 7 + [vp] * 10 + [i32]; L.orc_moe_decode.restype = i32
+    L.orc_moe_decode.argtypes = [i32] * 7 + [vp] * 9 + [i32]; L.orc_moe_decode.restype = i32
     L.orc_moe_prefill.argtypes = [i32] * 8 + [vp] * 8 + [i32, i32, vp, vp, i32]; L.orc_moe_prefill.restype = i32
     L.orc_randn.argtypes = [vp, i64, u64, f32]
     L.orc_random_blocks.argtypes = [i32, i64, u64, f32, vp]; L.orc_random_blocks.restype = i32
