@@ -81,6 +81,63 @@ int msq_matvec(void* stream, int qtype, const MsqBuffer* W, int rows, int cols, 
  * n_elems must be a multiple of the block size; out holds n_elems floats. */
 int msq_dequant(void* stream, int qtype, const MsqBuffer* W, int64_t n_elems, const MsqBuffer* out);
 
+/* ---------------------------------------------------------------------------------------------- MoE, one token */
+
+/* reference: kMaxRouted / kExpertDim / kExpertInter (quant.hpp:49). The reference hard-codes the expert shape; here
+ * dim / inter travel in the argument structs and 0 selects the reference constants. */
+#define MSQ_MAX_ROUTED 6
+#define MSQ_EXPERT_DIM 5120
+#define MSQ_EXPERT_INTER 2304
+
+/* reference: ms::q::ExpertSlot (quant.hpp:51-53): gate [dim -> inter], up [dim -> inter], down [inter -> dim] */
+typedef struct MsqExpertSlot { MsqBuffer gate, up, down; } MsqExpertSlot;
+
+/* reference: ms::q::MoeDecodeArgs (quant.hpp:55-71), field for field, plus dim / inter.
+ * Routed types: IQ1_S or IQ2_XXS (gate/up and down may differ). Shared type: Q6_K or Q8_0 as in the reference
+ * (quant.mm:255-261), and additionally IQ2_XXS or IQ1_S. */
+typedef struct MsqMoeDecodeArgs {
+  int t_gate_up;   /* routed gate/up type */
+  int t_down;      /* routed down type */
+  int n_routed;    /* 0..MSQ_MAX_ROUTED */
+  MsqExpertSlot slot[MSQ_MAX_ROUTED];
+  MsqBuffer weights; /* F32[n_routed] routing weights, device memory, may be written by an earlier kernel */
+  int has_shared;
+  int t_shared;    /* shared expert type, weight 1 */
+  MsqExpertSlot shared;
+  MsqBuffer x;     /* F32[dim] */
+  MsqBuffer y;     /* F32[dim], the result is ACCUMULATED into y */
+  MsqBuffer scratch; /* >= msq_moe_decode_scratch_bytes(inter): F32 h[(MSQ_MAX_ROUTED + 1)][inter] */
+  /* launch shape overrides, 0 = default: rows per wave (nr) and row-waves per workgroup (rsg) of the gate/up and
+   * down kernels. They never change a row's summation order (reference: quant.hpp:67-69). */
+  int gu_nr, gu_rsg, d_nr, d_rsg;
+  int dim, inter;  /* 0 = MSQ_EXPERT_DIM / MSQ_EXPERT_INTER; both multiples of 256, at most 32768 */
+} MsqMoeDecodeArgs;
+
+/* reference: ms::q::MoePart (quant.hpp:85): pieces of the table variant.
+ *   SHARED_GU then AFTER_SHARED_GU == ALL, bit-identical
+ *   SHARED then ROUTED             == ALL up to float summation order
+ *   SHARED_GU then SHARED_DOWN     == SHARED, bit-identical */
+enum { MSQ_PART_ALL = 0, MSQ_PART_SHARED_GU = 1, MSQ_PART_AFTER_SHARED_GU = 2, MSQ_PART_SHARED = 3,
+       MSQ_PART_ROUTED = 4, MSQ_PART_SHARED_DOWN = 5 };
+
+/* reference: ms::q::moe_decode_scratch_bytes (quant.hpp:72, quant.mm:264); inter = 0 means MSQ_EXPERT_INTER */
+size_t msq_moe_decode_scratch_bytes(int inter);
+
+/* reference: ms::q::encode_moe_decode (quant.hpp:73-75, quant.mm:266-315). Two kernels on the stream: gate + up +
+ * SwiGLU (u = clamp(up, -10, 10), g = min(gate, 10), h = silu(g) * u * weight) for all experts, then down for all
+ * experts accumulated into y. n_routed == 0 without a shared expert returns MSQ_OK and does nothing. */
+int msq_moe_decode(void* stream, const MsqMoeDecodeArgs* a);
+
+/* reference: ms::q::encode_moe_decode_table (quant.hpp:76-78, quant.mm:317-319). Routed matrices come from `table`:
+ * MSQ_MAX_ROUTED entries of three device addresses {gate, up, down} (uint64), read by the GPU when the kernels run,
+ * so the host may fill it after this call returned as long as it is complete before the GPU reaches the kernels.
+ * a->slot[] is ignored. The table must be readable from the device (device or pinned host memory). */
+int msq_moe_decode_table(void* stream, const MsqMoeDecodeArgs* a, const MsqBuffer* table);
+
+/* reference: ms::q::encode_moe_decode_table_part (quant.hpp:79-86, quant.mm:321-369). SHARED_GU / SHARED /
+ * SHARED_DOWN never read `table` (it may be NULL for them). */
+int msq_moe_decode_table_part(void* stream, const MsqMoeDecodeArgs* a, const MsqBuffer* table, int part);
+
 #ifdef __cplusplus
 }
 #endif

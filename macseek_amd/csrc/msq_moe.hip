@@ -1,0 +1,181 @@
+// C ABI: fused one-token MoE layer (see include/msq.h; reference host code src/kernels/quant.mm:252-369).
+#include <algorithm>
+
+#include "msq_host.h"
+#include "msq_moe.cuh"
+
+namespace msq {
+namespace {
+
+bool routed_type_ok(int t) { return t == MSQ_IQ1_S || t == MSQ_IQ2_XXS; }
+bool shared_type_ok(int t) { return t == MSQ_Q6_K || t == MSQ_Q8_0 || t == MSQ_IQ2_XXS || t == MSQ_IQ1_S; }
+
+template <class DR, class DS>
+void launch_gu_t(dim3 g, dim3 b, size_t lds, hipStream_t st, const MoeArgs& a) {
+  hipLaunchKernelGGL((moe_gu_kernel<DR, DS>), g, b, lds, st, a);
+}
+template <class DR, class DS>
+void launch_down_t(dim3 g, dim3 b, size_t lds, hipStream_t st, const MoeArgs& a) {
+  hipLaunchKernelGGL((moe_down_kernel<DR, DS>), g, b, lds, st, a);
+}
+template <class DR>
+size_t lds_words_for_shared(int ts, bool down) {
+  size_t s = 0;
+  switch (ts) {
+    case MSQ_IQ2_XXS: s = DecIQ2XXS::LDS_WORDS; break;
+    case MSQ_IQ1_S: s = DecIQ1S::LDS_WORDS; break;
+    default: s = 0;
+  }
+  return down ? DR::LDS_WORDS + s : std::max<size_t>(DR::LDS_WORDS, s);
+}
+// dispatch over (routed type, shared type)
+template <bool DOWN>
+size_t dispatch(int tr, int ts, dim3 g, dim3 b, size_t part_bytes, hipStream_t st, const MoeArgs& a) {
+#define MSQ_MOE_CASE(TR, DRT, TS, DST)                                                            \
+  if (tr == TR && ts == TS) {                                                                     \
+    const size_t lds = 4 * lds_words_for_shared<DRT>(ts, DOWN) + part_bytes;                      \
+    if (DOWN) launch_down_t<DRT, DST>(g, b, lds, st, a); else launch_gu_t<DRT, DST>(g, b, lds, st, a); \
+    return lds;                                                                                   \
+  }
+  MSQ_MOE_CASE(MSQ_IQ1_S, DecIQ1S, MSQ_Q6_K, DecQ6K)
+  MSQ_MOE_CASE(MSQ_IQ1_S, DecIQ1S, MSQ_Q8_0, DecQ8_0)
+  MSQ_MOE_CASE(MSQ_IQ1_S, DecIQ1S, MSQ_IQ2_XXS, DecIQ2XXS)
+  MSQ_MOE_CASE(MSQ_IQ1_S, DecIQ1S, MSQ_IQ1_S, DecIQ1S)
+  MSQ_MOE_CASE(MSQ_IQ2_XXS, DecIQ2XXS, MSQ_Q6_K, DecQ6K)
+  MSQ_MOE_CASE(MSQ_IQ2_XXS, DecIQ2XXS, MSQ_Q8_0, DecQ8_0)
+  MSQ_MOE_CASE(MSQ_IQ2_XXS, DecIQ2XXS, MSQ_IQ2_XXS, DecIQ2XXS)
+  MSQ_MOE_CASE(MSQ_IQ2_XXS, DecIQ2XXS, MSQ_IQ1_S, DecIQ1S)
+#undef MSQ_MOE_CASE
+  return 0;
+}
+
+int moe_decode_impl(hipStream_t st, const MsqMoeDecodeArgs* p, const MsqBuffer* table, int part, bool need_table) {
+  if (!p) return fail(MSQ_ERR_ARGUMENT, "macseek quant: moe_decode: null arguments");
+  const int dim = p->dim ? p->dim : MSQ_EXPERT_DIM, inter = p->inter ? p->inter : MSQ_EXPERT_INTER;
+  if (p->n_routed < 0 || p->n_routed > kMaxRouted) return unsupported("moe_decode n_routed", p->t_gate_up, p->n_routed, 0);
+  const bool shared_part = part == MSQ_PART_SHARED_GU || part == MSQ_PART_SHARED || part == MSQ_PART_SHARED_DOWN;
+  if (part < MSQ_PART_ALL || part > MSQ_PART_SHARED_DOWN) return unsupported("moe_decode part", p->t_gate_up, part, 0);
+  if (shared_part && !p->has_shared) return MSQ_OK;
+  if (p->n_routed + (p->has_shared ? 1 : 0) == 0) return MSQ_OK;
+  if (!routed_type_ok(p->t_gate_up) || !routed_type_ok(p->t_down) || (p->has_shared && !shared_type_ok(p->t_shared)))
+    return unsupported("moe_decode type combo", p->t_gate_up, 0, 0);
+  if (dim < 256 || inter < 256 || dim % 256 || inter % 256 || dim > 32768 || inter > 32768)
+    return unsupported("moe_decode expert shape", p->t_gate_up, inter, dim);
+  if (!buf_ok(&p->scratch, msq_moe_decode_scratch_bytes(inter)))
+    return fail(MSQ_ERR_SCRATCH, "macseek quant: moe_decode scratch too small unsupported (type %s rows 0 cols 0)",
+                msq_type_name_of(p->t_gate_up));
+  // which pieces this call runs (reference: quant.mm:329-334)
+  const bool gu_r = part == MSQ_PART_ALL || part == MSQ_PART_AFTER_SHARED_GU || part == MSQ_PART_ROUTED;
+  const bool gu_s = p->has_shared && (part == MSQ_PART_ALL || part == MSQ_PART_SHARED_GU || part == MSQ_PART_SHARED);
+  const bool d_r = gu_r;
+  const bool d_s = p->has_shared && (part == MSQ_PART_ALL || part == MSQ_PART_AFTER_SHARED_GU ||
+                                     part == MSQ_PART_SHARED || part == MSQ_PART_SHARED_DOWN);
+  const int nr = p->n_routed;
+  const bool routed_live = nr > 0;
+  if (!buf_ok(&p->x, (size_t)dim * 4) || !buf_ok(&p->y, (size_t)dim * 4))
+    return fail(MSQ_ERR_ARGUMENT, "macseek quant: moe_decode: x / y missing or too small");
+  if (routed_live && gu_r && !buf_ok(&p->weights, (size_t)nr * 4))
+    return fail(MSQ_ERR_ARGUMENT, "macseek quant: moe_decode: routing weights missing or too small");
+  const int ts = p->has_shared ? p->t_shared : MSQ_Q8_0;  // placeholder decoder when there is no shared expert
+  MoeArgs a{};
+  a.x = (const float*)bptr(&p->x); a.h = (float*)bptr_mut(&p->scratch); a.y = (float*)bptr_mut(&p->y);
+  a.wts = p->weights.dev ? (const float*)bptr(&p->weights) : nullptr;
+  a.n_routed = (uint32_t)nr; a.dim = (uint32_t)dim; a.inter = (uint32_t)inter;
+  a.rb_gu_r = (uint32_t)msq_type_row_bytes(p->t_gate_up, dim); a.rb_d_r = (uint32_t)msq_type_row_bytes(p->t_down, inter);
+  a.rb_gu_s = (uint32_t)msq_type_row_bytes(ts, dim); a.rb_d_s = (uint32_t)msq_type_row_bytes(ts, inter);
+  if (routed_live && gu_r) {
+    if (need_table) {
+      if (!buf_ok(table, (size_t)kMaxRouted * 24)) return fail(MSQ_ERR_ARGUMENT, "macseek quant: moe_decode: table missing or too small");
+      a.table = (const uint64_t*)bptr(table);
+    } else {
+      for (int i = 0; i < nr; i++) {
+        const MsqExpertSlot& s = p->slot[i];
+        if (!buf_ok(&s.gate, (size_t)a.rb_gu_r * inter) || !buf_ok(&s.up, (size_t)a.rb_gu_r * inter) ||
+            !buf_ok(&s.down, (size_t)a.rb_d_r * dim))
+          return fail(MSQ_ERR_ARGUMENT, "macseek quant: moe_decode: routed slot %d missing or too small", i);
+        a.gate[i] = bptr(&s.gate); a.up[i] = bptr(&s.up); a.down[i] = bptr(&s.down);
+      }
+    }
+  }
+  if (p->has_shared) {
+    const MsqExpertSlot& s = p->shared;
+    if (!buf_ok(&s.gate, (size_t)a.rb_gu_s * inter) || !buf_ok(&s.up, (size_t)a.rb_gu_s * inter) ||
+        !buf_ok(&s.down, (size_t)a.rb_d_s * dim))
+      return fail(MSQ_ERR_ARGUMENT, "macseek quant: moe_decode: shared expert missing or too small");
+    a.sgate = bptr(&s.gate); a.sup = bptr(&s.up); a.sdown = bptr(&s.down);
+  }
+  const int cus = device_info().cus;
+
+  // 1) gate + up + SwiGLU -> h
+  const int n_gu_r = (gu_r && routed_live) ? nr : 0;
+  if (n_gu_r > 0 || gu_s) {
+    const int units = dim / 32;
+    const int ks = (units + 63) / 64;
+    int rw = p->gu_rsg > 0 ? p->gu_rsg : std::max(1, 8 / ks);
+    if (rw * ks > 16) rw = std::max(1, 16 / ks);
+    const int rpw = p->gu_nr > 0 ? std::min(p->gu_nr, 64) : 8;
+    const int tile_rows = rw * rpw, threads = 64 * rw * ks;
+    a.ks = (uint32_t)ks; a.rpw = (uint32_t)rpw;
+    a.tiles_per_expert = (uint32_t)((inter + tile_rows - 1) / tile_rows);
+    a.run_routed = n_gu_r > 0; a.run_shared = gu_s;
+    const size_t part_bytes = (size_t)tile_rows * 2 * ks * 4;
+    // persistent workgroups, shared between the routed experts and the shared expert in proportion to their bytes
+    const long tiles_r = (long)n_gu_r * a.tiles_per_expert, tiles_s = gu_s ? a.tiles_per_expert : 0;
+    const int wg_per_cu = std::max(1, std::min(2048 / threads, 4));
+    const long total = std::min<long>(tiles_r + tiles_s, (long)cus * wg_per_cu);
+    const double br = (double)n_gu_r * a.rb_gu_r, bs = gu_s ? (double)a.rb_gu_s : 0.0;
+    long g_s = gu_s ? std::max<long>(1, (long)(total * bs / (br + bs) + 0.5)) : 0;
+    g_s = std::min(g_s, tiles_s);
+    long g_r = n_gu_r ? std::max<long>(1, std::min(tiles_r, total - g_s)) : 0;
+    a.grid_routed = (uint32_t)g_r;
+    if (!dispatch<false>(p->t_gate_up, ts, dim3((unsigned)(g_r + g_s)), dim3(threads), part_bytes, st, a))
+      return unsupported("moe_decode type combo", p->t_gate_up, 0, 0);
+    MSQ_HIP(hipGetLastError());
+  }
+  // 2) down for all experts, accumulated into y
+  const bool run_d_r = d_r && routed_live;
+  if (run_d_r || d_s) {
+    const int units = inter / 32;
+    const int ks = (units + 63) / 64;
+    const int ne = run_d_r ? nr : 1;
+    const int wpg = ne * ks;
+    if (wpg > 16) return unsupported("moe_decode inter too large for the down kernel", p->t_down, dim, inter);
+    int rw = p->d_rsg > 0 ? p->d_rsg : std::max(1, 8 / wpg);
+    if (rw * wpg > 16) rw = std::max(1, 16 / wpg);
+    const int rpw = p->d_nr > 0 ? std::min(p->d_nr, 64) : 16;
+    const int tile_rows = rw * rpw, threads = 64 * rw * wpg;
+    a.ks = (uint32_t)ks; a.rpw = (uint32_t)rpw;
+    a.run_routed = run_d_r; a.run_shared = d_s;
+    a.ntiles = (uint32_t)((dim + tile_rows - 1) / tile_rows);
+    const size_t slots = (size_t)(run_d_r ? nr * ks : 0) + (d_s ? ks : 0);
+    const size_t part_bytes = (size_t)tile_rows * slots * 4;
+    const int wg_per_cu = std::max(1, std::min(2048 / threads, 4));
+    const long grid = std::min<long>(a.ntiles, (long)cus * wg_per_cu);
+    if (!dispatch<true>(p->t_down, ts, dim3((unsigned)grid), dim3(threads), part_bytes, st, a))
+      return unsupported("moe_decode type combo", p->t_down, 0, 0);
+    MSQ_HIP(hipGetLastError());
+  }
+  return MSQ_OK;
+}
+
+}  // namespace
+}  // namespace msq
+
+using namespace msq;
+
+extern "C" {
+
+size_t msq_moe_decode_scratch_bytes(int inter) {
+  return sizeof(float) * (size_t)(kMaxRouted + 1) * (size_t)(inter > 0 ? inter : MSQ_EXPERT_INTER);
+}
+int msq_moe_decode(void* stream, const MsqMoeDecodeArgs* a) {
+  return moe_decode_impl((hipStream_t)stream, a, nullptr, MSQ_PART_ALL, false);
+}
+int msq_moe_decode_table(void* stream, const MsqMoeDecodeArgs* a, const MsqBuffer* table) {
+  return moe_decode_impl((hipStream_t)stream, a, table, MSQ_PART_ALL, true);
+}
+int msq_moe_decode_table_part(void* stream, const MsqMoeDecodeArgs* a, const MsqBuffer* table, int part) {
+  return moe_decode_impl((hipStream_t)stream, a, table, part, true);
+}
+
+}  // extern "C"

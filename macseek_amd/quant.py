@@ -8,7 +8,7 @@ import ctypes as C
 import enum
 
 from . import _lib
-from ._lib import MsqBuffer, MsqMvCfg
+from ._lib import MsqBuffer, MsqExpertSlot, MsqMoeDecodeArgs, MsqMvCfg
 
 
 class QType(enum.IntEnum):  # reference: src/kernels/quant_types.hpp:9-11 (ggml type ids)
@@ -121,3 +121,71 @@ def encode_matvec(e, t, W, rows, cols, x, y, accumulate=False, groups=1, cfg=Non
 def encode_dequant(e, t, W, n_elems, out):
     """Whole-buffer dequantization to fp32 (bit-exact with ref::dequant_row, tests/ref/dequant.cpp:34-120)."""
     _check(_lib.load().msq_dequant(e.handle, int(t), _bp(W), n_elems, _bp(out)))
+
+
+# ---------------------------------------------------------------------------------------------- MoE, one token
+kExpertDim, kExpertInter, kMaxRouted = 5120, 2304, 6  # reference: quant.hpp:49 (defaults of dim / inter here)
+
+
+class ExpertSlot:  # reference: ms::q::ExpertSlot (quant.hpp:51-53)
+    def __init__(self, gate=None, up=None, down=None):
+        self.gate, self.up, self.down = gate or Buffer(), up or Buffer(), down or Buffer()
+
+    def c(self):
+        return MsqExpertSlot(self.gate.c(), self.up.c(), self.down.c())
+
+
+class MoePart(enum.IntEnum):  # reference: ms::q::MoePart (quant.hpp:85)
+    All = 0
+    SharedGu = 1
+    AfterSharedGu = 2
+    Shared = 3
+    Routed = 4
+    SharedDown = 5
+
+
+class MoeDecodeArgs:
+    """reference: ms::q::MoeDecodeArgs (quant.hpp:55-71) plus dim / inter (defaults = the reference constants)."""
+
+    def __init__(self):
+        self.t_gate_up = QType.IQ1_S
+        self.t_down = QType.IQ1_S
+        self.n_routed = 6
+        self.slot = [ExpertSlot() for _ in range(kMaxRouted)]
+        self.weights = Buffer()
+        self.has_shared = True
+        self.t_shared = QType.Q6_K
+        self.shared = ExpertSlot()
+        self.x = Buffer()
+        self.y = Buffer()
+        self.scratch = Buffer()
+        self.gu_nr = self.gu_rsg = self.d_nr = self.d_rsg = 0
+        self.dim, self.inter = kExpertDim, kExpertInter
+
+    def c(self):
+        a = MsqMoeDecodeArgs()
+        a.t_gate_up, a.t_down, a.n_routed = int(self.t_gate_up), int(self.t_down), int(self.n_routed)
+        for i in range(kMaxRouted):
+            a.slot[i] = self.slot[i].c()
+        a.weights = self.weights.c()
+        a.has_shared, a.t_shared, a.shared = int(bool(self.has_shared)), int(self.t_shared), self.shared.c()
+        a.x, a.y, a.scratch = self.x.c(), self.y.c(), self.scratch.c()
+        a.gu_nr, a.gu_rsg, a.d_nr, a.d_rsg = self.gu_nr, self.gu_rsg, self.d_nr, self.d_rsg
+        a.dim, a.inter = self.dim, self.inter
+        return a
+
+
+def moe_decode_scratch_bytes(inter=kExpertInter):  # reference: quant.hpp:72
+    return _lib.load().msq_moe_decode_scratch_bytes(inter)
+
+
+def encode_moe_decode(e, a):  # reference: quant.hpp:73-75
+    _check(_lib.load().msq_moe_decode(e.handle, C.byref(a.c())))
+
+
+def encode_moe_decode_table(e, a, table):  # reference: quant.hpp:76-78
+    _check(_lib.load().msq_moe_decode_table(e.handle, C.byref(a.c()), _bp(table)))
+
+
+def encode_moe_decode_table_part(e, a, table, part):  # reference: quant.hpp:79-86
+    _check(_lib.load().msq_moe_decode_table_part(e.handle, C.byref(a.c()), _bp(table), int(part)))
