@@ -118,7 +118,10 @@ typedef struct MsqMoeDecodeArgs {
  *   SHARED then ROUTED             == ALL up to float summation order
  *   SHARED_GU then SHARED_DOWN     == SHARED, bit-identical */
 enum { MSQ_PART_ALL = 0, MSQ_PART_SHARED_GU = 1, MSQ_PART_AFTER_SHARED_GU = 2, MSQ_PART_SHARED = 3,
-       MSQ_PART_ROUTED = 4, MSQ_PART_SHARED_DOWN = 5 };
+       MSQ_PART_ROUTED = 4, MSQ_PART_SHARED_DOWN = 5,
+       /* no reference counterpart: the two kernels of ALL on their own (GU then DOWN == ALL, bit-identical), so a
+        * caller can time them separately or put other work between them */
+       MSQ_PART_GU = 6, MSQ_PART_DOWN = 7 };
 
 /* reference: ms::q::moe_decode_scratch_bytes (quant.hpp:72, quant.mm:264); inter = 0 means MSQ_EXPERT_INTER */
 size_t msq_moe_decode_scratch_bytes(int inter);

@@ -54,7 +54,7 @@ int moe_decode_impl(hipStream_t st, const MsqMoeDecodeArgs* p, const MsqBuffer* 
   const int dim = p->dim ? p->dim : MSQ_EXPERT_DIM, inter = p->inter ? p->inter : MSQ_EXPERT_INTER;
   if (p->n_routed < 0 || p->n_routed > kMaxRouted) return unsupported("moe_decode n_routed", p->t_gate_up, p->n_routed, 0);
   const bool shared_part = part == MSQ_PART_SHARED_GU || part == MSQ_PART_SHARED || part == MSQ_PART_SHARED_DOWN;
-  if (part < MSQ_PART_ALL || part > MSQ_PART_SHARED_DOWN) return unsupported("moe_decode part", p->t_gate_up, part, 0);
+  if (part < MSQ_PART_ALL || part > MSQ_PART_DOWN) return unsupported("moe_decode part", p->t_gate_up, part, 0);
   if (shared_part && !p->has_shared) return MSQ_OK;
   if (p->n_routed + (p->has_shared ? 1 : 0) == 0) return MSQ_OK;
   if (!routed_type_ok(p->t_gate_up) || !routed_type_ok(p->t_down) || (p->has_shared && !shared_type_ok(p->t_shared)))
@@ -65,11 +65,12 @@ int moe_decode_impl(hipStream_t st, const MsqMoeDecodeArgs* p, const MsqBuffer* 
     return fail(MSQ_ERR_SCRATCH, "macseek quant: moe_decode scratch too small unsupported (type %s rows 0 cols 0)",
                 msq_type_name_of(p->t_gate_up));
   // which pieces this call runs (reference: quant.mm:329-334)
-  const bool gu_r = part == MSQ_PART_ALL || part == MSQ_PART_AFTER_SHARED_GU || part == MSQ_PART_ROUTED;
-  const bool gu_s = p->has_shared && (part == MSQ_PART_ALL || part == MSQ_PART_SHARED_GU || part == MSQ_PART_SHARED);
-  const bool d_r = gu_r;
-  const bool d_s = p->has_shared && (part == MSQ_PART_ALL || part == MSQ_PART_AFTER_SHARED_GU ||
-                                     part == MSQ_PART_SHARED || part == MSQ_PART_SHARED_DOWN);
+  const bool gu_r = part == MSQ_PART_ALL || part == MSQ_PART_AFTER_SHARED_GU || part == MSQ_PART_ROUTED || part == MSQ_PART_GU;
+  const bool gu_s = p->has_shared && (part == MSQ_PART_ALL || part == MSQ_PART_SHARED_GU || part == MSQ_PART_SHARED ||
+                                      part == MSQ_PART_GU);
+  const bool d_r = part == MSQ_PART_ALL || part == MSQ_PART_AFTER_SHARED_GU || part == MSQ_PART_ROUTED || part == MSQ_PART_DOWN;
+  const bool d_s = p->has_shared && (part == MSQ_PART_ALL || part == MSQ_PART_AFTER_SHARED_GU || part == MSQ_PART_SHARED ||
+                                     part == MSQ_PART_SHARED_DOWN || part == MSQ_PART_DOWN);
   const int nr = p->n_routed;
   const bool routed_live = nr > 0;
   if (!buf_ok(&p->x, (size_t)dim * 4) || !buf_ok(&p->y, (size_t)dim * 4))
@@ -83,7 +84,7 @@ int moe_decode_impl(hipStream_t st, const MsqMoeDecodeArgs* p, const MsqBuffer* 
   a.n_routed = (uint32_t)nr; a.dim = (uint32_t)dim; a.inter = (uint32_t)inter;
   a.rb_gu_r = (uint32_t)msq_type_row_bytes(p->t_gate_up, dim); a.rb_d_r = (uint32_t)msq_type_row_bytes(p->t_down, inter);
   a.rb_gu_s = (uint32_t)msq_type_row_bytes(ts, dim); a.rb_d_s = (uint32_t)msq_type_row_bytes(ts, inter);
-  if (routed_live && gu_r) {
+  if (routed_live && (gu_r || d_r)) {
     if (need_table) {
       if (!buf_ok(table, (size_t)kMaxRouted * 24)) return fail(MSQ_ERR_ARGUMENT, "macseek quant: moe_decode: table missing or too small");
       a.table = (const uint64_t*)bptr(table);

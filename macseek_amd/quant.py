@@ -142,6 +142,8 @@ class MoePart(enum.IntEnum):  # reference: ms::q::MoePart (quant.hpp:85)
     Shared = 3
     Routed = 4
     SharedDown = 5
+    Gu = 6      # no reference counterpart: the gate/up kernel of All alone
+    Down = 7    # ... and its down kernel alone (Gu then Down == All, bit-identical)
 
 
 class MoeDecodeArgs:

@@ -152,6 +152,8 @@ def test_table_variant_and_parts(dev, dim, inter, sh):
     y4, h4 = run([q.MoePart.Shared])
     y5, h5 = run([q.MoePart.SharedGu, q.MoePart.SharedDown])
     assert torch.equal(y4, y5) and torch.equal(h4, h5)                  # bit-identical (quant.hpp:82)
+    y7, h7 = run([q.MoePart.Gu, q.MoePart.Down])
+    assert torch.equal(y_all, y7) and torch.equal(h_all, h7)
     # launch-shape overrides do not change any row's summation order (quant.hpp:67-69)
     y6 = up(L.y0.copy())
     a = L.args(y6)
