@@ -81,6 +81,12 @@ int msq_matvec(void* stream, int qtype, const MsqBuffer* W, int rows, int cols, 
  * n_elems must be a multiple of the block size; out holds n_elems floats. */
 int msq_dequant(void* stream, int qtype, const MsqBuffer* W, int64_t n_elems, const MsqBuffer* out);
 
+/* Achievable-bandwidth probe: streams `bytes` (multiple of 16, base 16-byte aligned) from `src` with 128-bit loads and
+ * writes one checksum word per workgroup to `sink` (>= 4096 bytes). The benchmark uses it as the measured-bandwidth
+ * denominator next to the 8 TB/s nominal peak (reference: q_bw_read_f4 / q_bw_read_chunk, src/kernels/quant_bench.metal:5-31,
+ * used by bench/qmatvec.mm:18-31). */
+int msq_bw_probe(void* stream, const MsqBuffer* src, size_t bytes, const MsqBuffer* sink);
+
 /* ---------------------------------------------------------------------------------------------- MoE, one token */
 
 /* reference: kMaxRouted / kExpertDim / kExpertInter (quant.hpp:49). The reference hard-codes the expert shape; here

@@ -132,6 +132,54 @@ __device__ __forceinline__ float wave_sum(float v) {
   return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
 }
 
+// Transposed partial reduction: N independent per-lane values (N = 1, 2, 4 or 8) are folded over the 8-lane group of
+// each lane in three DPP steps (lane i <-> 7 - i, then i <-> i ^ 1, then i <-> i ^ 2). A step that still has several
+// values to tell apart halves their number: a lane keeps the half its lane bit selects and receives its partner's
+// contribution to that half. Afterwards v[0] of lane l holds value number group8_sel<N>(l) summed over l's group.
+// This costs three ops per value pair instead of six full-wave steps per value; callers add the eight group sums of
+// a wave (and the K-split waves) in LDS in a fixed order.
+template <int CTRL>
+__device__ __forceinline__ float dpp_fold(float keep, float send) {
+  const int moved = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, send), CTRL, 0xF, 0xF, false);
+  return keep + __builtin_bit_cast(float, moved);
+}
+template <int N>
+__device__ __forceinline__ void group8_fold(float* v, uint32_t lane) {
+  static_assert(N == 1 || N == 2 || N == 4 || N == 8, "group8_fold: N must be 1, 2, 4 or 8");
+  const bool b0 = lane & 1u, b1 = lane & 2u, b2 = lane & 4u;
+  constexpr int N1 = N >= 2 ? N / 2 : 1, N2 = N >= 4 ? N / 4 : 1;
+  // step 1: partner 7 - i (row_half_mirror) differs in bit 2
+#pragma unroll
+  for (int i = 0; i < N1; i++) {
+    if constexpr (N >= 2) { const float lo = v[i], hi = v[i + N1]; v[i] = dpp_fold<0x141>(b2 ? hi : lo, b2 ? lo : hi); }
+    else v[i] = dpp_fold<0x141>(v[i], v[i]);
+  }
+  // step 2: partner i ^ 1 (quad_perm [1,0,3,2]) differs in bit 0
+#pragma unroll
+  for (int i = 0; i < N2; i++) {
+    if constexpr (N >= 4) { const float lo = v[i], hi = v[i + N2]; v[i] = dpp_fold<0xB1>(b0 ? hi : lo, b0 ? lo : hi); }
+    else v[i] = dpp_fold<0xB1>(v[i], v[i]);
+  }
+  // step 3: partner i ^ 2 (quad_perm [2,3,0,1]) differs in bit 1
+  if constexpr (N >= 8) { const float lo = v[0], hi = v[1]; v[0] = dpp_fold<0x4E>(b1 ? hi : lo, b1 ? lo : hi); }
+  else v[0] = dpp_fold<0x4E>(v[0], v[0]);
+}
+// group8_fold followed by one more step (lane i <-> i ^ 8, row_ror:8): v[0] holds the sum over the lane's 16-lane row.
+template <int N>
+__device__ __forceinline__ void row16_fold(float* v, uint32_t lane) {
+  group8_fold<N>(v, lane);
+  v[0] = dpp_fold<0x128>(v[0], v[0]);
+}
+// number of the value lane l holds after group8_fold<N>
+template <int N>
+__device__ __forceinline__ uint32_t group8_sel(uint32_t lane) {
+  uint32_t s = 0;
+  if (N >= 2) s += ((lane >> 2) & 1u) * (N / 2);
+  if (N >= 4) s += (lane & 1u) * (N / 4);
+  if (N >= 8) s += ((lane >> 1) & 1u) * (N / 8);
+  return s;
+}
+
 // ------------------------------------------------------------------------------------------------ LDS table copies
 __device__ __forceinline__ void copy_words16(uint32_t* dst, const uint32_t* src, int nwords, int tid, int nthreads) {
   const uint4* s = (const uint4*)src;

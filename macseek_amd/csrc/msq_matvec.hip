@@ -23,6 +23,18 @@ const DeviceInfo& device_info() {
   return info;
 }
 
+// Plain streaming read: every workgroup walks contiguous 16 KiB chunks grid-stride, one 128-bit load per lane per step.
+__global__ __launch_bounds__(1024) void bw_probe_kernel(const uint4* __restrict__ src, size_t n16, uint32_t* __restrict__ sink) {
+  uint4 acc = {0, 0, 0, 0};
+  const size_t chunk = 1024;  // uint4 per workgroup step
+  for (size_t base = (size_t)blockIdx.x * chunk; base < n16; base += (size_t)gridDim.x * chunk) {
+    const size_t i = base + threadIdx.x;
+    if (i < n16) { const uint4 v = src[i]; acc.x ^= v.x; acc.y ^= v.y; acc.z ^= v.z; acc.w ^= v.w; }
+  }
+  const uint32_t r = acc.x ^ acc.y ^ acc.z ^ acc.w;
+  if (r == 0x9E3779B9u) sink[blockIdx.x & 1023] = r;  // practically never true: keeps the loads alive without a store stream
+}
+
 namespace {
 
 // Launch shape of the decode matvec. units = cols / UNIT columns-slices per row; a wave covers 64 * iters of them.
@@ -148,6 +160,18 @@ int msq_matvec(void* stream, int t, const MsqBuffer* W, int rows, int cols, cons
     case MSQ_BF16: return launch_mv<DecDense<MSQ_BF16>>(st, s, a);
   }
   return unsupported("matvec", t, rows, cols);
+}
+
+int msq_bw_probe(void* stream, const MsqBuffer* src, size_t bytes, const MsqBuffer* sink) {
+  if (!buf_ok(src, bytes) || !buf_ok(sink, 4096) || bytes % 16 || ((uintptr_t)bptr(src) & 15))
+    return fail(MSQ_ERR_ARGUMENT, "macseek quant: bw_probe: buffer missing, too small or misaligned");
+  if (bytes == 0) return MSQ_OK;
+  const size_t n16 = bytes / 16;
+  const long grid = std::min<long>((long)((n16 + 1023) / 1024), (long)device_info().cus * 2);
+  hipLaunchKernelGGL(bw_probe_kernel, dim3((unsigned)grid), dim3(1024), 0, (hipStream_t)stream, (const uint4*)bptr(src), n16,
+                     (uint32_t*)bptr_mut(sink));
+  MSQ_HIP(hipGetLastError());
+  return MSQ_OK;
 }
 
 int msq_dequant(void* stream, int t, const MsqBuffer* W, int64_t n, const MsqBuffer* out) {

@@ -5,12 +5,19 @@
 // Expert e < n_routed is a routed expert (decoder DR); the shared expert (decoder DS, weight 1) keeps its h row at
 // index n_routed. Expert matrices are reached either through pointers passed by value or through a device-resident
 // table of 6 x {gate, up, down} 64-bit addresses that the host may fill after the launch was enqueued.
+//
+// Both kernels are persistent: about one 16-wave workgroup per CU, so the codebook tables are staged into LDS and the
+// activations into registers once per CU. Every wave owns a contiguous run of rows and a fixed K slice, streams its
+// rows with the next group's loads in flight while the current group is decoded, and parks per-row partial sums in
+// LDS; a workgroup synchronises only once per chunk of rows, to add the K-split / per-expert partials in a fixed
+// order and run the epilogue.
 #pragma once
 #include "msq_device.cuh"
 
 namespace msq {
 
 constexpr int kMaxRouted = 6;
+constexpr int kMoeChunkRows = 128;  // rows a workgroup finishes between two synchronisations
 
 struct MoeArgs {
   const float* x;        // [dim]
@@ -23,14 +30,14 @@ struct MoeArgs {
   const uint8_t* down[kMaxRouted];
   const uint8_t *sgate, *sup, *sdown;
   uint32_t n_routed;     // h row of the shared expert
-  uint32_t run_routed;   // experts this launch computes: routed ones (0 or n_routed) ...
+  uint32_t run_routed;   // experts this launch computes: routed ones (0 or 1) ...
   uint32_t run_shared;   // ... and / or the shared one
   uint32_t dim, inter;
   uint32_t rb_gu_r, rb_d_r, rb_gu_s, rb_d_s;  // row bytes: routed gate/up, routed down, shared gate/up, shared down
-  uint32_t ks, rpw;      // K-split waves, rows per wave per tile
-  uint32_t tiles_per_expert;  // gate/up: row tiles per expert
-  uint32_t grid_routed;       // gate/up: workgroups [0, grid_routed) take routed tiles, the rest shared tiles
-  uint32_t ntiles;            // down: row tiles
+  uint32_t ks;           // K-split waves
+  uint32_t grid_routed;  // gate/up: workgroups [0, grid_routed) take routed rows, the rest shared rows
+  uint32_t rows_per_wg_r, rows_per_wg_s;  // gate/up: virtual rows (expert * inter + row) per workgroup
+  uint32_t rows_per_wg;  // down: rows of y per workgroup
 };
 
 __device__ __forceinline__ float swiglu(float g, float u, float w) {  // quant_moe.metal:23-27
@@ -39,54 +46,107 @@ __device__ __forceinline__ float swiglu(float g, float u, float w) {  // quant_m
   return g / (1.f + expf(-g)) * u * w;
 }
 
-// gate + up + SwiGLU for the experts [e0, e0 + ne) of one kind; workgroup `wg` of `nwg` walks their row tiles.
+// Rows a wave keeps in flight per prefetch group: as many as fit about 24 registers of raw block bytes per buffer.
 template <class D>
-__device__ __forceinline__ void moe_gu_run(const MoeArgs& a, uint32_t* smem, bool shared, uint32_t wg, uint32_t nwg) {
+constexpr int rows_in_flight(int matrices) {
+  const int words = (int)(sizeof(typename D::Raw) / 4) * matrices;
+  return words <= 6 ? 4 : words <= 12 ? 2 : 1;
+}
+
+__device__ __forceinline__ uint32_t uniform(uint32_t v) { return (uint32_t)__builtin_amdgcn_readfirstlane((int)v); }
+
+// gate + up + SwiGLU over the virtual rows [wg * per, ...) of one kind of expert (routed: e * inter + r; shared: r).
+template <class D, int RPW>
+__device__ __forceinline__ void moe_gu_run(const MoeArgs& a, uint32_t* smem, const bool shared, const uint32_t wg) {
   uint32_t* tbl = smem;
   float* part = (float*)(smem + D::LDS_WORDS);
-  const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6, nwaves = blockDim.x >> 6;
+  const uint32_t tid = threadIdx.x, lane = tid & 63u;
+  const uint32_t wave = uniform(tid >> 6), nwaves = blockDim.x >> 6;
   const uint32_t KS = a.ks, ks = wave % KS, rw = wave / KS, RW = nwaves / KS;
-  const uint32_t tile_rows = RW * a.rpw;
   const uint32_t units = a.dim / D::UNIT;
   const uint32_t row_bytes = shared ? a.rb_gu_s : a.rb_gu_r;
-  const uint32_t n_exp = shared ? 1u : a.n_routed;
+  const uint32_t total = (shared ? 1u : a.n_routed) * a.inter;
+  const uint32_t per = shared ? a.rows_per_wg_s : a.rows_per_wg_r;
+  const uint32_t wg_begin = wg * per, wg_end = min(total, wg_begin + per);
 
-  D::fill_lds(tbl, (int)tid, (int)blockDim.x);
   const uint32_t u0 = ks * 64u + lane;
   const bool valid = u0 < units;
   const uint32_t unit = valid ? u0 : units - 1;
-  const typename D::X xr = D::load_x(a.x, unit);
-  if (D::LDS_WORDS) __syncthreads();
+  const uint32_t PSTRIDE = 4 * KS + 1;  // partial sums per (row, matrix): 4 sixteen-lane rows per K-split wave, padded
 
-  const uint32_t ntiles = n_exp * a.tiles_per_expert;
-  for (uint32_t tile = wg; tile < ntiles; tile += nwg) {
-    const uint32_t e = tile / a.tiles_per_expert;
-    const uint32_t tile_row0 = (tile - e * a.tiles_per_expert) * tile_rows;
-    const uint8_t *G, *U;
-    if (shared) { G = a.sgate; U = a.sup; }
-    else if (a.table) { G = (const uint8_t*)a.table[3 * e]; U = (const uint8_t*)a.table[3 * e + 1]; }
-    else { G = a.gate[e]; U = a.up[e]; }
-    const uint32_t row0 = tile_row0 + rw * a.rpw;
-    for (uint32_t j = 0; j < a.rpw; j++) {
-      const uint32_t row = min(row0 + j, a.inter - 1);
-      const size_t off = (size_t)row * row_bytes;
-      const typename D::Raw rg = D::load(G + off, unit), ru = D::load(U + off, unit);
-      float ag = dec_dot<D>(rg, xr, tbl, unit), au = dec_dot<D>(ru, xr, tbl, unit);
-      ag = wave_sum(valid ? ag : 0.f);
-      au = wave_sum(valid ? au : 0.f);
-      if (lane == 0) {
-        part[((rw * a.rpw + j) * 2 + 0) * KS + ks] = ag;
-        part[((rw * a.rpw + j) * 2 + 1) * KS + ks] = au;
+  // address of virtual row v of the gate (which = 0) or up (1) matrices
+  auto row_ptr = [&](uint32_t v, int which) -> const uint8_t* {
+    const uint32_t e = shared ? 0u : v / a.inter, r = v - e * a.inter;
+    const uint8_t* base;
+    if (shared) base = which ? a.sup : a.sgate;
+    else if (a.table) base = (const uint8_t*)a.table[3 * e + which];
+    else base = which ? a.up[e] : a.gate[e];
+    return base + (size_t)r * row_bytes;
+  };
+
+  typename D::X xr;
+  bool first = true;
+  for (uint32_t c0 = wg_begin; c0 < wg_end; c0 += kMoeChunkRows) {
+    const uint32_t c1 = min(wg_end, c0 + kMoeChunkRows), n = c1 - c0;
+    // rows of this chunk are dealt to the row-waves in contiguous runs
+    const uint32_t run = (n + RW - 1) / RW;
+    const uint32_t w0 = min(c0 + rw * run, c1), w1 = min(w0 + run, c1);
+    typename D::Raw cg[RPW], cu[RPW], ng[RPW], nu[RPW];
+    if (w0 < w1) {
+#pragma unroll
+      for (int j = 0; j < RPW; j++) {
+        const uint32_t v = min(w0 + j, w1 - 1);
+        cg[j] = D::load(row_ptr(v, 0), unit);
+        cu[j] = D::load(row_ptr(v, 1), unit);
+      }
+    }
+    if (first) {  // tables and activations arrive while the first weight rows are in flight
+      D::fill_lds(tbl, (int)tid, (int)blockDim.x);
+      xr = D::load_x(a.x, unit);
+      __syncthreads();
+      first = false;
+    }
+    for (uint32_t r0 = w0; r0 < w1; r0 += RPW) {
+      const bool more = r0 + RPW < w1;
+      if (more) {
+#pragma unroll
+        for (int j = 0; j < RPW; j++) {
+          const uint32_t v = min(r0 + RPW + j, w1 - 1);
+          ng[j] = D::load(row_ptr(v, 0), unit);
+          nu[j] = D::load(row_ptr(v, 1), unit);
+        }
+      }
+      float acc[2 * RPW];  // value 2 j + m: row j of the group, m = 0 gate, 1 up
+#pragma unroll
+      for (int j = 0; j < RPW; j++) {
+        const float g = dec_dot<D>(cg[j], xr, tbl, unit), u = dec_dot<D>(cu[j], xr, tbl, unit);
+        acc[2 * j] = valid ? g : 0.f;
+        acc[2 * j + 1] = valid ? u : 0.f;
+        asm volatile("" ::: "memory");  // one row pair's table lookups live at a time (register pressure)
+      }
+      row16_fold<2 * RPW>(acc, lane);
+      {
+        const uint32_t k = group8_sel<2 * RPW>(lane), j = k >> 1, m = k & 1u;
+        if (!(lane & 8u) && r0 + j < w1) part[((r0 + j - c0) * 2 + m) * PSTRIDE + ks * 4 + (lane >> 4)] = acc[0];
+      }
+      if (more) {
+#pragma unroll
+        for (int j = 0; j < RPW; j++) { cg[j] = ng[j]; cu[j] = nu[j]; }
       }
     }
     __syncthreads();
-    if (tid < tile_rows) {
-      const uint32_t row = tile_row0 + tid;
-      if (row < a.inter) {
-        float g = 0.f, u = 0.f;
-        for (uint32_t k = 0; k < KS; k++) { g += part[(tid * 2) * KS + k]; u += part[(tid * 2 + 1) * KS + k]; }
+    // thread q sums the partials of (row q / 2, matrix q % 2); gate and up then meet in the even lane
+    for (uint32_t q0 = 0; q0 < 2 * n; q0 += blockDim.x) {
+      const uint32_t q = q0 + tid;
+      float sum = 0.f;
+      if (q < 2 * n)
+        for (uint32_t k = 0; k < 4 * KS; k++) sum += part[q * PSTRIDE + k];
+      const float other = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, sum), 0xB1, 0xF, 0xF, false));
+      if (q < 2 * n && !(q & 1u)) {
+        const uint32_t v = c0 + (q >> 1);
+        const uint32_t e = shared ? 0u : v / a.inter, r = v - e * a.inter;
         const uint32_t he = shared ? a.n_routed : e;
-        a.h[(size_t)he * a.inter + row] = swiglu(g, u, shared ? 1.f : a.wts[e]);
+        a.h[(size_t)he * a.inter + r] = swiglu(sum, other, shared ? 1.f : a.wts[e]);
       }
     }
     __syncthreads();
@@ -96,79 +156,102 @@ __device__ __forceinline__ void moe_gu_run(const MoeArgs& a, uint32_t* smem, boo
 template <class DR, class DS>
 __global__ __launch_bounds__(1024) void moe_gu_kernel(const MoeArgs a) {
   extern __shared__ __attribute__((aligned(16))) uint32_t smem[];
-  if (blockIdx.x < a.grid_routed) moe_gu_run<DR>(a, smem, false, blockIdx.x, a.grid_routed);
-  else moe_gu_run<DS>(a, smem, true, blockIdx.x - a.grid_routed, gridDim.x - a.grid_routed);
+  if (blockIdx.x < a.grid_routed) moe_gu_run<DR, rows_in_flight<DR>(2)>(a, smem, false, blockIdx.x);
+  else moe_gu_run<DS, rows_in_flight<DS>(2)>(a, smem, true, blockIdx.x - a.grid_routed);
 }
 
 // down: workgroup = RW row-groups x (NE expert-waves x KS K-split waves). In a row-group, wave (e, ks) owns routed
-// expert e's K-slice ks of every row of the tile; afterwards the same waves share out the shared expert's rows.
+// expert e's K-slice ks of the row-group's rows; afterwards the same waves share out the shared expert's rows.
 // Per row the partial sums are added in the fixed order (expert 0 ks 0.., expert 1 .., shared ks 0..).
 template <class DR, class DS>
 __global__ __launch_bounds__(1024) void moe_down_kernel(const MoeArgs a) {
+  constexpr int RPW = rows_in_flight<DR>(1);
   extern __shared__ __attribute__((aligned(16))) uint32_t smem[];
   constexpr int TBL = DR::LDS_WORDS + DS::LDS_WORDS;
   uint32_t* tbl_r = smem;
   uint32_t* tbl_s = smem + DR::LDS_WORDS;
   float* part = (float*)(smem + TBL);
 
-  const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6, nwaves = blockDim.x >> 6;
+  const uint32_t tid = threadIdx.x, lane = tid & 63u;
+  const uint32_t wave = uniform(tid >> 6), nwaves = blockDim.x >> 6;
   const uint32_t KS = a.ks;
   const uint32_t NE = a.run_routed ? a.n_routed : 0u;       // routed experts computed here
-  const uint32_t wpg = max(NE, 1u) * KS;                    // waves per row-group
+  const uint32_t E = max(NE, 1u);
+  const uint32_t wpg = E * KS;                              // waves per row-group
   const uint32_t RW = nwaves / wpg, rg = wave / wpg, wl = wave % wpg;
   const uint32_t e = wl / KS, ks = wl % KS;
-  const uint32_t tile_rows = RW * a.rpw;
-  const uint32_t slots = NE * KS + (a.run_shared ? KS : 0u);  // partial sums per row
-
-  if (NE) DR::fill_lds(tbl_r, (int)tid, (int)blockDim.x);
-  if (a.run_shared) DS::fill_lds(tbl_s, (int)tid, (int)blockDim.x);
+  const uint32_t slots = 4 * (NE * KS + (a.run_shared ? KS : 0u));  // partial sums per row: 4 per contributing wave
+  const uint32_t PSTRIDE = slots + 1;
 
   const uint32_t u0 = ks * 64u + lane;
   const uint32_t units_r = a.inter / DR::UNIT, units_s = a.inter / DS::UNIT;
   const bool valid_r = NE && u0 < units_r, valid_s = a.run_shared && u0 < units_s;
   const uint32_t unit_r = u0 < units_r ? u0 : units_r - 1, unit_s = u0 < units_s ? u0 : units_s - 1;
+  const uint8_t* Dr = nullptr;
+  if (NE) Dr = a.table ? (const uint8_t*)a.table[3 * e + 2] : a.down[e];
+
+  const uint32_t wg_begin = blockIdx.x * a.rows_per_wg, wg_end = min(a.dim, wg_begin + a.rows_per_wg);
   typename DR::X xr;
   typename DS::X xs;
-  const uint8_t* Dr = nullptr;
-  if (NE) {
-    xr = DR::load_x(a.h + (size_t)e * a.inter, unit_r);
-    Dr = a.table ? (const uint8_t*)a.table[3 * e + 2] : a.down[e];
-  }
-  if (a.run_shared) xs = DS::load_x(a.h + (size_t)a.n_routed * a.inter, unit_s);
-  if (TBL) __syncthreads();
-
-  for (uint32_t tile = blockIdx.x; tile < a.ntiles; tile += gridDim.x) {
-    const uint32_t row0 = tile * tile_rows + rg * a.rpw;
+  bool first = true;
+  for (uint32_t c0 = wg_begin; c0 < wg_end; c0 += kMoeChunkRows) {
+    const uint32_t c1 = min(wg_end, c0 + kMoeChunkRows), n = c1 - c0;
+    const uint32_t run = (n + RW - 1) / RW;
+    const uint32_t w0 = min(c0 + rg * run, c1), w1 = min(w0 + run, c1);
+    typename DR::Raw cur[RPW], nxt[RPW];
+    if (NE && w0 < w1) {
+#pragma unroll
+      for (int j = 0; j < RPW; j++) cur[j] = DR::load(Dr + (size_t)min(w0 + j, w1 - 1) * a.rb_d_r, unit_r);
+    }
+    if (first) {
+      if (NE) { DR::fill_lds(tbl_r, (int)tid, (int)blockDim.x); xr = DR::load_x(a.h + (size_t)e * a.inter, unit_r); }
+      if (a.run_shared) { DS::fill_lds(tbl_s, (int)tid, (int)blockDim.x); xs = DS::load_x(a.h + (size_t)a.n_routed * a.inter, unit_s); }
+      __syncthreads();
+      first = false;
+    }
     if (NE) {
-#pragma unroll 4
-      for (uint32_t j = 0; j < a.rpw; j++) {
-        const uint32_t row = min(row0 + j, a.dim - 1);
-        const typename DR::Raw r = DR::load(Dr + (size_t)row * a.rb_d_r, unit_r);
-        float acc = dec_dot<DR>(r, xr, tbl_r, unit_r);
-        acc = wave_sum(valid_r ? acc : 0.f);
-        if (lane == 0) part[(rg * a.rpw + j) * slots + e * KS + ks] = acc;
+      for (uint32_t r0 = w0; r0 < w1; r0 += RPW) {
+        const bool more = r0 + RPW < w1;
+        if (more) {
+#pragma unroll
+          for (int j = 0; j < RPW; j++) nxt[j] = DR::load(Dr + (size_t)min(r0 + RPW + j, w1 - 1) * a.rb_d_r, unit_r);
+        }
+        float acc[RPW];
+#pragma unroll
+        for (int j = 0; j < RPW; j++) {
+          const float v = dec_dot<DR>(cur[j], xr, tbl_r, unit_r);
+          acc[j] = valid_r ? v : 0.f;
+          asm volatile("" ::: "memory");
+        }
+        row16_fold<RPW>(acc, lane);
+        {
+          const uint32_t j = group8_sel<RPW>(lane);
+          if (!(lane & 8u) && r0 + j < w1) part[(r0 + j - c0) * PSTRIDE + 4 * (e * KS + ks) + (lane >> 4)] = acc[0];
+        }
+        if (more) {
+#pragma unroll
+          for (int j = 0; j < RPW; j++) cur[j] = nxt[j];
+        }
       }
     }
     if (a.run_shared) {
-      // the row-group's waves with K-slice ks take the shared expert's rows e, e + E, ... of the tile
-      const uint32_t E = max(NE, 1u);
-#pragma unroll 2
-      for (uint32_t j = e; j < a.rpw; j += E) {
-        const uint32_t row = min(row0 + j, a.dim - 1);
-        const typename DS::Raw r = DS::load(a.sdown + (size_t)row * a.rb_d_s, unit_s);
-        float acc = dec_dot<DS>(r, xs, tbl_s, unit_s);
-        acc = wave_sum(valid_s ? acc : 0.f);
-        if (lane == 0) part[(rg * a.rpw + j) * slots + NE * KS + ks] = acc;
+      // the row-group's waves with K-slice ks take the shared expert's rows w0 + e, w0 + e + E, ...
+      for (uint32_t r0 = w0 + e; r0 < w1; r0 += 2 * E) {
+        const uint32_t r1 = r0 + E;
+        const typename DS::Raw ra = DS::load(a.sdown + (size_t)r0 * a.rb_d_s, unit_s);
+        const typename DS::Raw rb = DS::load(a.sdown + (size_t)min(r1, w1 - 1) * a.rb_d_s, unit_s);
+        const float va = dec_dot<DS>(ra, xs, tbl_s, unit_s), vb = dec_dot<DS>(rb, xs, tbl_s, unit_s);
+        float acc[2] = {valid_s ? va : 0.f, valid_s ? vb : 0.f};
+        row16_fold<2>(acc, lane);
+        const uint32_t r = group8_sel<2>(lane) ? r1 : r0;
+        if (!(lane & 8u) && r < w1) part[(r - c0) * PSTRIDE + 4 * (NE * KS + ks) + (lane >> 4)] = acc[0];
       }
     }
     __syncthreads();
-    if (tid < tile_rows) {
-      const uint32_t row = tile * tile_rows + tid;
-      if (row < a.dim) {
-        float s = 0.f;
-        for (uint32_t k = 0; k < slots; k++) s += part[tid * slots + k];
-        a.y[row] += s;
-      }
+    for (uint32_t t = tid; t < n; t += blockDim.x) {
+      float s = 0.f;
+      for (uint32_t k = 0; k < slots; k++) s += part[t * PSTRIDE + k];
+      a.y[c0 + t] += s;
     }
     __syncthreads();
   }

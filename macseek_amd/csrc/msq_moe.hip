@@ -1,5 +1,6 @@
 // C ABI: fused one-token MoE layer (see include/msq.h; reference host code src/kernels/quant.mm:252-369).
 #include <algorithm>
+#include <cstdlib>
 
 #include "msq_host.h"
 #include "msq_moe.cuh"
@@ -17,6 +18,11 @@ void launch_gu_t(dim3 g, dim3 b, size_t lds, hipStream_t st, const MoeArgs& a) {
 template <class DR, class DS>
 void launch_down_t(dim3 g, dim3 b, size_t lds, hipStream_t st, const MoeArgs& a) {
   hipLaunchKernelGGL((moe_down_kernel<DR, DS>), g, b, lds, st, a);
+}
+// launch-shape knobs for experiments (the reference exposes MACSEEK_MOE_* the same way, quant.mm:274-276)
+int env_int(const char* name, int dflt) {
+  const char* v = getenv(name);
+  return v && *v ? atoi(v) : dflt;
 }
 template <class DR>
 size_t lds_words_for_shared(int ts, bool down) {
@@ -108,26 +114,26 @@ int moe_decode_impl(hipStream_t st, const MsqMoeDecodeArgs* p, const MsqBuffer* 
   const int cus = device_info().cus;
 
   // 1) gate + up + SwiGLU -> h
+  static const int env_gu_wgs = env_int("MSQ_MOE_GU_WGS", 1), env_d_wgs = env_int("MSQ_MOE_D_WGS", 1);
+  static const int env_gu_rsg = env_int("MSQ_MOE_GU_RSG", 0), env_d_rsg = env_int("MSQ_MOE_D_RSG", 0);
   const int n_gu_r = (gu_r && routed_live) ? nr : 0;
   if (n_gu_r > 0 || gu_s) {
     const int units = dim / 32;
     const int ks = (units + 63) / 64;
-    int rw = p->gu_rsg > 0 ? p->gu_rsg : std::max(1, 8 / ks);
+    int rw = p->gu_rsg > 0 ? p->gu_rsg : env_gu_rsg > 0 ? env_gu_rsg : std::max(1, 16 / ks);
     if (rw * ks > 16) rw = std::max(1, 16 / ks);
-    const int rpw = p->gu_nr > 0 ? std::min(p->gu_nr, 64) : 8;
-    const int tile_rows = rw * rpw, threads = 64 * rw * ks;
-    a.ks = (uint32_t)ks; a.rpw = (uint32_t)rpw;
-    a.tiles_per_expert = (uint32_t)((inter + tile_rows - 1) / tile_rows);
+    const int threads = 64 * rw * ks;
+    a.ks = (uint32_t)ks;
     a.run_routed = n_gu_r > 0; a.run_shared = gu_s;
-    const size_t part_bytes = (size_t)tile_rows * 2 * ks * 4;
-    // persistent workgroups, shared between the routed experts and the shared expert in proportion to their bytes
-    const long tiles_r = (long)n_gu_r * a.tiles_per_expert, tiles_s = gu_s ? a.tiles_per_expert : 0;
-    const int wg_per_cu = std::max(1, std::min(2048 / threads, 4));
-    const long total = std::min<long>(tiles_r + tiles_s, (long)cus * wg_per_cu);
+    const size_t part_bytes = (size_t)kMoeChunkRows * 2 * (4 * ks + 1) * 4;
+    // persistent workgroups, dealt to the routed experts and the shared expert in proportion to their bytes
+    const long rows_r = (long)n_gu_r * inter, rows_s = gu_s ? inter : 0;
+    const long total = std::max<long>(2, (long)cus * std::max(1, env_gu_wgs));
     const double br = (double)n_gu_r * a.rb_gu_r, bs = gu_s ? (double)a.rb_gu_s : 0.0;
     long g_s = gu_s ? std::max<long>(1, (long)(total * bs / (br + bs) + 0.5)) : 0;
-    g_s = std::min(g_s, tiles_s);
-    long g_r = n_gu_r ? std::max<long>(1, std::min(tiles_r, total - g_s)) : 0;
+    long g_r = n_gu_r ? std::max<long>(1, total - g_s) : 0;
+    if (g_r) { a.rows_per_wg_r = (uint32_t)((rows_r + g_r - 1) / g_r); g_r = (rows_r + a.rows_per_wg_r - 1) / a.rows_per_wg_r; }
+    if (g_s) { a.rows_per_wg_s = (uint32_t)((rows_s + g_s - 1) / g_s); g_s = (rows_s + a.rows_per_wg_s - 1) / a.rows_per_wg_s; }
     a.grid_routed = (uint32_t)g_r;
     if (!dispatch<false>(p->t_gate_up, ts, dim3((unsigned)(g_r + g_s)), dim3(threads), part_bytes, st, a))
       return unsupported("moe_decode type combo", p->t_gate_up, 0, 0);
@@ -141,17 +147,16 @@ int moe_decode_impl(hipStream_t st, const MsqMoeDecodeArgs* p, const MsqBuffer* 
     const int ne = run_d_r ? nr : 1;
     const int wpg = ne * ks;
     if (wpg > 16) return unsupported("moe_decode inter too large for the down kernel", p->t_down, dim, inter);
-    int rw = p->d_rsg > 0 ? p->d_rsg : std::max(1, 8 / wpg);
+    int rw = p->d_rsg > 0 ? p->d_rsg : env_d_rsg > 0 ? env_d_rsg : std::max(1, 16 / wpg);
     if (rw * wpg > 16) rw = std::max(1, 16 / wpg);
-    const int rpw = p->d_nr > 0 ? std::min(p->d_nr, 64) : 16;
-    const int tile_rows = rw * rpw, threads = 64 * rw * wpg;
-    a.ks = (uint32_t)ks; a.rpw = (uint32_t)rpw;
+    const int threads = 64 * rw * wpg;
+    a.ks = (uint32_t)ks;
     a.run_routed = run_d_r; a.run_shared = d_s;
-    a.ntiles = (uint32_t)((dim + tile_rows - 1) / tile_rows);
-    const size_t slots = (size_t)(run_d_r ? nr * ks : 0) + (d_s ? ks : 0);
-    const size_t part_bytes = (size_t)tile_rows * slots * 4;
-    const int wg_per_cu = std::max(1, std::min(2048 / threads, 4));
-    const long grid = std::min<long>(a.ntiles, (long)cus * wg_per_cu);
+    const size_t slots = 4 * ((size_t)(run_d_r ? nr * ks : 0) + (d_s ? ks : 0));
+    const size_t part_bytes = (size_t)kMoeChunkRows * (slots + 1) * 4;
+    const long total = std::max<long>(1, (long)cus * std::max(1, env_d_wgs));
+    a.rows_per_wg = (uint32_t)((dim + total - 1) / total);
+    const long grid = (dim + a.rows_per_wg - 1) / a.rows_per_wg;
     if (!dispatch<true>(p->t_down, ts, dim3((unsigned)grid), dim3(threads), part_bytes, st, a))
       return unsupported("moe_decode type combo", p->t_down, 0, 0);
     MSQ_HIP(hipGetLastError());
