@@ -18,6 +18,7 @@ namespace msq {
 
 constexpr int kMaxRouted = 6;
 constexpr int kMoeChunkRows = 128;  // rows a workgroup finishes between two synchronisations
+constexpr bool kStagedGateUp = false;  // stream gate/up weights through LDS staging (coalesced 128-bit loads)
 
 struct MoeArgs {
   const float* x;        // [dim]
@@ -57,7 +58,7 @@ __device__ __forceinline__ uint32_t uniform(uint32_t v) { return (uint32_t)__bui
 
 // gate + up + SwiGLU over the virtual rows [wg * per, ...) of one kind of expert (routed: e * inter + r; shared: r).
 template <class D, int RPW>
-__device__ __forceinline__ void moe_gu_run(const MoeArgs& a, uint32_t* smem, const bool shared, const uint32_t wg) {
+__device__ __forceinline__ void moe_gu_run_direct(const MoeArgs& a, uint32_t* smem, const bool shared, const uint32_t wg) {
   uint32_t* tbl = smem;
   float* part = (float*)(smem + D::LDS_WORDS);
   const uint32_t tid = threadIdx.x, lane = tid & 63u;
@@ -153,11 +154,126 @@ __device__ __forceinline__ void moe_gu_run(const MoeArgs& a, uint32_t* smem, con
   }
 }
 
+// Same computation with the weights streamed through LDS staging (decoders with SLICE_BYTES > 0): per row pair a wave
+// issues two coalesced 128-bit loads (its K slice of the gate row and of the up row), DEPTH row pairs ahead.
+template <class D>
+__device__ __forceinline__ void moe_gu_run_staged(const MoeArgs& a, uint32_t* smem, const bool shared, const uint32_t wg) {
+  constexpr int DEPTH = MSQ_GU_DEPTH;
+  uint32_t* tbl = smem;
+  const uint32_t tid = threadIdx.x, lane = tid & 63u;
+  const uint32_t wave = uniform(tid >> 6), nwaves = blockDim.x >> 6;
+  const uint32_t KS = a.ks, ks = wave % KS, rw = wave / KS, RW = nwaves / KS;
+  const uint32_t PSTRIDE = 4 * KS + 1;
+  float* part = (float*)(smem + D::LDS_WORDS);
+  uint8_t* stage_g = (uint8_t*)(part + kMoeChunkRows * 2 * PSTRIDE) + (size_t)wave * 2 * kStageBytes;
+  uint8_t* stage_u = stage_g + kStageBytes;
+  const uint32_t units = a.dim / D::UNIT;
+  const uint32_t row_bytes = shared ? a.rb_gu_s : a.rb_gu_r;
+  const uint32_t total = (shared ? 1u : a.n_routed) * a.inter;
+  const uint32_t per = shared ? a.rows_per_wg_s : a.rows_per_wg_r;
+  const uint32_t wg_begin = wg * per, wg_end = min(total, wg_begin + per);
+
+  const uint32_t u0 = ks * 64u + lane;
+  const bool valid = u0 < units;
+  const uint32_t unit = valid ? u0 : units - 1;           // activations: idle lanes shadow the last unit
+  const uint32_t lunit = valid ? lane : (units - 1) & 63u;  // unit inside the staged slice
+  const uint32_t slice_off = ks * (uint32_t)D::SLICE_BYTES;
+  const uint32_t slice_bytes = min((uint32_t)D::SLICE_BYTES, row_bytes - slice_off);
+
+  auto row_ptr = [&](uint32_t v, int which) -> const uint8_t* {
+    const uint32_t e = shared ? 0u : v / a.inter, r = v - e * a.inter;
+    const uint8_t* base;
+    if (shared) base = which ? a.sup : a.sgate;
+    else if (a.table) base = (const uint8_t*)a.table[3 * e + which];
+    else base = which ? a.up[e] : a.gate[e];
+    return base + (size_t)r * row_bytes + slice_off;
+  };
+
+  typename D::X xr;
+  bool first = true;
+  for (uint32_t c0 = wg_begin; c0 < wg_end; c0 += kMoeChunkRows) {
+    const uint32_t c1 = min(wg_end, c0 + kMoeChunkRows), n = c1 - c0;
+    const uint32_t run = (n + RW - 1) / RW;
+    const uint32_t w0 = min(c0 + rw * run, c1), w1 = min(w0 + run, c1);
+    uint4 pg[DEPTH], pu[DEPTH];
+    uint32_t sg[DEPTH], su[DEPTH];  // shift of each in-flight slice inside its first 16-byte granule
+#pragma unroll
+    for (int s = 0; s < DEPTH; s++) {
+      if (w0 + s < w1) {
+        const uint8_t *g = row_ptr(w0 + s, 0), *u = row_ptr(w0 + s, 1);
+        pg[s] = slice_load(g, slice_bytes, lane); sg[s] = (uint32_t)((uintptr_t)g & 15u);
+        pu[s] = slice_load(u, slice_bytes, lane); su[s] = (uint32_t)((uintptr_t)u & 15u);
+      }
+    }
+    if (first) {  // tables and activations arrive while the first weight rows are in flight
+      D::fill_lds(tbl, (int)tid, (int)blockDim.x);
+      xr = D::load_x(a.x, unit);
+      __syncthreads();
+      first = false;
+    }
+    for (uint32_t r0 = w0; r0 < w1; r0 += DEPTH) {
+      float acc[2 * DEPTH];
+#pragma unroll
+      for (int s = 0; s < DEPTH; s++) {
+        if (r0 + s < w1) {  // wave-uniform
+          slice_stage(stage_g, pg[s], lane);
+          slice_stage(stage_u, pu[s], lane);
+          const uint32_t shg = sg[s], shu = su[s];
+          if (r0 + s + DEPTH < w1) {  // refill the slot: DEPTH row pairs stay in flight
+            const uint8_t *g = row_ptr(r0 + s + DEPTH, 0), *u = row_ptr(r0 + s + DEPTH, 1);
+            pg[s] = slice_load(g, slice_bytes, lane); sg[s] = (uint32_t)((uintptr_t)g & 15u);
+            pu[s] = slice_load(u, slice_bytes, lane); su[s] = (uint32_t)((uintptr_t)u & 15u);
+          }
+          const typename D::Raw rg = D::load(stage_g + shg, lunit), ru = D::load(stage_u + shu, lunit);
+          const float g = dec_dot<D>(rg, xr, tbl, unit), u = dec_dot<D>(ru, xr, tbl, unit);
+          acc[2 * s] = valid ? g : 0.f;
+          acc[2 * s + 1] = valid ? u : 0.f;
+        } else {
+          acc[2 * s] = 0.f; acc[2 * s + 1] = 0.f;
+        }
+        asm volatile("" ::: "memory");  // one row pair's table lookups live at a time (register pressure)
+      }
+      row16_fold<2 * DEPTH>(acc, lane);
+      {
+        const uint32_t k = group8_sel<2 * DEPTH>(lane), j = k >> 1, m = k & 1u;
+        if (!(lane & 8u) && r0 + j < w1) part[((r0 + j - c0) * 2 + m) * PSTRIDE + ks * 4 + (lane >> 4)] = acc[0];
+      }
+    }
+    __syncthreads();
+    for (uint32_t q0 = 0; q0 < 2 * n; q0 += blockDim.x) {
+      const uint32_t q = q0 + tid;
+      float sum = 0.f;
+      if (q < 2 * n)
+        for (uint32_t k = 0; k < 4 * KS; k++) sum += part[q * PSTRIDE + k];
+      const float other = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, sum), 0xB1, 0xF, 0xF, false));
+      if (q < 2 * n && !(q & 1u)) {
+        const uint32_t v = c0 + (q >> 1);
+        const uint32_t e = shared ? 0u : v / a.inter, r = v - e * a.inter;
+        const uint32_t he = shared ? a.n_routed : e;
+        a.h[(size_t)he * a.inter + r] = swiglu(sum, other, shared ? 1.f : a.wts[e]);
+      }
+    }
+    __syncthreads();
+  }
+}
+
+template <class D>
+__device__ __forceinline__ void moe_gu_run(const MoeArgs& a, uint32_t* smem, const bool shared, const uint32_t wg) {
+  if constexpr (kStagedGateUp && D::SLICE_BYTES > 0) moe_gu_run_staged<D>(a, smem, shared, wg);
+  else moe_gu_run_direct<D, rows_in_flight<D>(2)>(a, smem, shared, wg);
+}
+
+#ifndef MSQ_GU_DEPTH
+#define MSQ_GU_DEPTH 4
+#endif
+#ifndef MSQ_GU_MINBLOCKS
+#define MSQ_GU_MINBLOCKS 1
+#endif
 template <class DR, class DS>
-__global__ __launch_bounds__(1024) void moe_gu_kernel(const MoeArgs a) {
+__global__ __launch_bounds__(1024, MSQ_GU_MINBLOCKS) void moe_gu_kernel(const MoeArgs a) {
   extern __shared__ __attribute__((aligned(16))) uint32_t smem[];
-  if (blockIdx.x < a.grid_routed) moe_gu_run<DR, rows_in_flight<DR>(2)>(a, smem, false, blockIdx.x);
-  else moe_gu_run<DS, rows_in_flight<DS>(2)>(a, smem, true, blockIdx.x - a.grid_routed);
+  if (blockIdx.x < a.grid_routed) moe_gu_run<DR>(a, smem, false, blockIdx.x);
+  else moe_gu_run<DS>(a, smem, true, blockIdx.x - a.grid_routed);
 }
 
 // down: workgroup = RW row-groups x (NE expert-waves x KS K-split waves). In a row-group, wave (e, ks) owns routed
