@@ -158,7 +158,7 @@ __device__ __forceinline__ void moe_gu_run_direct(const MoeArgs& a, uint32_t* sm
 // issues two coalesced 128-bit loads (its K slice of the gate row and of the up row), DEPTH row pairs ahead.
 template <class D>
 __device__ __forceinline__ void moe_gu_run_staged(const MoeArgs& a, uint32_t* smem, const bool shared, const uint32_t wg) {
-  constexpr int DEPTH = MSQ_GU_DEPTH;
+  constexpr int DEPTH = 4;
   uint32_t* tbl = smem;
   const uint32_t tid = threadIdx.x, lane = tid & 63u;
   const uint32_t wave = uniform(tid >> 6), nwaves = blockDim.x >> 6;
@@ -263,14 +263,8 @@ __device__ __forceinline__ void moe_gu_run(const MoeArgs& a, uint32_t* smem, con
   else moe_gu_run_direct<D, rows_in_flight<D>(2)>(a, smem, shared, wg);
 }
 
-#ifndef MSQ_GU_DEPTH
-#define MSQ_GU_DEPTH 4
-#endif
-#ifndef MSQ_GU_MINBLOCKS
-#define MSQ_GU_MINBLOCKS 1
-#endif
 template <class DR, class DS>
-__global__ __launch_bounds__(1024, MSQ_GU_MINBLOCKS) void moe_gu_kernel(const MoeArgs a) {
+__global__ __launch_bounds__(1024) void moe_gu_kernel(const MoeArgs a) {
   extern __shared__ __attribute__((aligned(16))) uint32_t smem[];
   if (blockIdx.x < a.grid_routed) moe_gu_run<DR>(a, smem, false, blockIdx.x);
   else moe_gu_run<DS>(a, smem, true, blockIdx.x - a.grid_routed);
