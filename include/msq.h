@@ -76,6 +76,15 @@ int msq_matvec_cfg(int qtype, int rows, int cols, MsqMvCfg* out);
 int msq_matvec(void* stream, int qtype, const MsqBuffer* W, int rows, int cols, const MsqBuffer* x,
                const MsqBuffer* y, int accumulate, int groups, const MsqMvCfg* cfg);
 
+/* reference: ms::q::encode_matvec_n (quant.hpp:32-35, quant.mm:129-156).
+ * Y[n x rows] (+)= X[n x cols] . W^T for n in 1..16 (one weight read serves all n tokens). X row stride is
+ * cols * groups, Y row stride is rows. n == 1 is exactly msq_matvec. For n >= 2 the block formats, F16 and BF16 run
+ * on the matrix cores with activations rounded to fp16 (BF16 weights: split into two bf16 terms) and exact weights;
+ * the reference rounds activations to fp16 the same way and, from n >= 8, weights too (quant.mm:133-137). F32 weights,
+ * and block-diagonal calls whose group size is not a multiple of 16 rows, are served as n decode matvecs. */
+int msq_matvec_n(void* stream, int qtype, const MsqBuffer* W, int rows, int cols, const MsqBuffer* X,
+                 const MsqBuffer* Y, int n, int accumulate, int groups);
+
 /* Whole-buffer dequantization to fp32, bit-exact with the reference's CPU dequantizer
  * (reference: ref::dequant_row, tests/ref/dequant.cpp:34-120; GPU relative: q_deq_f16, quant_mm.metal:143-154).
  * n_elems must be a multiple of the block size; out holds n_elems floats. */

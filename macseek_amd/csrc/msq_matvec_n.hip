@@ -1,0 +1,78 @@
+// C ABI: small-N matvec (see include/msq.h; reference host code src/kernels/quant.mm:129-156).
+#include <algorithm>
+
+#include "msq_host.h"
+#include "msq_mvn.cuh"
+
+namespace msq {
+namespace {
+
+template <class F>
+int launch_mvn(hipStream_t st, MvnArgs a) {
+  const uint32_t total_steps = a.cols / 32u;
+  const uint32_t chunk_steps = 16u * kMvnMaxSteps;  // 16 waves x 16 steps = 8192 columns per launch
+  const int cus = device_info().cus;
+  for (uint32_t first = 0; first < total_steps; first += chunk_steps) {
+    MvnArgs c = a;
+    c.nsteps = std::min(chunk_steps, total_steps - first);
+    c.col0 = 32u * first;
+    c.col0_bytes = (uint32_t)msq_type_row_bytes_of_cols(a, c.col0);
+    if (first > 0) c.accumulate = 1u;
+    const uint32_t ks = std::min<uint32_t>(16u, c.nsteps);
+    c.steps_per_wave = (c.nsteps + ks - 1) / ks;
+    const uint32_t waves = (c.nsteps + c.steps_per_wave - 1) / c.steps_per_wave;
+    const size_t lds = (size_t)F::LDS_WORDS * 4 + (size_t)waves * 16 * 17 * 4;
+    const int wg_per_cu = std::max(1, std::min<int>(2048 / (64 * (int)waves), 2));
+    const long grid = std::min<long>(c.ntiles, (long)cus * wg_per_cu);
+    hipLaunchKernelGGL((mvn_kernel<F>), dim3((unsigned)grid), dim3(64 * waves), lds, st, c);
+    MSQ_HIP(hipGetLastError());
+  }
+  return MSQ_OK;
+}
+
+}  // namespace
+}  // namespace msq
+
+using namespace msq;
+
+extern "C" int msq_matvec_n(void* stream, int t, const MsqBuffer* W, int rows, int cols, const MsqBuffer* X,
+                            const MsqBuffer* Y, int n, int accumulate, int groups) {
+  if (n == 1) return msq_matvec(stream, t, W, rows, cols, X, Y, accumulate, groups, nullptr);
+  const int be = msq_type_block_elems(t);
+  const int colmul = be == 1 ? 256 : be;
+  if (!msq_matvec_supported(t) || n < 1 || n > 16 || rows < 1 || cols < 1 || cols % colmul || groups < 1 || rows % groups)
+    return unsupported("matvec_n", t, rows, cols);
+  const size_t rb = msq_type_row_bytes(t, cols);
+  const size_t xs = (size_t)cols * groups;
+  if (!buf_ok(W, rb * (size_t)rows) || !buf_ok(X, xs * n * 4) || !buf_ok(Y, (size_t)rows * n * 4))
+    return fail(MSQ_ERR_ARGUMENT, "macseek quant: matvec_n: buffer missing or too small (type %s rows %d cols %d n %d)",
+                msq_type_name_of(t), rows, cols, n);
+  const int rpg = rows / groups;
+  if (t == MSQ_F32 || (groups > 1 && rpg % 16)) {  // served as n decode matvecs
+    for (int i = 0; i < n; i++) {
+      const MsqBuffer xi{X->dev, X->off + (size_t)i * xs * 4, xs * 4}, yi{Y->dev, Y->off + (size_t)i * rows * 4, (size_t)rows * 4};
+      const int rc = msq_matvec(stream, t, W, rows, cols, &xi, &yi, accumulate, groups, nullptr);
+      if (rc != MSQ_OK) return rc;
+    }
+    return MSQ_OK;
+  }
+  MvnArgs a{};
+  a.W = bptr(W); a.X = (const float*)bptr(X); a.Y = (float*)bptr_mut(Y);
+  a.rows = (uint32_t)rows; a.cols = (uint32_t)cols; a.row_bytes = (uint32_t)rb; a.n = (uint32_t)n;
+  a.x_stride = (uint32_t)xs; a.y_stride = (uint32_t)rows;
+  a.rows_per_group = (uint32_t)rpg; a.x_group_stride = (uint32_t)cols; a.accumulate = accumulate ? 1u : 0u;
+  a.ntiles = (uint32_t)((rows + 15) / 16);
+  a.qtype = t;
+  hipStream_t st = (hipStream_t)stream;
+  switch (t) {
+    case MSQ_IQ1_S: return launch_mvn<FragIQ1S>(st, a);
+    case MSQ_IQ2_XXS: return launch_mvn<FragIQ2XXS>(st, a);
+    case MSQ_Q8_0: return launch_mvn<FragQ8_0>(st, a);
+    case MSQ_IQ4_NL: return launch_mvn<FragIQ4NL>(st, a);
+    case MSQ_Q6_K: return launch_mvn<FragQ6K>(st, a);
+    case MSQ_Q5_K: return launch_mvn<FragQ5K>(st, a);
+    case MSQ_F16: return launch_mvn<FragDense16<MSQ_F16>>(st, a);
+    case MSQ_BF16: return launch_mvn<FragDense16<MSQ_BF16>>(st, a);
+  }
+  return unsupported("matvec_n", t, rows, cols);
+}

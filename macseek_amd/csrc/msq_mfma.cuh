@@ -1,0 +1,204 @@
+// MFMA building blocks for the multi-token paths (small-N matvec_n and the prefill grouped MoE GEMM).
+//
+// v_mfma_f32_16x16x32_{f16,bf16}: D[16 x 16] += A[16 x 32] . B[32 x 16], one wave.
+//   A operand: lane l holds row  (l % 16), eight K positions 8 * (l / 16) .. + 7   (activations: row = token)
+//   B operand: lane l holds col  (l % 16), the same eight K positions               (weights: col = weight row)
+//   D operand: lane l holds col  (l % 16), rows 4 * (l / 16) + i, i = 0..3          (token, weight row)
+// A and B only have to agree on which matrix column each K position means, so every format is free to pick the
+// column order that makes its fragment cheap to decode (Frag::col_of).
+//
+// A fragment decoder turns the bytes of 8 weights of one row into 8 exact fp16 (or bf16) payloads plus an fp32 scale
+// that is applied to the MFMA result, so weights are never rounded: weight = scale * payload (+ add, Q5_K only, which
+// multiplies the per-token sum of the K step's activations).
+#pragma once
+#include "msq_device.cuh"
+
+namespace msq {
+
+typedef __bf16 bf8_t __attribute__((ext_vector_type(8)));
+
+__device__ __forceinline__ f4_t mfma_f16(const uint32_t a[4], const uint32_t b[4], f4_t c) {
+  typedef uint32_t u4_t __attribute__((ext_vector_type(4)));
+  const u4_t av = {a[0], a[1], a[2], a[3]}, bv = {b[0], b[1], b[2], b[3]};
+  return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8_t, av), __builtin_bit_cast(h8_t, bv), c, 0, 0, 0);
+}
+__device__ __forceinline__ f4_t mfma_bf16(const uint32_t a[4], const uint32_t b[4], f4_t c) {
+  typedef uint32_t u4_t __attribute__((ext_vector_type(4)));
+  const u4_t av = {a[0], a[1], a[2], a[3]}, bv = {b[0], b[1], b[2], b[3]};
+  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf8_t, av), __builtin_bit_cast(bf8_t, bv), c, 0, 0, 0);
+}
+
+__device__ __forceinline__ uint32_t pk_add_f16(uint32_t a, uint32_t b) {
+  const h2_t r = as_h2(a) + as_h2(b);
+  return __builtin_bit_cast(uint32_t, r);
+}
+// float -> bf16 bits, round to nearest even (finite inputs)
+__device__ __forceinline__ uint32_t bf16_rne(float f) {
+  const uint32_t u = __builtin_bit_cast(uint32_t, f);
+  return (u + 0x7FFFu + ((u >> 16) & 1u)) >> 16;
+}
+
+// ================================================================================================ fragments
+// Interface of a fragment decoder F (one K step = 32 matrix columns, chunk q = l / 16 of the step, 8 positions p):
+//   BF16_MATH          payloads are bf16 (activations are then split into two bf16 terms) instead of fp16
+//   HAS_ADD            weight = scale * payload + add
+//   LDS_WORDS, fill_lds
+//   col_of(q, p)       column (0..31 inside the step) that position p of chunk q stands for
+//   get(row, step, q, tbl, h, scale, add)   payloads of the 8 weights of weight row `row` (pointer to its first byte)
+struct FragOut {
+  uint32_t h[4];
+  float scale, add;
+};
+
+struct FragIQ1S {
+  static constexpr bool BF16_MATH = false, HAS_ADD = false;
+  static constexpr int LDS_WORDS = MSQ_IQ1S_GRID_N * 4;
+  __device__ static void fill_lds(uint32_t* lds, int tid, int nt) { copy_words16(lds, g_tbl_iq1s.w, LDS_WORDS, tid, nt); }
+  __device__ static uint32_t col_of(uint32_t q, uint32_t p) { return 8u * q + p; }
+  __device__ static FragOut get(const uint8_t* row, uint32_t step, uint32_t q, const uint32_t* tbl) {
+    const uint8_t* b = row + (step >> 3) * 50u;
+    const uint32_t ib = step & 7u;
+    const uint32_t qh = ld16(b + 34 + 2 * ib);
+    const uint32_t idx = ld8(b + 2 + 4 * ib + q) | (((qh >> (3 * q)) & 7u) << 8);
+    const uint4 g = ((const uint4*)tbl)[idx];
+    const uint32_t delta2 = (qh & 0x8000u) ? 0xB000B000u : 0x30003000u;  // -0.125 / +0.125 in both halves
+    FragOut o;
+    o.h[0] = pk_add_f16(g.x, delta2); o.h[1] = pk_add_f16(g.y, delta2);  // grid + delta is exact in fp16
+    o.h[2] = pk_add_f16(g.z, delta2); o.h[3] = pk_add_f16(g.w, delta2);
+    o.scale = half_bits_to_float(ld16(b)) * (float)(2u * ((qh >> 12) & 7u) + 1u);
+    o.add = 0.f;
+    return o;
+  }
+};
+
+struct FragIQ2XXS {
+  static constexpr bool BF16_MATH = false, HAS_ADD = false;
+  static constexpr int LDS_WORDS = MSQ_IQ2XXS_GRID_N * 4 + 128 * 4;
+  __device__ static void fill_lds(uint32_t* lds, int tid, int nt) { DecIQ2XXS::fill_lds(lds, tid, nt); }
+  __device__ static uint32_t col_of(uint32_t q, uint32_t p) { return 8u * q + p; }
+  __device__ static FragOut get(const uint8_t* row, uint32_t step, uint32_t q, const uint32_t* tbl) {
+    const uint8_t* b = row + (step >> 3) * 66u;
+    const uint8_t* a8 = b + 2 + 8 * (step & 7u);
+    const uint32_t a1 = ld32(a8 + 4);
+    const uint4 g = ((const uint4*)tbl)[ld8(a8 + q)];
+    const uint4 s = ((const uint4*)(tbl + MSQ_IQ2XXS_GRID_N * 4))[(a1 >> (7 * q)) & 127u];
+    FragOut o;
+    o.h[0] = g.x ^ s.x; o.h[1] = g.y ^ s.y; o.h[2] = g.z ^ s.z; o.h[3] = g.w ^ s.w;
+    o.scale = half_bits_to_float(ld16(b)) * (0.5f + (float)(a1 >> 28)) * 0.25f;
+    o.add = 0.f;
+    return o;
+  }
+};
+
+struct FragQ8_0 {
+  static constexpr bool BF16_MATH = false, HAS_ADD = false;
+  static constexpr int LDS_WORDS = 0;
+  __device__ static void fill_lds(uint32_t*, int, int) {}
+  __device__ static uint32_t col_of(uint32_t q, uint32_t p) { return 8u * q + p; }
+  __device__ static FragOut get(const uint8_t* row, uint32_t step, uint32_t q, const uint32_t*) {
+    const uint8_t* b = row + step * 34u;
+    const u64_a2 v = ld64(b + 2 + 8 * q);
+    const uint32_t lo = v.x ^ 0x80808080u, hi = v.y ^ 0x80808080u;  // bytes become q + 128
+    const uint32_t bias = 0xE480E480u;                              // -1152 in both halves
+    FragOut o;
+    o.h[0] = pk_add_f16(bytes01_to_h2_1024(lo), bias); o.h[1] = pk_add_f16(bytes23_to_h2_1024(lo), bias);
+    o.h[2] = pk_add_f16(bytes01_to_h2_1024(hi), bias); o.h[3] = pk_add_f16(bytes23_to_h2_1024(hi), bias);
+    o.scale = half_bits_to_float(ld16(b));
+    o.add = 0.f;
+    return o;
+  }
+};
+
+// IQ4_NL: byte j of a block holds columns j (low nibble) and j + 16 (high nibble); chunk q takes bytes 4q .. 4q + 3, so
+// its positions (2i, 2i + 1) stand for columns (4q + i, 4q + i + 16) and one table lookup per byte yields both.
+struct FragIQ4NL {
+  static constexpr bool BF16_MATH = false, HAS_ADD = false;
+  static constexpr int LDS_WORDS = 256;
+  __device__ static void fill_lds(uint32_t* lds, int tid, int nt) { copy_words16(lds, g_tbl_iq4nl.w, 256, tid, nt); }
+  __device__ static uint32_t col_of(uint32_t q, uint32_t p) { return 4u * q + (p >> 1) + 16u * (p & 1u); }
+  __device__ static FragOut get(const uint8_t* row, uint32_t step, uint32_t q, const uint32_t* tbl) {
+    const uint8_t* b = row + step * 18u;
+    const uint32_t v = ld32(b + 2 + 4 * q);
+    FragOut o;
+    o.h[0] = tbl[v & 0xFFu]; o.h[1] = tbl[(v >> 8) & 0xFFu]; o.h[2] = tbl[(v >> 16) & 0xFFu]; o.h[3] = tbl[v >> 24];
+    o.scale = half_bits_to_float(ld16(b));
+    o.add = 0.f;
+    return o;
+  }
+};
+
+// Q6_K: the 16-column scale groups are half a K step wide, so a step is issued as two MFMAs (chunks 0-1, chunks 2-3);
+// get() returns the scale of the lane's own half and get_scales() both halves' scales of the lane's row.
+struct FragQ6K {
+  static constexpr bool BF16_MATH = false, HAS_ADD = false;
+  static constexpr int LDS_WORDS = 0;
+  __device__ static void fill_lds(uint32_t*, int, int) {}
+  __device__ static uint32_t col_of(uint32_t q, uint32_t p) { return 8u * q + p; }
+  __device__ static FragOut get(const uint8_t* row, uint32_t step, uint32_t q, const uint32_t*) {
+    const uint8_t* b = row + (step >> 3) * 210u;
+    const uint32_t e0 = 32u * (step & 7u) + 8u * q, h = e0 >> 7, k = (e0 & 127u) >> 5, l0 = e0 & 31u;
+    const u64_a2 ql = ld64(b + 64 * h + 32 * (k & 1u) + l0), qh = ld64(b + 128 + 32 * h + l0);
+    const uint32_t sh4 = 4u * (k >> 1), sh2 = 2u * k;
+    const uint32_t q0 = ((ql.x >> sh4) & 0x0F0F0F0Fu) | (((qh.x >> sh2) & 0x03030303u) << 4);
+    const uint32_t q1 = ((ql.y >> sh4) & 0x0F0F0F0Fu) | (((qh.y >> sh2) & 0x03030303u) << 4);
+    const uint32_t bias = 0xE420E420u;  // -1056 = -(1024 + 32) in both halves
+    FragOut o;
+    o.h[0] = pk_add_f16(bytes01_to_h2_1024(q0), bias); o.h[1] = pk_add_f16(bytes23_to_h2_1024(q0), bias);
+    o.h[2] = pk_add_f16(bytes01_to_h2_1024(q1), bias); o.h[3] = pk_add_f16(bytes23_to_h2_1024(q1), bias);
+    o.scale = 0.f;
+    o.add = 0.f;
+    return o;
+  }
+  __device__ static void get_scales(const uint8_t* row, uint32_t step, float& sa, float& sb) {
+    const uint8_t* b = row + (step >> 3) * 210u;
+    const uint32_t e0 = 32u * (step & 7u), h = e0 >> 7, k = (e0 & 127u) >> 5;
+    const uint32_t sc = ld16(b + 192 + 8 * h + 2 * k);
+    const float d = half_bits_to_float(ld16(b + 208));
+    sa = d * (float)(int)(int8_t)(sc & 0xFFu);
+    sb = d * (float)(int)(int8_t)(sc >> 8);
+  }
+};
+
+struct FragQ5K {
+  static constexpr bool BF16_MATH = false, HAS_ADD = true;
+  static constexpr int LDS_WORDS = 0;
+  __device__ static void fill_lds(uint32_t*, int, int) {}
+  __device__ static uint32_t col_of(uint32_t q, uint32_t p) { return 8u * q + p; }
+  __device__ static FragOut get(const uint8_t* row, uint32_t step, uint32_t q, const uint32_t*) {
+    const uint8_t* b = row + (step >> 3) * 176u;
+    const uint32_t is = step & 7u, g = is >> 1, run = is & 1u, l0 = 8u * q;
+    const u64_a2 ql = ld64(b + 48 + 32 * g + l0), qh = ld64(b + 16 + l0);
+    const uint32_t q0 = ((ql.x >> (4 * run)) & 0x0F0F0F0Fu) | (((qh.x >> is) & 0x01010101u) << 4);
+    const uint32_t q1 = ((ql.y >> (4 * run)) & 0x0F0F0F0Fu) | (((qh.y >> is) & 0x01010101u) << 4);
+    const uint32_t bias = 0xE400E400u;  // -1024 in both halves
+    const uint8_t* s = b + 4;
+    uint32_t sc, mn;
+    if (is < 4) { sc = ld8(s + is) & 63u; mn = ld8(s + is + 4) & 63u; }
+    else { sc = (ld8(s + is + 4) & 0xFu) | ((ld8(s + is - 4) >> 6) << 4); mn = (ld8(s + is + 4) >> 4) | ((ld8(s + is) >> 6) << 4); }
+    const uint32_t dd = ld32(b);
+    FragOut o;
+    o.h[0] = pk_add_f16(bytes01_to_h2_1024(q0), bias); o.h[1] = pk_add_f16(bytes23_to_h2_1024(q0), bias);
+    o.h[2] = pk_add_f16(bytes01_to_h2_1024(q1), bias); o.h[3] = pk_add_f16(bytes23_to_h2_1024(q1), bias);
+    o.scale = half_bits_to_float(dd & 0xFFFFu) * (float)sc;
+    o.add = -(half_bits_to_float(dd >> 16) * (float)mn);
+    return o;
+  }
+};
+
+template <int QT>  // MSQ_F16 or MSQ_BF16
+struct FragDense16 {
+  static constexpr bool BF16_MATH = QT == MSQ_BF16, HAS_ADD = false;
+  static constexpr int LDS_WORDS = 0;
+  __device__ static void fill_lds(uint32_t*, int, int) {}
+  __device__ static uint32_t col_of(uint32_t q, uint32_t p) { return 8u * q + p; }
+  __device__ static FragOut get(const uint8_t* row, uint32_t step, uint32_t q, const uint32_t*) {
+    const u128_a2 v = ld128(row + 64u * step + 16u * q);
+    FragOut o;
+    o.h[0] = v.x; o.h[1] = v.y; o.h[2] = v.z; o.h[3] = v.w;
+    o.scale = 1.f;
+    o.add = 0.f;
+    return o;
+  }
+};
+
+}  // namespace msq

@@ -118,6 +118,10 @@ def encode_matvec(e, t, W, rows, cols, x, y, accumulate=False, groups=1, cfg=Non
                                   C.byref(c) if c is not None else None))
 
 
+def encode_matvec_n(e, t, W, rows, cols, X, Y, n, accumulate=False, groups=1):  # reference: quant.hpp:32-35
+    _check(_lib.load().msq_matvec_n(e.handle, int(t), _bp(W), rows, cols, _bp(X), _bp(Y), n, int(bool(accumulate)), groups))
+
+
 def encode_dequant(e, t, W, n_elems, out):
     """Whole-buffer dequantization to fp32 (bit-exact with ref::dequant_row, tests/ref/dequant.cpp:34-120)."""
     _check(_lib.load().msq_dequant(e.handle, int(t), _bp(W), n_elems, _bp(out)))

@@ -1,0 +1,94 @@
+"""GPU parity of msq_matvec_n (n = 2..16 activation rows, one weight read) against the CPU oracle, through the C ABI.
+
+Mirrors the reference's tests/test_quant_matvec_n.mm: all types, block-diagonal groups, accumulate, and two references
+-- one with the activations rounded to fp16 (what the kernel stages; tight bound) and the pure F32 one (documented
+error of the fp16 staging) -- plus the BASELINE configs[4] shapes at N in {1, 2, 4, 8, 16}."""
+import numpy as np
+import pytest
+import torch
+
+import oracle as O
+from macseek_amd import quant as q
+from util import TOL_NORTH_STAR, place_in_arena, up
+
+pytestmark = pytest.mark.gpu
+
+CASES = [  # (type, rows, cols, groups, n, accumulate): tests/test_quant_matvec_n.mm:15-21
+    (O.Q6_K, 1280, 5120, 1, 2, False), (O.Q5_K, 1280, 5120, 1, 3, True), (O.Q8_0, 2304, 5120, 1, 5, False),
+    (O.IQ1_S, 2304, 5120, 1, 8, False), (O.IQ2_XXS, 5120, 2304, 1, 16, True), (O.IQ1_S, 5120, 2304, 1, 13, False),
+    (O.Q6_K, 8192, 4096, 8, 6, False), (O.BF16, 512, 5120, 1, 4, False), (O.F32, 24, 20480, 1, 5, False),
+    (O.F16, 300, 1280, 1, 16, False), (O.Q6_K, 32768, 1280, 1, 9, False),
+    (O.IQ4_NL, 1024, 4096, 1, 7, True), (O.Q5_K, 37, 256, 1, 2, False), (O.Q8_0, 16, 32, 1, 16, False),
+    (O.Q6_K, 24, 512, 3, 3, False),           # group size 8 rows: served as n decode matvecs
+    (O.Q8_0, 64, 16384, 1, 4, False),         # wider than one launch covers: K chunks accumulate
+]
+BASELINE5 = [(O.Q6_K, 1536, 7168), (O.Q5_K, 512, 7168), (O.IQ4_NL, 7168, 4096), (O.BF16, 384, 7168)]
+CASES += [(t, r, c, 1, n, False) for (t, r, c) in BASELINE5 for n in (1, 2, 4, 8, 16)]
+
+
+def half_round(x, t):
+    if t == O.BF16:  # bf16 weights: activations split into two bf16 terms (16 significant bits)
+        b = x.view(np.uint32).astype(np.uint64)
+        hi = (((b + 0x7FFF + ((b >> 16) & 1)) >> 16) << 16).astype(np.uint32).view(np.float32)
+        r = (x - hi).astype(np.float32)
+        b2 = r.view(np.uint32).astype(np.uint64)
+        lo = (((b2 + 0x7FFF + ((b2 >> 16) & 1)) >> 16) << 16).astype(np.uint32).view(np.float32)
+        return (hi.astype(np.float64) + lo.astype(np.float64)).astype(np.float32)  # exact: 16 bits fit a float
+    return x.astype(np.float16).astype(np.float32)
+
+
+@pytest.mark.parametrize("t,rows,cols,groups,n,acc", CASES, ids=lambda v: None)
+def test_matvec_n_vs_oracle(dev, t, rows, cols, groups, n, acc):
+    Wb = O.random_blocks(t, rows * cols, 21 + rows)
+    xs = cols * groups
+    X = O.randn(xs * n, 31 + n)
+    Y0 = O.randn(rows * n, 41)
+    arena, (W,) = place_in_arena([Wb])
+    Xd, Yd = up(X), up(Y0.copy())
+    e = q.Enc()
+    q.encode_matvec_n(e, t, W, rows, cols, q.Buffer.of(Xd), q.Buffer.of(Yd), n, acc, groups)
+    e.wait()
+    got = Yd.cpu().numpy().astype(np.float64).reshape(n, rows)
+    assert np.all(np.isfinite(got))
+    uses_mfma = n > 1 and t != O.F32 and not (groups > 1 and (rows // groups) % 16)
+    Xh = half_round(X, t) if uses_mfma else X
+    if not uses_mfma and t not in (O.F32, O.F16, O.BF16, O.Q8_0):
+        Xh = X.astype(np.float16).astype(np.float32)  # the decode (n = 1) path stages fp16 pairs for the block formats
+    err_h = err_f = err_ns = 0.0
+    for tok in range(n):
+        for hv, Xs in ((1, Xh), (0, X)):
+            ry, mag, wn2 = O.matvec(t, Wb, rows, cols, Xs[tok * xs:(tok + 1) * xs], groups)
+            y0 = Y0[tok * rows:(tok + 1) * rows].astype(np.float64)
+            if acc:
+                ry, mag = ry + y0, mag + np.abs(y0)
+            d = np.abs(got[tok] - ry)
+            ev = float(np.max(d / (mag + 1e-12)))
+            if hv:
+                err_h = max(err_h, ev)
+            else:
+                err_f = max(err_f, ev)
+                xn = np.repeat(np.sqrt((Xs[tok * xs:(tok + 1) * xs].astype(np.float64) ** 2).reshape(groups, cols).sum(1)), rows // groups)
+                err_ns = max(err_ns, float(np.max(d / (np.sqrt(wn2 + (y0 ** 2 if acc else 0)) * xn + 1e-30))))
+    print(f"  {O.TYPE_NAMES[t]:8s} [{cols:5d} -> {rows:5d}] g{groups} n={n:<2d} {'acc' if acc else '   '} "
+          f"err(x staged) {err_h:.2e}  err(vs F32) {err_f:.2e}  north-star {err_ns:.2e}")
+    # reference bounds: 2e-6 against the half-x reference for its F32-FMA kernel (n < 8), 1e-4 on its tile path,
+    # 2e-4 against the F32 reference (tests/test_quant_matvec_n.mm:45-46)
+    assert err_h <= 1e-5 and err_f <= 2e-4 and err_ns <= TOL_NORTH_STAR
+
+
+def test_matvec_n_misuse_and_untouched_rows(dev):
+    W = q.Buffer.of(torch.zeros(1 << 20, dtype=torch.uint8, device=dev))
+    v = q.Buffer.of(torch.zeros(1 << 16, dtype=torch.float32, device=dev))
+    e = q.Enc()
+    with pytest.raises(q.QuantError, match=r"macseek quant: matvec_n unsupported \(type Q6_K rows 16 cols 256\)"):
+        q.encode_matvec_n(e, q.QType.Q6_K, W, 16, 256, v, v, 17)
+    with pytest.raises(q.QuantError):
+        q.encode_matvec_n(e, q.QType.Q6_K, W, 16, 100, v, v, 2)
+    # rows beyond `rows` and tokens beyond n are never written
+    rows, cols, n = 21, 512, 3
+    Wb = O.random_blocks(O.IQ2_XXS, rows * cols, 1)
+    Wd, Xd = up(Wb), up(O.randn(cols * n, 2))
+    Y = torch.full((rows * 16 + 32,), 5.0, dtype=torch.float32, device=dev)
+    q.encode_matvec_n(e, q.QType.IQ2_XXS, q.Buffer.of(Wd), rows, cols, q.Buffer.of(Xd), q.Buffer.of(Y), n)
+    e.wait()
+    assert bool((Y[rows * n:] == 5.0).all()) and not bool((Y[:rows * n] == 5.0).any())
