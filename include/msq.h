@@ -156,6 +156,47 @@ int msq_moe_decode_table(void* stream, const MsqMoeDecodeArgs* a, const MsqBuffe
  * SHARED_DOWN never read `table` (it may be NULL for them). */
 int msq_moe_decode_table_part(void* stream, const MsqMoeDecodeArgs* a, const MsqBuffer* table, int part);
 
+/* ---------------------------------------------------------------------------------------------- MoE, prefill */
+
+/* reference: ms::q::MoePrefillArgs (quant.hpp:93-116), field for field, plus dim / inter / x_is_bf16.
+ * Routing is expert-sorted: routed expert j (0..n_exp-1, any subset of the layer's experts) owns entries
+ * [offs[j], offs[j+1]) of tok[] (token row in X) and wt[] (routing weight). slot_of[t * k_per_token + k] is the entry
+ * index of token t's k-th routed expert (-1 = none). Routed types: IQ1_S or IQ2_XXS; shared type: Q6_K, Q8_0, IQ2_XXS
+ * or IQ1_S. */
+typedef struct MsqMoePrefillArgs {
+  int t_gate_up, t_down;
+  int n_tokens;                 /* rows of X / Y */
+  int n_exp;                    /* routed experts with >= 1 token */
+  const MsqExpertSlot* slots;   /* host [n_exp] */
+  const int* offs;              /* host [n_exp + 1], offs[0] = 0, offs[n_exp] = total entries */
+  MsqBuffer tok;                /* device int32[total] */
+  MsqBuffer wt;                 /* device F32[total] */
+  MsqBuffer slot_of;            /* device int32[n_tokens * k_per_token] */
+  int k_per_token;
+  int has_shared;
+  int t_shared;
+  MsqExpertSlot shared;
+  MsqBuffer X;                  /* F32 (or BF16 when x_is_bf16) [n_tokens x dim] */
+  MsqBuffer Y;                  /* F32 [n_tokens x dim], ACCUMULATED */
+  MsqBuffer scratch;            /* >= msq_moe_prefill_scratch_bytes(total, n_tokens, n_exp, dim, inter) */
+  int path;                     /* reference kernel-family selector (quant.hpp:111-114): accepted, one family here */
+  int shared_dense;             /* reference shared-expert route selector (quant.hpp:115): accepted, one route here */
+  int dim, inter;               /* 0 = MSQ_EXPERT_DIM / MSQ_EXPERT_INTER; multiples of 256, at most 8192 */
+  int x_is_bf16;                /* activations are bf16 instead of the reference's F32 */
+} MsqMoePrefillArgs;
+
+/* reference: ms::q::moe_prefill_scratch_bytes (quant.hpp:117, quant.mm:427-431). Layout (caller-owned device memory):
+ * header (expert pointer table, offsets, token-tile table) | Xg fp16[(total+n) x dim] | H fp16[(total+n) x inter] |
+ * Z f32[(total+n) x dim]. The header is filled by an asynchronous copy on the stream, so unlike the reference the
+ * scratch may still be in use by earlier work on the same stream. */
+size_t msq_moe_prefill_scratch_bytes(int total_entries, int n_tokens, int n_exp, int dim, int inter);
+
+/* reference: ms::q::encode_moe_prefill (quant.hpp:118, quant.mm:433-612). Enqueues gather, grouped gate/up GEMM +
+ * SwiGLU, grouped down GEMM and the ordered reduction into Y. Activations and H are staged as fp16 (as in the
+ * reference), weights are used exactly. The result is bit-identical from run to run. n_tokens <= 0 returns MSQ_OK and
+ * does nothing (quant.mm:435). */
+int msq_moe_prefill(void* stream, const MsqMoePrefillArgs* a);
+
 #ifdef __cplusplus
 }
 #endif

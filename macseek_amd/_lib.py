@@ -60,6 +60,8 @@ SIGNATURES = {
     "msq_moe_decode": (C.c_int, [C.c_void_p, C.POINTER(MsqMoeDecodeArgs)]),
     "msq_moe_decode_table": (C.c_int, [C.c_void_p, C.POINTER(MsqMoeDecodeArgs), _BP]),
     "msq_moe_decode_table_part": (C.c_int, [C.c_void_p, C.POINTER(MsqMoeDecodeArgs), _BP, C.c_int]),
+    "msq_moe_prefill_scratch_bytes": (C.c_size_t, [C.c_int, C.c_int, C.c_int, C.c_int, C.c_int]),
+    "msq_moe_prefill": (C.c_int, [C.c_void_p, C.POINTER(MsqMoePrefillArgs)]),
 }
 
 

@@ -17,6 +17,8 @@ namespace msq {
 
 typedef __bf16 bf8_t __attribute__((ext_vector_type(8)));
 
+constexpr int kMvnMaxSteps = 16;  // K steps (of 32 columns) whose activations one wave keeps in registers
+
 __device__ __forceinline__ f4_t mfma_f16(const uint32_t a[4], const uint32_t b[4], f4_t c) {
   typedef uint32_t u4_t __attribute__((ext_vector_type(4)));
   const u4_t av = {a[0], a[1], a[2], a[3]}, bv = {b[0], b[1], b[2], b[3]};

@@ -11,8 +11,6 @@
 
 namespace msq {
 
-constexpr int kMvnMaxSteps = 16;  // K steps (of 32 columns) one wave can hold activations for
-
 struct MvnArgs {
   const uint8_t* W;
   const float* X;

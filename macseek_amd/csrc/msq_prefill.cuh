@@ -1,0 +1,227 @@
+// Prefill MoE: grouped GEMM over experts on the matrix cores (reference operator: ms::q::encode_moe_prefill,
+// src/kernels/quant.mm:433-612; reference kernels q_moe_gather / q_moe_rgu / q_moe_rdown / q_moe_reduce,
+// src/kernels/quant_moe_prefill.metal:22-29,190-239,275-303,330-344).
+//
+//   gather : Xg[i] = fp16(X[tok[i]]) for the expert-sorted entries, then Xg[total + t] = fp16(X[t]) (shared expert)
+//   gate/up: H[i][r] = fp16(silu(min(Xg_e[i].Wg[r], 10)) * clamp(Xg_e[i].Wu[r], -10, 10) * wt[i])
+//   down   : Z[i][c] = H_e[i] . Wd[c]   (fp32, one row per entry)
+//   reduce : Y[t] += Z[total + t] + sum_k Z[slot_of[t][k]]   in that fixed order
+//
+// GEMM work item = (token tile of up to 16 entries of one expert, chunk of weight-row tiles). A workgroup is up to 16
+// waves that split K; each wave keeps the token tile's activations of its K steps in registers as MFMA A fragments,
+// and the workgroup walks the 16-row weight tiles of its chunk. A tile's raw block bytes (16 contiguous rows) are
+// copied into LDS with fully coalesced 128-bit loads, one tile ahead through registers, and decoded from there into
+// B fragments; weights stay exact (fp16 payloads, fp32 scales applied to the MFMA result). The K-split partial tiles
+// meet in LDS and are added in wave order, so results do not depend on scheduling.
+#pragma once
+#include "msq_mfma.cuh"
+
+namespace msq {
+
+struct PfArgs {
+  const uint16_t* A;        // activations fp16 [(total + n) x K]: Xg (gate/up) or H (down)
+  uint16_t* H;              // gate/up output fp16 [(total + n) x inter]
+  float* Z;                 // down output fp32 [(total + n) x dim]
+  const float* wt;          // routing weight per entry [total]
+  const uint64_t* ptrs;     // (n_exp + 1) x {gate, up, down} device addresses (the shared expert is entry n_exp)
+  const uint32_t* offs;     // n_exp + 2 entry offsets
+  const uint32_t* tiles;    // token tiles: pairs {expert index, first entry of the tile inside the expert}
+  uint32_t ntiles;          // token tiles this launch covers
+  uint32_t total;           // routed entries: entries at or beyond use weight 1 (shared expert)
+  uint32_t K, N;            // gate/up: K = dim, N = inter; down: K = inter, N = dim
+  uint32_t row_bytes;
+  uint32_t nsteps, steps_per_wave;
+  uint32_t chunk_tiles;     // weight-row tiles per work item
+  uint32_t nchunks;         // ceil(N / 16 / chunk_tiles)
+  uint32_t staged;          // 1: weight tiles go through LDS staging
+};
+
+constexpr int kPfStageGranules = 3;  // 16-byte granules per thread per matrix the staging path can hold (48 KiB / 1024 threads)
+
+template <class F, bool GU>
+__global__ __launch_bounds__(1024) void moe_pf_gemm_kernel(const PfArgs a) {
+  constexpr int NM = GU ? 2 : 1;
+  extern __shared__ __attribute__((aligned(16))) uint32_t smem[];
+  uint32_t* tbl = smem;
+  float* red = (float*)(smem + F::LDS_WORDS);  // [NM][wave][token][17]
+  const uint32_t tid = threadIdx.x, lane = tid & 63u, nthreads = blockDim.x;
+  const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6)), nwaves = nthreads >> 6;
+  uint8_t* stage = (uint8_t*)(red + NM * nwaves * 16 * 17);  // [NM][tile window]
+  const uint32_t m16 = lane & 15u, q = lane >> 4;
+  const uint32_t S = a.steps_per_wave, s0 = wave * S;
+  const uint32_t tile_bytes = 16u * a.row_bytes;
+  const uint32_t window = (tile_bytes + 15u + 15u) & ~15u;  // staged window per matrix, rounded to granules
+
+  F::fill_lds(tbl, (int)tid, (int)nthreads);
+
+  const uint32_t item = blockIdx.x;
+  const uint32_t mt = item / a.nchunks, rc = item - mt * a.nchunks;
+  const uint32_t e = a.tiles[2 * mt], t0 = a.tiles[2 * mt + 1];
+  const uint32_t base = a.offs[e] + t0;                       // first entry (row of A / H / Z) of the token tile
+  const uint32_t mtok = min(16u, a.offs[e + 1] - base);
+  const uint8_t* W[NM];
+  if (GU) { W[0] = (const uint8_t*)a.ptrs[3 * e]; W[NM - 1] = (const uint8_t*)a.ptrs[3 * e + 1]; }
+  else W[0] = (const uint8_t*)a.ptrs[3 * e + 2];
+
+  // A fragments of this wave's K steps: token m16 of the tile, chunk q
+  uint32_t xa[kMvnMaxSteps][4];
+#pragma unroll
+  for (int i = 0; i < kMvnMaxSteps; i++) {
+    const uint32_t step = s0 + i;
+    uint4 v = {0u, 0u, 0u, 0u};
+    if ((uint32_t)i < S && step < a.nsteps && m16 < mtok) {
+      const uint16_t* xs = a.A + (size_t)(base + m16) * a.K + 32u * step;
+      v = *(const uint4*)(xs + 8u * q);  // every format used here keeps the natural column order (col_of = 8 q + p)
+    }
+    xa[i][0] = v.x; xa[i][1] = v.y; xa[i][2] = v.z; xa[i][3] = v.w;
+  }
+
+  const uint32_t ntile_rows = (a.N + 15u) / 16u;
+  const uint32_t tile_first = rc * a.chunk_tiles, tile_last = min(ntile_rows, tile_first + a.chunk_tiles);
+  // staging: thread i owns granules i, i + nthreads, ... of each matrix' aligned window
+  uint4 pf[NM][kPfStageGranules];
+  auto issue = [&](uint32_t tile) {
+#pragma unroll
+    for (int m = 0; m < NM; m++) {
+      const uint8_t* start = W[m] + (size_t)tile * tile_bytes;
+      const uint32_t shift = (uint32_t)((uintptr_t)start & 15u);
+      // the last tile of a matrix may be short: never read beyond the last row's granule
+      const uint32_t rows_here = min(16u, a.N - tile * 16u);
+      const uint32_t valid = shift + rows_here * a.row_bytes;
+#pragma unroll
+      for (int g = 0; g < kPfStageGranules; g++) {
+        const uint32_t gi = tid + g * nthreads;
+        uint4 v = {0u, 0u, 0u, 0u};
+        if (16u * gi < valid) v = *(const uint4*)(start - shift + 16u * gi);
+        pf[m][g] = v;
+      }
+    }
+  };
+  if (a.staged && tile_first < tile_last) issue(tile_first);
+  __syncthreads();  // tables ready
+
+  const uint32_t ones[4] = {0x3C003C00u, 0x3C003C00u, 0x3C003C00u, 0x3C003C00u};
+  for (uint32_t tile = tile_first; tile < tile_last; tile++) {
+    const uint8_t* wr[NM];
+    if (a.staged) {
+#pragma unroll
+      for (int m = 0; m < NM; m++) {
+#pragma unroll
+        for (int g = 0; g < kPfStageGranules; g++) {
+          const uint32_t gi = tid + g * nthreads;
+          if (16u * gi < window) ((uint4*)(stage + (size_t)m * window))[gi] = pf[m][g];
+        }
+        const uint32_t shift = (uint32_t)((uintptr_t)(W[m] + (size_t)tile * tile_bytes) & 15u);
+        wr[m] = stage + (size_t)m * window + shift + m16 * a.row_bytes;
+      }
+      if (tile + 1 < tile_last) issue(tile + 1);  // next tile's bytes travel while this one is decoded
+      __syncthreads();
+    } else {
+      const uint32_t row = min(tile * 16u + m16, a.N - 1);
+#pragma unroll
+      for (int m = 0; m < NM; m++) wr[m] = W[m] + (size_t)row * a.row_bytes;
+    }
+    f4_t acc[NM];
+#pragma unroll
+    for (int m = 0; m < NM; m++) acc[m] = f4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int i = 0; i < kMvnMaxSteps; i++) {
+      const uint32_t step = s0 + i;
+      if ((uint32_t)i < S && step < a.nsteps) {  // wave-uniform
+        const f4_t zero = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int m = 0; m < NM; m++) {
+          const FragOut f = F::get(wr[m], step, q, tbl);
+          if constexpr (requires(float& s) { F::get_scales(wr[m], step, s, s); }) {
+            float sa, sb;
+            F::get_scales(wr[m], step, sa, sb);
+            uint32_t ha[4], hb[4];
+#pragma unroll
+            for (int p = 0; p < 4; p++) { ha[p] = q < 2 ? f.h[p] : 0u; hb[p] = q < 2 ? 0u : f.h[p]; }
+            acc[m] += sa * mfma_f16(xa[i], ha, zero) + sb * mfma_f16(xa[i], hb, zero);
+          } else {
+            acc[m] += f.scale * mfma_f16(xa[i], f.h, zero);
+            if constexpr (F::HAS_ADD) acc[m] += f.add * mfma_f16(xa[i], ones, zero);
+          }
+        }
+      }
+    }
+#pragma unroll
+    for (int m = 0; m < NM; m++)
+#pragma unroll
+      for (int i = 0; i < 4; i++) red[((m * nwaves + wave) * 16u + 4u * q + i) * 17u + m16] = acc[m][i];
+    __syncthreads();
+    for (uint32_t idx = tid; idx < 16u * mtok; idx += nthreads) {
+      const uint32_t t = idx >> 4, r = idx & 15u, orow = tile * 16u + r;
+      if (orow < a.N) {
+        float s[NM];
+#pragma unroll
+        for (int m = 0; m < NM; m++) {
+          s[m] = 0.f;
+          for (uint32_t w = 0; w < nwaves; w++) s[m] += red[((m * nwaves + w) * 16u + t) * 17u + r];
+        }
+        const uint32_t entry = base + t;
+        if constexpr (GU) {
+          float g = fminf(s[0], 10.f), u = fminf(fmaxf(s[NM - 1], -10.f), 10.f);
+          const float w = entry < a.total ? a.wt[entry] : 1.f;
+          const float h = g / (1.f + expf(-g)) * u * w;
+          a.H[(size_t)entry * a.N + orow] = __builtin_bit_cast(uint16_t, (_Float16)h);
+        } else {
+          a.Z[(size_t)entry * a.N + orow] = s[0];
+        }
+      }
+    }
+    __syncthreads();
+  }
+}
+
+// Xg[i] = fp16(X[src(i)]): i < total gathers token tok[i]; rows total .. total + n - 1 are the tokens themselves
+template <bool X_BF16>
+__global__ __launch_bounds__(256) void moe_pf_gather_kernel(const void* __restrict__ X, uint16_t* __restrict__ Xg,
+                                                            const int* __restrict__ tok, uint32_t total, uint32_t nrows,
+                                                            uint32_t dim) {
+  const uint32_t i = blockIdx.y;
+  if (i >= nrows) return;
+  const uint32_t src = i < total ? (uint32_t)tok[i] : i - total;
+  for (uint32_t c4 = blockIdx.x * blockDim.x + threadIdx.x; c4 < dim / 4; c4 += gridDim.x * blockDim.x) {
+    float4 v;
+    if constexpr (X_BF16) {
+      const uint2 b = ((const uint2*)((const uint16_t*)X + (size_t)src * dim))[c4];
+      v = make_float4(__builtin_bit_cast(float, b.x << 16), __builtin_bit_cast(float, b.x & 0xFFFF0000u),
+                      __builtin_bit_cast(float, b.y << 16), __builtin_bit_cast(float, b.y & 0xFFFF0000u));
+    } else {
+      v = ((const float4*)((const float*)X + (size_t)src * dim))[c4];
+    }
+    uint2 o;
+    o.x = pack_h2(v.x, v.y);
+    o.y = pack_h2(v.z, v.w);
+    ((uint2*)(Xg + (size_t)i * dim))[c4] = o;
+  }
+}
+
+// Y[t] += Z[total + t] (shared) + sum_k Z[slot_of[t][k]] in fixed k order; tokens without any entry are left alone
+__global__ __launch_bounds__(256) void moe_pf_reduce_kernel(const float* __restrict__ Z, float* __restrict__ Y,
+                                                            const int* __restrict__ slot_of, uint32_t n, uint32_t total,
+                                                            uint32_t dim, uint32_t k_per_token, uint32_t has_shared) {
+  const uint32_t t = blockIdx.y;
+  if (t >= n) return;
+  for (uint32_t c4 = blockIdx.x * blockDim.x + threadIdx.x; c4 < dim / 4; c4 += gridDim.x * blockDim.x) {
+    float4 s = has_shared ? ((const float4*)(Z + (size_t)(total + t) * dim))[c4] : make_float4(0.f, 0.f, 0.f, 0.f);
+    bool any = has_shared != 0;
+    for (uint32_t k = 0; k < k_per_token; k++) {
+      const int i = slot_of[t * k_per_token + k];
+      if (i >= 0) {
+        const float4 z = ((const float4*)(Z + (size_t)i * dim))[c4];
+        s.x += z.x; s.y += z.y; s.z += z.z; s.w += z.w;
+        any = true;
+      }
+    }
+    if (!any) continue;
+    float4* y = (float4*)(Y + (size_t)t * dim) + c4;
+    float4 o = *y;
+    o.x += s.x; o.y += s.y; o.z += s.z; o.w += s.w;
+    *y = o;
+  }
+}
+
+}  // namespace msq

@@ -1,0 +1,178 @@
+// C ABI: prefill MoE (see include/msq.h; reference host code src/kernels/quant.mm:372-612).
+#include <algorithm>
+#include <vector>
+
+#include "msq_host.h"
+#include "msq_prefill.cuh"
+
+namespace msq {
+namespace {
+
+size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
+size_t header_bytes(int total, int n, int n_exp) {
+  const size_t tiles = (size_t)n_exp + total / 16 + n / 16 + 4;  // token tiles of up to 16 entries
+  return align256(24 * (size_t)(n_exp + 1) + 4 * (size_t)(n_exp + 2) + 8 * tiles);
+}
+bool routed_ok(int t) { return t == MSQ_IQ1_S || t == MSQ_IQ2_XXS; }
+bool shared_ok(int t) { return t == MSQ_Q6_K || t == MSQ_Q8_0 || t == MSQ_IQ2_XXS || t == MSQ_IQ1_S; }
+
+template <class F, bool GU>
+int launch_gemm_t(hipStream_t st, PfArgs a, int cus) {
+  const uint32_t waves = (a.nsteps + a.steps_per_wave - 1) / a.steps_per_wave;
+  const uint32_t threads = 64 * waves;
+  constexpr int NM = GU ? 2 : 1;
+  const size_t window = ((size_t)16 * a.row_bytes + 30) & ~(size_t)15;
+  const size_t base_lds = (size_t)F::LDS_WORDS * 4 + (size_t)NM * waves * 16 * 17 * 4;
+  a.staged = (window <= (size_t)threads * kPfStageGranules * 16 && base_lds + NM * window <= 150 * 1024) ? 1u : 0u;
+  const size_t lds = base_lds + (a.staged ? NM * window : 0);
+  const uint32_t ntile_rows = (a.N + 15) / 16;
+  // enough work items to fill the chip a few times, at least 8 weight tiles per item to amortise the A fragments
+  uint32_t nchunks = std::max<uint32_t>(1, std::min<uint32_t>((4u * (uint32_t)cus + a.ntiles - 1) / a.ntiles, (ntile_rows + 7) / 8));
+  a.chunk_tiles = (ntile_rows + nchunks - 1) / nchunks;
+  a.nchunks = (ntile_rows + a.chunk_tiles - 1) / a.chunk_tiles;
+  static bool attr_set = false;  // per instantiation: allow more than 64 KiB of dynamic LDS
+  if (!attr_set) {
+    MSQ_HIP(hipFuncSetAttribute((const void*)moe_pf_gemm_kernel<F, GU>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+    attr_set = true;
+  }
+  hipLaunchKernelGGL((moe_pf_gemm_kernel<F, GU>), dim3(a.ntiles * a.nchunks), dim3(threads), lds, st, a);
+  MSQ_HIP(hipGetLastError());
+  return MSQ_OK;
+}
+template <bool GU>
+int launch_gemm(int t, hipStream_t st, const PfArgs& a, int cus) {
+  switch (t) {
+    case MSQ_IQ1_S: return launch_gemm_t<FragIQ1S, GU>(st, a, cus);
+    case MSQ_IQ2_XXS: return launch_gemm_t<FragIQ2XXS, GU>(st, a, cus);
+    case MSQ_Q6_K: return launch_gemm_t<FragQ6K, GU>(st, a, cus);
+    case MSQ_Q8_0: return launch_gemm_t<FragQ8_0, GU>(st, a, cus);
+  }
+  return unsupported("moe_prefill types", t, 0, 0);
+}
+
+}  // namespace
+}  // namespace msq
+
+using namespace msq;
+
+extern "C" {
+
+size_t msq_moe_prefill_scratch_bytes(int total, int n, int n_exp, int dim, int inter) {
+  if (dim <= 0) dim = MSQ_EXPERT_DIM;
+  if (inter <= 0) inter = MSQ_EXPERT_INTER;
+  const size_t rows = (size_t)std::max(total, 0) + (size_t)std::max(n, 0);
+  return header_bytes(std::max(total, 0), std::max(n, 0), std::max(n_exp, 0)) + align256(rows * dim * 2) +
+         align256(rows * inter * 2) + align256(rows * dim * 4);
+}
+
+int msq_moe_prefill(void* stream, const MsqMoePrefillArgs* p) {
+  if (!p) return fail(MSQ_ERR_ARGUMENT, "macseek quant: moe_prefill: null arguments");
+  const int n = p->n_tokens, ne = p->n_exp;
+  if (n <= 0) return MSQ_OK;
+  const int dim = p->dim ? p->dim : MSQ_EXPERT_DIM, inter = p->inter ? p->inter : MSQ_EXPERT_INTER;
+  if (ne < 0 || (ne > 0 && (!p->slots || !p->offs))) return fail(MSQ_ERR_ARGUMENT, "macseek quant: moe_prefill: slots / offs missing");
+  const int total = ne > 0 ? p->offs[ne] : 0;
+  if (!routed_ok(p->t_gate_up) || !routed_ok(p->t_down) || (p->has_shared && !shared_ok(p->t_shared)))
+    return unsupported("moe_prefill types", p->t_gate_up, 0, 0);
+  if (dim < 256 || inter < 256 || dim % 256 || inter % 256 || dim > 8192 || inter > 8192)
+    return unsupported("moe_prefill expert shape", p->t_gate_up, inter, dim);
+  if (total < 0 || p->k_per_token < 0) return fail(MSQ_ERR_ARGUMENT, "macseek quant: moe_prefill: negative counts");
+  for (int j = 0; j < ne; j++)
+    if (p->offs[j + 1] < p->offs[j] || p->offs[0] != 0) return fail(MSQ_ERR_ARGUMENT, "macseek quant: moe_prefill: offs not ascending from 0");
+  if (!buf_ok(&p->scratch, msq_moe_prefill_scratch_bytes(total, n, ne, dim, inter)))
+    return fail(MSQ_ERR_SCRATCH, "macseek quant: moe_prefill scratch too small unsupported (type %s rows %d cols %d)",
+                msq_type_name_of(p->t_gate_up), total, n);
+  const size_t xbytes = (size_t)n * dim * (p->x_is_bf16 ? 2 : 4);
+  if (!buf_ok(&p->X, xbytes) || !buf_ok(&p->Y, (size_t)n * dim * 4))
+    return fail(MSQ_ERR_ARGUMENT, "macseek quant: moe_prefill: X / Y missing or too small");
+  if (total > 0 && (!buf_ok(&p->tok, (size_t)total * 4) || !buf_ok(&p->wt, (size_t)total * 4)))
+    return fail(MSQ_ERR_ARGUMENT, "macseek quant: moe_prefill: tok / wt missing or too small");
+  if (p->k_per_token > 0 && !buf_ok(&p->slot_of, (size_t)n * p->k_per_token * 4))
+    return fail(MSQ_ERR_ARGUMENT, "macseek quant: moe_prefill: slot_of missing or too small");
+  const size_t rb_gu = msq_type_row_bytes(p->t_gate_up, dim), rb_d = msq_type_row_bytes(p->t_down, inter);
+  const size_t rb_sgu = msq_type_row_bytes(p->t_shared, dim), rb_sd = msq_type_row_bytes(p->t_shared, inter);
+  for (int j = 0; j < ne; j++) {
+    const MsqExpertSlot& s = p->slots[j];
+    if (!buf_ok(&s.gate, rb_gu * inter) || !buf_ok(&s.up, rb_gu * inter) || !buf_ok(&s.down, rb_d * dim))
+      return fail(MSQ_ERR_ARGUMENT, "macseek quant: moe_prefill: expert slot %d missing or too small", j);
+  }
+  if (p->has_shared && (!buf_ok(&p->shared.gate, rb_sgu * inter) || !buf_ok(&p->shared.up, rb_sgu * inter) ||
+                        !buf_ok(&p->shared.down, rb_sd * dim)))
+    return fail(MSQ_ERR_ARGUMENT, "macseek quant: moe_prefill: shared expert missing or too small");
+
+  hipStream_t st = (hipStream_t)stream;
+  const int cus = device_info().cus;
+  // ---- header: expert pointer table, offsets, token-tile tables (routed tiles first, then the shared expert's)
+  const size_t hbytes = header_bytes(total, n, ne);
+  std::vector<uint8_t> hdr(hbytes, 0);
+  uint64_t* ptrs = (uint64_t*)hdr.data();
+  uint32_t* offs = (uint32_t*)(hdr.data() + 24 * (size_t)(ne + 1));
+  uint32_t* tiles = offs + (ne + 2);
+  for (int j = 0; j < ne; j++) {
+    ptrs[3 * j] = (uint64_t)(uintptr_t)bptr(&p->slots[j].gate);
+    ptrs[3 * j + 1] = (uint64_t)(uintptr_t)bptr(&p->slots[j].up);
+    ptrs[3 * j + 2] = (uint64_t)(uintptr_t)bptr(&p->slots[j].down);
+    offs[j] = (uint32_t)p->offs[j];
+  }
+  offs[ne] = (uint32_t)total;
+  offs[ne + 1] = (uint32_t)(total + n);
+  if (p->has_shared) {
+    ptrs[3 * ne] = (uint64_t)(uintptr_t)bptr(&p->shared.gate);
+    ptrs[3 * ne + 1] = (uint64_t)(uintptr_t)bptr(&p->shared.up);
+    ptrs[3 * ne + 2] = (uint64_t)(uintptr_t)bptr(&p->shared.down);
+  }
+  uint32_t nt_routed = 0, nt_shared = 0;
+  for (int j = 0; j < ne; j++)
+    for (int t0 = 0; t0 < p->offs[j + 1] - p->offs[j]; t0 += 16) { tiles[2 * nt_routed] = (uint32_t)j; tiles[2 * nt_routed + 1] = (uint32_t)t0; nt_routed++; }
+  if (p->has_shared)
+    for (int t0 = 0; t0 < n; t0 += 16) { tiles[2 * (nt_routed + nt_shared)] = (uint32_t)ne; tiles[2 * (nt_routed + nt_shared) + 1] = (uint32_t)t0; nt_shared++; }
+  uint8_t* sc = bptr_mut(&p->scratch);
+  // pageable source: the copy is staged by the runtime before this call returns, and ordered on the stream
+  MSQ_HIP(hipMemcpyAsync(sc, hdr.data(), 24 * (size_t)(ne + 1) + 4 * (size_t)(ne + 2) + 8 * (size_t)(nt_routed + nt_shared),
+                         hipMemcpyHostToDevice, st));
+  const size_t rows = (size_t)total + n;
+  uint16_t* Xg = (uint16_t*)(sc + hbytes);
+  uint16_t* H = (uint16_t*)((uint8_t*)Xg + align256(rows * dim * 2));
+  float* Z = (float*)((uint8_t*)H + align256(rows * inter * 2));
+  const uint64_t* d_ptrs = (const uint64_t*)sc;
+  const uint32_t* d_offs = (const uint32_t*)(sc + 24 * (size_t)(ne + 1));
+  const uint32_t* d_tiles = d_offs + (ne + 2);
+
+  // 1) gather + convert
+  const uint32_t grows = (uint32_t)(total + (p->has_shared ? n : 0));
+  if (grows > 0) {
+    const dim3 grid((dim / 4 + 255) / 256, grows), block(256);
+    const int* tok = total > 0 ? (const int*)bptr(&p->tok) : nullptr;
+    if (p->x_is_bf16) hipLaunchKernelGGL((moe_pf_gather_kernel<true>), grid, block, 0, st, (const void*)bptr(&p->X), Xg, tok, (uint32_t)total, grows, (uint32_t)dim);
+    else hipLaunchKernelGGL((moe_pf_gather_kernel<false>), grid, block, 0, st, (const void*)bptr(&p->X), Xg, tok, (uint32_t)total, grows, (uint32_t)dim);
+    MSQ_HIP(hipGetLastError());
+  }
+  PfArgs a{};
+  a.H = H; a.Z = Z; a.wt = total > 0 ? (const float*)bptr(&p->wt) : nullptr;
+  a.ptrs = d_ptrs; a.offs = d_offs; a.total = (uint32_t)total;
+  auto steps = [&](uint32_t K) {
+    a.K = K; a.nsteps = K / 32;
+    const uint32_t ks = std::min<uint32_t>(16u, a.nsteps);
+    a.steps_per_wave = (a.nsteps + ks - 1) / ks;
+  };
+  int rc;
+  // 2) gate + up + SwiGLU -> H
+  a.A = Xg; a.N = (uint32_t)inter; steps((uint32_t)dim);
+  if (nt_routed) { a.tiles = d_tiles; a.ntiles = nt_routed; a.row_bytes = (uint32_t)rb_gu; if ((rc = launch_gemm<true>(p->t_gate_up, st, a, cus))) return rc; }
+  if (nt_shared) { a.tiles = d_tiles + 2 * nt_routed; a.ntiles = nt_shared; a.row_bytes = (uint32_t)rb_sgu; if ((rc = launch_gemm<true>(p->t_shared, st, a, cus))) return rc; }
+  // 3) down -> Z
+  a.A = H; a.N = (uint32_t)dim; steps((uint32_t)inter);
+  if (nt_routed) { a.tiles = d_tiles; a.ntiles = nt_routed; a.row_bytes = (uint32_t)rb_d; if ((rc = launch_gemm<false>(p->t_down, st, a, cus))) return rc; }
+  if (nt_shared) { a.tiles = d_tiles + 2 * nt_routed; a.ntiles = nt_shared; a.row_bytes = (uint32_t)rb_sd; if ((rc = launch_gemm<false>(p->t_shared, st, a, cus))) return rc; }
+  // 4) ordered reduction into Y
+  if (nt_routed || nt_shared) {
+    const dim3 grid((dim / 4 + 255) / 256, (unsigned)n), block(256);
+    hipLaunchKernelGGL(moe_pf_reduce_kernel, grid, block, 0, st, (const float*)Z, (float*)bptr_mut(&p->Y),
+                       p->k_per_token > 0 ? (const int*)bptr(&p->slot_of) : nullptr, (uint32_t)n, (uint32_t)total, (uint32_t)dim,
+                       (uint32_t)(nt_routed ? p->k_per_token : 0), (uint32_t)(p->has_shared ? 1 : 0));
+    MSQ_HIP(hipGetLastError());
+  }
+  return MSQ_OK;
+}
+
+}  // extern "C"

@@ -8,7 +8,7 @@ import ctypes as C
 import enum
 
 from . import _lib
-from ._lib import MsqBuffer, MsqExpertSlot, MsqMoeDecodeArgs, MsqMvCfg
+from ._lib import MsqBuffer, MsqExpertSlot, MsqMoeDecodeArgs, MsqMoePrefillArgs, MsqMvCfg
 
 
 class QType(enum.IntEnum):  # reference: src/kernels/quant_types.hpp:9-11 (ggml type ids)
@@ -195,3 +195,51 @@ def encode_moe_decode_table(e, a, table):  # reference: quant.hpp:76-78
 
 def encode_moe_decode_table_part(e, a, table, part):  # reference: quant.hpp:79-86
     _check(_lib.load().msq_moe_decode_table_part(e.handle, C.byref(a.c()), _bp(table), int(part)))
+
+
+# ---------------------------------------------------------------------------------------------- MoE, prefill
+class MoePrefillArgs:
+    """reference: ms::q::MoePrefillArgs (quant.hpp:93-116) plus dim / inter / x_is_bf16. `slots` is a list of
+    ExpertSlot (host), `offs` a list of n_exp + 1 ints (host); tok / wt / slot_of / X / Y / scratch are device Buffers."""
+
+    def __init__(self):
+        self.t_gate_up = QType.IQ1_S
+        self.t_down = QType.IQ1_S
+        self.n_tokens = 0
+        self.n_exp = 0
+        self.slots = []
+        self.offs = [0]
+        self.tok = Buffer()
+        self.wt = Buffer()
+        self.slot_of = Buffer()
+        self.k_per_token = 6
+        self.has_shared = True
+        self.t_shared = QType.Q6_K
+        self.shared = ExpertSlot()
+        self.X = Buffer()
+        self.Y = Buffer()
+        self.scratch = Buffer()
+        self.path = -1
+        self.shared_dense = -1
+        self.dim, self.inter = kExpertDim, kExpertInter
+        self.x_is_bf16 = False
+
+    def c(self):
+        a = MsqMoePrefillArgs()
+        a.t_gate_up, a.t_down, a.n_tokens, a.n_exp = int(self.t_gate_up), int(self.t_down), self.n_tokens, self.n_exp
+        self._slots = (MsqExpertSlot * max(1, self.n_exp))(*[s.c() for s in self.slots[:self.n_exp]])
+        self._offs = (C.c_int * (self.n_exp + 1))(*self.offs[:self.n_exp + 1])
+        a.slots, a.offs = self._slots, self._offs
+        a.tok, a.wt, a.slot_of = self.tok.c(), self.wt.c(), self.slot_of.c()
+        a.k_per_token, a.has_shared, a.t_shared, a.shared = self.k_per_token, int(bool(self.has_shared)), int(self.t_shared), self.shared.c()
+        a.X, a.Y, a.scratch = self.X.c(), self.Y.c(), self.scratch.c()
+        a.path, a.shared_dense, a.dim, a.inter, a.x_is_bf16 = self.path, self.shared_dense, self.dim, self.inter, int(bool(self.x_is_bf16))
+        return a
+
+
+def moe_prefill_scratch_bytes(total_entries, n_tokens, n_exp=384, dim=kExpertDim, inter=kExpertInter):  # reference: quant.hpp:117
+    return _lib.load().msq_moe_prefill_scratch_bytes(total_entries, n_tokens, n_exp, dim, inter)
+
+
+def encode_moe_prefill(e, a):  # reference: quant.hpp:118
+    _check(_lib.load().msq_moe_prefill(e.handle, C.byref(a.c())))
