@@ -241,13 +241,124 @@ def bench_matvec(torch, args, t, rows, cols, d_sigma, label):
     }
 
 
+# ------------------------------------------------------------------------------------------------ prefill grouped GEMM
+MFMA_PEAK_TFLOPS = 2500.0  # MI355X dense fp16 / bf16 matrix-core peak
+
+
+def zipf_routing(n, n_exp, k, s, seed):
+    """top-k distinct experts per token, popularity ~ rank^-s over a seeded expert permutation (bench/qmatmul.mm:135-152)."""
+    rng = np.random.default_rng(seed)
+    pw = np.zeros(n_exp)
+    pw[rng.permutation(n_exp)] = 1.0 / np.arange(1, n_exp + 1) ** s
+    # Gumbel top-k = sampling without replacement proportional to pw
+    g = np.log(pw)[None, :] + rng.gumbel(size=(n, n_exp))
+    ids = np.argsort(-g, axis=1)[:, :k]
+    w = rng.random((n, k)).astype(np.float32) + 0.1
+    w = w / w.sum(1, keepdims=True)  # renormalised routing weights
+    return ids, w
+
+
+def bench_moe_prefill(torch, steps, warmup, with_cpu=True):
+    from macseek_amd import _lib
+    from macseek_amd import quant as q
+    import oracle as O
+    dev = torch.device("cuda:0")
+    L = _lib.load()
+    N, DIM, INTER, NE, TOPK = 2048, 7168, 2048, 384, 6
+    t = q.QType.IQ2_XXS
+    gu_b, dn_b = q.row_bytes(t, DIM) * INTER, q.row_bytes(t, INTER) * DIM
+    per_exp = 2 * gu_b + dn_b
+    arena = gen_blocks(torch, t, NE * per_exp // 66, 0.01, 7, dev)
+    ids, w = zipf_routing(N, NE, TOPK, 1.1, 4321)
+    counts = np.bincount(ids.ravel(), minlength=NE)
+    used = np.nonzero(counts)[0]
+    order = np.lexsort((np.repeat(np.arange(N), TOPK), ids.ravel()))  # expert-sorted, token order inside an expert
+    tok = (order // TOPK).astype(np.int32)
+    wt = w.ravel()[order].astype(np.float32)
+    slot_of = np.empty(N * TOPK, dtype=np.int32)
+    slot_of[order] = np.arange(N * TOPK, dtype=np.int32)
+    offs = np.concatenate([[0], np.cumsum(counts[used])]).astype(np.int32)
+    total = int(offs[-1])
+    A = q.Buffer.of(arena)
+    a = q.MoePrefillArgs()
+    a.t_gate_up = a.t_down = t
+    a.has_shared = False
+    a.n_tokens, a.n_exp, a.k_per_token, a.dim, a.inter, a.x_is_bf16 = N, len(used), TOPK, DIM, INTER, True
+    a.slots = [q.ExpertSlot(A.sub(int(e) * per_exp, gu_b), A.sub(int(e) * per_exp + gu_b, gu_b), A.sub(int(e) * per_exp + 2 * gu_b, dn_b)) for e in used]
+    a.offs = [int(v) for v in offs]
+    X = torch.randn(N, DIM, device=dev).to(torch.bfloat16)
+    Y = torch.zeros(N, DIM, device=dev)
+    tok_d, wt_d, slot_d = torch.from_numpy(tok).to(dev), torch.from_numpy(wt).to(dev), torch.from_numpy(slot_of).to(dev)
+    scratch = torch.empty(q.moe_prefill_scratch_bytes(total, N, len(used), DIM, INTER), dtype=torch.uint8, device=dev)
+    a.tok, a.wt, a.slot_of, a.X, a.Y, a.scratch = (q.Buffer.of(v) for v in (tok_d, wt_d, slot_d, X, Y, scratch))
+    ca = a.c()
+
+    def call():
+        rc = L.msq_moe_prefill(C.c_void_p(torch.cuda.current_stream().cuda_stream), C.byref(ca))
+        if rc != 0:
+            raise RuntimeError(L.msq_last_error().decode())
+
+    for _ in range(max(1, warmup)):
+        call()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        call()
+    torch.cuda.synchronize()
+    ms_step = (time.perf_counter() - t0) * 1e3 / steps
+    flops = 2.0 * 3 * DIM * INTER * total
+    value = flops / (ms_step * 1e-3) / 1e12
+    # dominant kernel: the routed gate/up GEMM (two thirds of the FLOPs), timed alone through the phase skip mask
+    os.environ["MSQ_MOEP_SKIP"] = str(1 | 4 | 8 | 16 | 32)
+    gu_mean, gu_med, gu_min = event_ms_per_launch(torch, lambda i: call(), max(3, min(steps, 10)))
+    os.environ["MSQ_MOEP_SKIP"] = str(1 | 2 | 4 | 16 | 32)
+    dn_mean, _, _ = event_ms_per_launch(torch, lambda i: call(), max(3, min(steps, 10)))
+    os.environ["MSQ_MOEP_SKIP"] = "0"
+    gu_flops = 2.0 * 2 * DIM * INTER * total
+    achieved = gu_flops / (gu_mean * 1e-3) / 1e12
+    out = {
+        "value": value, "unit": "TFLOP/s", "ms_per_step": ms_step, "dtype": "f16 MFMA (bf16 activations staged as f16, exact IQ2_XXS weights), f32 accumulate",
+        "config": {"workload": "BASELINE configs[3]: prefill grouped MoE GEMM, 2048 tokens x 7168 bf16, top-6 of 384 experts, "
+                               "Zipf(1.1) popularity, IQ2_XXS gate/up 2048x7168 + down 7168x2048, outputs combined with routing weights",
+                   "entries": total, "experts_used": int(len(used)), "tokens_per_expert_max": int(counts.max()),
+                   "tokens_per_expert_median": float(np.median(counts[used])), "flops_per_step": flops,
+                   "weight_bytes_touched": int(len(used)) * per_exp},
+        "roofline": {"bound": "mfma", "achieved": achieved, "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": achieved / MFMA_PEAK_TFLOPS,
+                     "traffic": None, "kernel": "moe_pf_gemm_kernel<FragIQ2XXS,gate/up>", "flops_per_launch": gu_flops,
+                     "avg_launch_us": gu_mean * 1e3, "min_launch_us": gu_min * 1e3,
+                     "weight_GBps": int(len(used)) * 2 * gu_b / (gu_mean * 1e-3) / 1e9,
+                     "second_kernel": {"kernel": "moe_pf_gemm_kernel<FragIQ2XXS,down>", "avg_launch_us": dn_mean * 1e3,
+                                       "achieved": 2.0 * DIM * INTER * total / (dn_mean * 1e-3) / 1e12}},
+        "pct_of_mfma_peak": 100 * value / MFMA_PEAK_TFLOPS,
+    }
+    if with_cpu:
+        nth = cores()
+        n_chk = 4
+        chk = np.arange(n_chk, dtype=np.int32)
+        need = sorted(set(int(e) for e in ids[:n_chk].ravel()))
+        host = {e: (arena[e * per_exp:e * per_exp + gu_b].cpu().numpy(), arena[e * per_exp + gu_b:e * per_exp + 2 * gu_b].cpu().numpy(),
+                    arena[e * per_exp + 2 * gu_b:(e + 1) * per_exp].cpu().numpy()) for e in need}
+        dummy = host[need[0]]
+        G = [host.get(int(e), dummy)[0] for e in used]; U = [host.get(int(e), dummy)[1] for e in used]; D = [host.get(int(e), dummy)[2] for e in used]
+        Xh = X.float().cpu().numpy()
+        t0 = time.perf_counter()
+        O.moe_prefill(int(t), int(t), int(t), N, len(used), False, DIM, INTER, G, U, D, offs, tok, wt, Xh, chk, 1,
+                      np.zeros((N, DIM), np.float32), nthreads=nth)
+        el = time.perf_counter() - t0
+        cpu_flops = 2.0 * 3 * DIM * INTER * n_chk * TOPK
+        out["cpu_baseline"] = {"value": cpu_flops / el / 1e12, "unit": "TFLOP/s", "cores": nth, "kind": "port",
+                               "sample": "%d tokens x top-6 of the same routing through oracle.c moe_prefill (dequant each needed "
+                                         "expert row, double dots), %.1f s; whole job = x%d" % (n_chk, el, N // n_chk)}
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=500)
     ap.add_argument("--warmup", type=int, default=100)
     ap.add_argument("--workload", default="moe_decode",
-                    choices=["moe_decode", "matvec_iq1s", "matvec_iq2xxs", "q8_0"])
+                    choices=["moe_decode", "moe_prefill", "matvec_iq1s", "matvec_iq2xxs", "q8_0"])
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU (one MI355X per box); --gpus %d is not supported" % args.gpus, file=sys.stderr)
@@ -262,6 +373,14 @@ def main():
     if L.msq_init() != 0:
         print("bench.py: " + L.msq_last_error().decode(), file=sys.stderr)
         sys.exit(1)
+    if args.workload == "moe_prefill":
+        r = bench_moe_prefill(torch, max(1, min(args.steps, 20)), max(1, min(args.warmup, 3)))
+        out = {"metric": METRIC, "value": r["value"], "unit": "TFLOP/s", "n_gpus": 1, "steps": max(1, min(args.steps, 20)),
+               "warmup": max(1, min(args.warmup, 3)), "ms_per_step": r["ms_per_step"], "higher_is_better": True, "scaling": "weak",
+               "vs_baseline": None, "dtype": r["dtype"], "data": "synthetic", "config": r["config"], "roofline": r["roofline"],
+               "cpu_baseline": r["cpu_baseline"], "pct_of_mfma_peak": r["pct_of_mfma_peak"]}
+        print(json.dumps(out))
+        return
     if args.workload == "moe_decode":
         r = bench_moe_decode(torch, args)
     elif args.workload == "matvec_iq1s":
@@ -274,6 +393,12 @@ def main():
            "ms_per_step": r["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
            "dtype": r["dtype"], "data": "synthetic", "config": r["config"], "roofline": r["roofline"],
            "cpu_baseline": r["cpu_baseline"], "pct_of_hbm_peak": r["pct_of_hbm_peak"]}
+    if args.workload == "moe_decode":
+        # the metric's second half, measured in the same run on the same device (BASELINE configs[3])
+        torch.cuda.empty_cache()
+        p = bench_moe_prefill(torch, 5, 2, with_cpu=False)
+        out["prefill_moe_gemm"] = {"value": p["value"], "unit": "TFLOP/s", "ms_per_step": p["ms_per_step"],
+                                   "pct_of_mfma_peak": p["pct_of_mfma_peak"], "config": p["config"], "roofline": p["roofline"]}
     print(json.dumps(out))
 
 

@@ -40,6 +40,22 @@ def build(verbose=True):
     return OUT
 
 
+def build_shim_test(verbose=True):
+    """tests/cpp/shim_test: the C++ operator shim exercised like the reference's own test programs."""
+    root = os.path.join(HERE, "..")
+    src = os.path.join(root, "tests", "cpp", "shim_test.cpp")
+    out = os.path.join(root, "tests", "cpp", "shim_test")
+    r = subprocess.run([HIPCC, "-x", "hip", "--offload-arch=gfx950", "-O2", "-std=c++20", "-Wno-unused-command-line-argument",
+                        "-I" + os.path.join(root, "include"), src, "-o", out, "-L" + HERE, "-lmsq", "-Wl,-rpath," + os.path.abspath(HERE)],
+                       stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("shim_test build failed:\n" + r.stdout)
+    if verbose:
+        print("built", out)
+    return out
+
+
 if __name__ == "__main__":
     build()
+    build_shim_test()
     sys.exit(0)

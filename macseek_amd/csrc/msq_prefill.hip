@@ -1,5 +1,6 @@
 // C ABI: prefill MoE (see include/msq.h; reference host code src/kernels/quant.mm:372-612).
 #include <algorithm>
+#include <cstdlib>
 #include <vector>
 
 #include "msq_host.h"
@@ -102,6 +103,10 @@ int msq_moe_prefill(void* stream, const MsqMoePrefillArgs* p) {
 
   hipStream_t st = (hipStream_t)stream;
   const int cus = device_info().cus;
+  // PROFILING ONLY (wrong output): MSQ_MOEP_SKIP bit mask 1 gather, 2 routed gate/up, 4 shared gate/up, 8 routed down,
+  // 16 shared down, 32 reduce -- read on every call (reference: MACSEEK_MOEP_SKIP, src/kernels/quant.mm:520-522)
+  const char* skip_env = getenv("MSQ_MOEP_SKIP");
+  const int skip = skip_env && *skip_env ? atoi(skip_env) : 0;
   // ---- header: expert pointer table, offsets, token-tile tables (routed tiles first, then the shared expert's)
   const size_t hbytes = header_bytes(total, n, ne);
   std::vector<uint8_t> hdr(hbytes, 0);
@@ -140,7 +145,7 @@ int msq_moe_prefill(void* stream, const MsqMoePrefillArgs* p) {
 
   // 1) gather + convert
   const uint32_t grows = (uint32_t)(total + (p->has_shared ? n : 0));
-  if (grows > 0) {
+  if (grows > 0 && !(skip & 1)) {
     const dim3 grid((dim / 4 + 255) / 256, grows), block(256);
     const int* tok = total > 0 ? (const int*)bptr(&p->tok) : nullptr;
     if (p->x_is_bf16) hipLaunchKernelGGL((moe_pf_gather_kernel<true>), grid, block, 0, st, (const void*)bptr(&p->X), Xg, tok, (uint32_t)total, grows, (uint32_t)dim);
@@ -158,14 +163,14 @@ int msq_moe_prefill(void* stream, const MsqMoePrefillArgs* p) {
   int rc;
   // 2) gate + up + SwiGLU -> H
   a.A = Xg; a.N = (uint32_t)inter; steps((uint32_t)dim);
-  if (nt_routed) { a.tiles = d_tiles; a.ntiles = nt_routed; a.row_bytes = (uint32_t)rb_gu; if ((rc = launch_gemm<true>(p->t_gate_up, st, a, cus))) return rc; }
-  if (nt_shared) { a.tiles = d_tiles + 2 * nt_routed; a.ntiles = nt_shared; a.row_bytes = (uint32_t)rb_sgu; if ((rc = launch_gemm<true>(p->t_shared, st, a, cus))) return rc; }
+  if (nt_routed && !(skip & 2)) { a.tiles = d_tiles; a.ntiles = nt_routed; a.row_bytes = (uint32_t)rb_gu; if ((rc = launch_gemm<true>(p->t_gate_up, st, a, cus))) return rc; }
+  if (nt_shared && !(skip & 4)) { a.tiles = d_tiles + 2 * nt_routed; a.ntiles = nt_shared; a.row_bytes = (uint32_t)rb_sgu; if ((rc = launch_gemm<true>(p->t_shared, st, a, cus))) return rc; }
   // 3) down -> Z
   a.A = H; a.N = (uint32_t)dim; steps((uint32_t)inter);
-  if (nt_routed) { a.tiles = d_tiles; a.ntiles = nt_routed; a.row_bytes = (uint32_t)rb_d; if ((rc = launch_gemm<false>(p->t_down, st, a, cus))) return rc; }
-  if (nt_shared) { a.tiles = d_tiles + 2 * nt_routed; a.ntiles = nt_shared; a.row_bytes = (uint32_t)rb_sd; if ((rc = launch_gemm<false>(p->t_shared, st, a, cus))) return rc; }
+  if (nt_routed && !(skip & 8)) { a.tiles = d_tiles; a.ntiles = nt_routed; a.row_bytes = (uint32_t)rb_d; if ((rc = launch_gemm<false>(p->t_down, st, a, cus))) return rc; }
+  if (nt_shared && !(skip & 16)) { a.tiles = d_tiles + 2 * nt_routed; a.ntiles = nt_shared; a.row_bytes = (uint32_t)rb_sd; if ((rc = launch_gemm<false>(p->t_shared, st, a, cus))) return rc; }
   // 4) ordered reduction into Y
-  if (nt_routed || nt_shared) {
+  if ((nt_routed || nt_shared) && !(skip & 32)) {
     const dim3 grid((dim / 4 + 255) / 256, (unsigned)n), block(256);
     hipLaunchKernelGGL(moe_pf_reduce_kernel, grid, block, 0, st, (const float*)Z, (float*)bptr_mut(&p->Y),
                        p->k_per_token > 0 ? (const int*)bptr(&p->slot_of) : nullptr, (uint32_t)n, (uint32_t)total, (uint32_t)dim,

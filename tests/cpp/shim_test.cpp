@@ -1,0 +1,72 @@
+// The C++ shim (include/macseek_amd/quant.hpp) driven the way the reference's own tests drive ms::q
+// (tests/test_quant_matvec.mm:31-47): build inputs, encode on an Enc, wait, compare. Known answers only, so the
+// program needs nothing but the library: Q8_0 blocks with d = 1/8 and quants j - 16 against an exact host dot, the
+// same through encode_matvec_n, and the abort-on-misuse contract in a child process.
+#include <hip/hip_runtime.h>
+#include <sys/wait.h>
+#include <unistd.h>
+
+#include <cmath>
+#include <cstring>
+#include <vector>
+
+#include "macseek_amd/quant.hpp"
+
+#define HIP_OK(e) do { hipError_t r_ = (e); if (r_ != hipSuccess) { fprintf(stderr, "HIP: %s\n", hipGetErrorString(r_)); return 2; } } while (0)
+
+static ms::Buffer upload(const void* p, size_t n) {
+  void* d = nullptr;
+  if (hipMalloc(&d, n) != hipSuccess || hipMemcpy(d, p, n, hipMemcpyHostToDevice) != hipSuccess) abort();
+  return ms::Buffer{d, 0, n};
+}
+
+int main() {
+  namespace mq = ms::q;
+  const int rows = 48, cols = 512, n = 3;
+  std::vector<uint8_t> W((size_t)rows * mq::row_bytes(mq::QType::Q8_0, cols));
+  std::vector<float> x((size_t)cols * n), want((size_t)rows * n, 0.f);
+  for (size_t i = 0; i < x.size(); i++) x[i] = (float)((int)(i * 7 % 13) - 6) * 0.25f;  // exact in fp16
+  for (int r = 0; r < rows; r++)
+    for (int b = 0; b < cols / 32; b++) {
+      uint8_t* blk = W.data() + ((size_t)r * (cols / 32) + b) * 34;
+      const uint16_t d = 0x3000;  // fp16 0.125
+      memcpy(blk, &d, 2);
+      for (int j = 0; j < 32; j++) blk[2 + j] = (uint8_t)(int8_t)((j + r + b) % 33 - 16);
+      for (int t = 0; t < n; t++)
+        for (int j = 0; j < 32; j++) want[(size_t)t * rows + r] += 0.125f * (float)((j + r + b) % 33 - 16) * x[(size_t)t * cols + b * 32 + j];
+    }
+  ms::Buffer bw = upload(W.data(), W.size()), bx = upload(x.data(), x.size() * 4);
+  std::vector<float> zero((size_t)rows * n, 0.f), got((size_t)rows * n);
+  ms::Buffer by = upload(zero.data(), zero.size() * 4);
+  ms::Enc e;
+  int fails = 0;
+  mq::encode_matvec(e, mq::QType::Q8_0, bw, rows, cols, bx, by);  // n = 1: first activation row
+  HIP_OK(hipStreamSynchronize((hipStream_t)e.stream));
+  HIP_OK(hipMemcpy(got.data(), by.buf, rows * 4, hipMemcpyDeviceToHost));
+  for (int r = 0; r < rows; r++) if (std::fabs(got[r] - want[r]) > 1e-4f * (1.f + std::fabs(want[r]))) fails++;
+  printf("  encode_matvec   Q8_0 [%d -> %d] %s\n", cols, rows, fails ? "FAIL" : "ok");
+  mq::encode_matvec_n(e, mq::QType::Q8_0, bw, rows, cols, bx, by, n);
+  HIP_OK(hipStreamSynchronize((hipStream_t)e.stream));
+  HIP_OK(hipMemcpy(got.data(), by.buf, got.size() * 4, hipMemcpyDeviceToHost));
+  int f2 = 0;
+  for (size_t i = 0; i < got.size(); i++) if (std::fabs(got[i] - want[i]) > 1e-4f * (1.f + std::fabs(want[i]))) f2++;
+  printf("  encode_matvec_n Q8_0 [%d -> %d] n=%d %s\n", cols, rows, n, f2 ? "FAIL" : "ok");
+  fails += f2;
+  if (mq::matvec_cfg(mq::QType::Q8_0, rows, cols).ks < 1) fails++;
+  // misuse aborts like the reference (src/kernels/quant.mm:34-37): cols not a multiple of the block size
+  fflush(stdout);
+  const pid_t pid = fork();
+  if (pid == 0) {
+    fclose(stderr);
+    ms::Enc e2;
+    mq::encode_matvec(e2, mq::QType::Q6_K, bw, 4, 300, bx, by);
+    _exit(0);
+  }
+  int st = 0;
+  waitpid(pid, &st, 0);
+  const bool aborted = WIFSIGNALED(st) && WTERMSIG(st) == SIGABRT;
+  printf("  misuse aborts: %s\n", aborted ? "ok" : "FAIL");
+  fails += !aborted;
+  printf(fails ? "FAILED (%d)\n" : "all OK\n", fails);
+  return fails ? 1 : 0;
+}
