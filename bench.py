@@ -169,13 +169,14 @@ def bench_moe_decode(torch, args):
     xh = host(x)
     t0 = time.perf_counter()
     n_cpu = 0
-    while True:
+    while not args.gpu_only:
         O.moe_decode(int(tr), int(tr), int(ts), TOPK, True, DIM, INTER, G, U, D, wts[i0], xh, np.zeros(DIM, np.float32), nthreads=nth)
         n_cpu += 1
         el = time.perf_counter() - t0
         if el > 10.0 or n_cpu >= 200:
             break
-    cpu_value = step_bytes * n_cpu / el / 1e9
+    el = time.perf_counter() - t0
+    cpu_value = step_bytes * n_cpu / el / 1e9 if n_cpu else None
 
     return {
         "value": value, "ms_per_step": ms_step, "dtype": "f16 activations x IQ1_S/IQ2_XXS codebook weights, f32 accumulate",
@@ -359,6 +360,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=100)
     ap.add_argument("--workload", default="moe_decode",
                     choices=["moe_decode", "moe_prefill", "matvec_iq1s", "matvec_iq2xxs", "q8_0"])
+    ap.add_argument("--gpu-only", action="store_true",
+                    help="profiling runs: skip the CPU baseline leg and the prefill appendix of the default workload")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU (one MI355X per box); --gpus %d is not supported" % args.gpus, file=sys.stderr)
@@ -393,7 +396,7 @@ def main():
            "ms_per_step": r["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
            "dtype": r["dtype"], "data": "synthetic", "config": r["config"], "roofline": r["roofline"],
            "cpu_baseline": r["cpu_baseline"], "pct_of_hbm_peak": r["pct_of_hbm_peak"]}
-    if args.workload == "moe_decode":
+    if args.workload == "moe_decode" and not args.gpu_only:
         # the metric's second half, measured in the same run on the same device (BASELINE configs[3])
         torch.cuda.empty_cache()
         p = bench_moe_prefill(torch, 5, 2, with_cpu=False)

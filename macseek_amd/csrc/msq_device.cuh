@@ -93,11 +93,50 @@ typedef uint32_t __attribute__((aligned(2), may_alias)) u32_a2;
 struct __attribute__((packed, aligned(2))) u64_a2 { uint32_t x, y; };
 struct __attribute__((packed, aligned(2))) u128_a2 { uint32_t x, y, z, w; };
 
-__device__ __forceinline__ uint32_t ld8(const uint8_t* p) { return *p; }
-__device__ __forceinline__ uint32_t ld16(const uint8_t* p) { return *(const uint16_t*)p; }
-__device__ __forceinline__ uint32_t ld32(const uint8_t* p) { return *(const u32_a2*)p; }
-__device__ __forceinline__ u64_a2 ld64(const uint8_t* p) { return *(const u64_a2*)p; }
-__device__ __forceinline__ u128_a2 ld128(const uint8_t* p) { return *(const u128_a2*)p; }
+typedef uint32_t __attribute__((ext_vector_type(2), aligned(2))) u32x2_a2;
+typedef uint32_t __attribute__((ext_vector_type(4), aligned(2))) u32x4_a2;
+
+// Weight pointers that reach a kernel through a table or a struct are "generic" to the compiler, and generic loads are
+// FLAT instructions: they count against the LDS counter as well, so every wait for a table lookup would also wait for
+// the weight prefetches in flight. Such pointers are therefore cast to the global address space (gptr_t) once, and
+// the byte loaders exist for both kinds of pointer.
+#define MSQ_GLOBAL __attribute__((address_space(1)))
+typedef const MSQ_GLOBAL uint8_t* gptr_t;
+__device__ __forceinline__ gptr_t as_global(const void* p) { return (gptr_t)p; }
+
+// Range-checked buffer loads: the descriptor covers `bytes` bytes at `base`; a load whose offset falls outside returns
+// zero without touching memory. A pipelined loop can thus issue its prefetches unconditionally (an empty descriptor for
+// the rows past the end), which keeps the number of loads in flight known at every wait.
+typedef __amdgpu_buffer_rsrc_t rsrc_t;
+__device__ __forceinline__ rsrc_t make_rsrc(const void* base, uint32_t bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)bytes, 0x00020000);
+}
+__device__ __forceinline__ uint32_t buf_ld16(rsrc_t r, uint32_t voff, uint32_t soff) {
+  return (uint16_t)__builtin_amdgcn_raw_buffer_load_b16(r, (int)voff, (int)soff, 0);
+}
+__device__ __forceinline__ uint32_t buf_ld32(rsrc_t r, uint32_t voff, uint32_t soff) {
+  return (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(r, (int)voff, (int)soff, 0);
+}
+__device__ __forceinline__ u64_a2 buf_ld64(rsrc_t r, uint32_t voff, uint32_t soff) {
+  const auto v = __builtin_amdgcn_raw_buffer_load_b64(r, (int)voff, (int)soff, 0);
+  return {(uint32_t)v[0], (uint32_t)v[1]};
+}
+
+#define MSQ_LOADERS(AS)                                                                                               \
+  __device__ __forceinline__ uint32_t ld8(const AS uint8_t* p) { return *p; }                                         \
+  __device__ __forceinline__ uint32_t ld16(const AS uint8_t* p) { return *(const AS uint16_t*)p; }                    \
+  __device__ __forceinline__ uint32_t ld32(const AS uint8_t* p) { return *(const AS u32_a2*)p; }                      \
+  __device__ __forceinline__ u64_a2 ld64(const AS uint8_t* p) {                                                       \
+    const u32x2_a2 v = *(const AS u32x2_a2*)p;                                                                        \
+    return {v.x, v.y};                                                                                                \
+  }                                                                                                                   \
+  __device__ __forceinline__ u128_a2 ld128(const AS uint8_t* p) {                                                     \
+    const u32x4_a2 v = *(const AS u32x4_a2*)p;                                                                        \
+    return {v.x, v.y, v.z, v.w};                                                                                      \
+  }
+MSQ_LOADERS()
+MSQ_LOADERS(MSQ_GLOBAL)
+#undef MSQ_LOADERS
 
 __device__ __forceinline__ float half_bits_to_float(uint32_t b) {
   return (float)__builtin_bit_cast(_Float16, (uint16_t)b);
@@ -193,11 +232,12 @@ __device__ __forceinline__ void copy_words16(uint32_t* dst, const uint32_t* src,
 // the slice. The window goes to a per-wave LDS staging area, from which every lane picks the few bytes of its own
 // unit; `shift` (slice start within its first granule) is wave-uniform.
 constexpr int kStageBytes = 576;  // per staged slice: up to 528 slice bytes + 15 shift, rounded to 64
-__device__ __forceinline__ uint4 slice_load(const uint8_t* start, uint32_t nbytes, uint32_t lane) {
+typedef uint32_t __attribute__((ext_vector_type(4))) u32x4;
+__device__ __forceinline__ uint4 slice_load(gptr_t start, uint32_t nbytes, uint32_t lane) {
   const uint32_t shift = (uint32_t)((uintptr_t)start & 15u);
-  uint4 v = {0u, 0u, 0u, 0u};
-  if (16u * lane < shift + nbytes) v = *(const uint4*)(start - shift + 16u * lane);
-  return v;
+  u32x4 v = {0u, 0u, 0u, 0u};
+  if (16u * lane < shift + nbytes) v = *(const MSQ_GLOBAL u32x4*)(start - shift + 16u * lane);
+  return {v.x, v.y, v.z, v.w};
 }
 __device__ __forceinline__ void slice_stage(uint8_t* stage, const uint4& v, uint32_t lane) {
   if (lane < kStageBytes / 16) ((uint4*)stage)[lane] = v;
@@ -250,10 +290,20 @@ struct DecIQ1S {
     r.sx = sum_h2(r.v, 16);
     return r;
   }
-  __device__ static Raw load(const uint8_t* row, uint32_t u) {
-    const uint8_t* b = row + (u >> 3) * 50u;
+  template <class P>
+  __device__ static Raw load(P row, uint32_t u) {
+    const P b = row + (u >> 3) * 50u;
     const uint32_t ib = u & 7u;
     return {ld32(b + 2 + 4 * ib), ld16(b + 34 + 2 * ib), ld16(b)};
+  }
+  // the same bytes through a buffer descriptor: Off holds the lane's byte offsets inside a row, soff the row's offset
+  struct Off { uint32_t qs, qh, d; };
+  __device__ static Off offsets(uint32_t u) {
+    const uint32_t b = (u >> 3) * 50u, ib = u & 7u;
+    return {b + 2 + 4 * ib, b + 34 + 2 * ib, b};
+  }
+  __device__ static Raw fetch(rsrc_t rs, const Off& o, uint32_t soff) {
+    return {buf_ld32(rs, o.qs, soff), buf_ld16(rs, o.qh, soff), buf_ld16(rs, o.d, soff)};
   }
   __device__ static float dot(const Raw& r, const X& x, const uint32_t* lds) {
     const uint4* grid = (const uint4*)lds;
@@ -266,6 +316,33 @@ struct DecIQ1S {
       acc = dot2(g.y, x.v[4 * l + 1], acc);
       acc = dot2(g.z, x.v[4 * l + 2], acc);
       acc = dot2(g.w, x.v[4 * l + 3], acc);
+    }
+    const float dl = half_bits_to_float(r.d) * (float)(2u * ((r.qh >> 12) & 7u) + 1u);
+    const float delta = (r.qh & 0x8000u) ? -0.125f : 0.125f;
+    return dl * (acc + delta * x.sx);
+  }
+  // the same dot split for software pipelining: lookup() only issues the table reads of a stage, partial() consumes
+  // them (the last stage applies the scale), so a caller can keep the next stage's reads in flight during the math
+  static constexpr int STAGES = 1;
+  struct Look { uint4 g[4]; };
+  __device__ static Look lookup(const Raw& r, int, const uint32_t* lds) {
+    const uint8_t* grid = (const uint8_t*)lds;
+    Look k;
+#pragma unroll
+    for (int l = 0; l < 4; l++) {
+      const uint32_t off = (((r.qs >> (8 * l)) & 0xFFu) << 4) | (((r.qh >> (3 * l)) & 7u) << 12);
+      k.g[l] = *(const uint4*)(grid + off);
+    }
+    return k;
+  }
+  __device__ static float partial(const Raw& r, const Look& k, const X& x, int, float) {
+    float acc = 0.f;
+#pragma unroll
+    for (int l = 0; l < 4; l++) {
+      acc = dot2(k.g[l].x, x.v[4 * l + 0], acc);
+      acc = dot2(k.g[l].y, x.v[4 * l + 1], acc);
+      acc = dot2(k.g[l].z, x.v[4 * l + 2], acc);
+      acc = dot2(k.g[l].w, x.v[4 * l + 3], acc);
     }
     const float dl = half_bits_to_float(r.d) * (float)(2u * ((r.qh >> 12) & 7u) + 1u);
     const float delta = (r.qh & 0x8000u) ? -0.125f : 0.125f;
@@ -289,10 +366,20 @@ struct DecIQ2XXS {
     r.sx = 0.f;
     return r;
   }
-  __device__ static Raw load(const uint8_t* row, uint32_t u) {
-    const uint8_t* b = row + (u >> 3) * 66u;
+  template <class P>
+  __device__ static Raw load(P row, uint32_t u) {
+    const P b = row + (u >> 3) * 66u;
     const u64_a2 a = ld64(b + 2 + 8 * (u & 7u));
     return {a.x, a.y, ld16(b)};
+  }
+  struct Off { uint32_t a, d; };
+  __device__ static Off offsets(uint32_t u) {
+    const uint32_t b = (u >> 3) * 66u;
+    return {b + 2 + 8 * (u & 7u), b};
+  }
+  __device__ static Raw fetch(rsrc_t rs, const Off& o, uint32_t soff) {
+    const u64_a2 a = buf_ld64(rs, o.a, soff);
+    return {a.x, a.y, buf_ld16(rs, o.d, soff)};
   }
   __device__ static float dot(const Raw& r, const X& x, const uint32_t* lds) {
     const uint4* grid = (const uint4*)lds;
@@ -310,6 +397,33 @@ struct DecIQ2XXS {
     const float db = half_bits_to_float(r.d) * (0.5f + (float)(r.a1 >> 28)) * 0.25f;
     return db * acc;
   }
+  // two pipeline stages of two grid entries each (see DecIQ1S)
+  static constexpr int STAGES = 2;
+  struct Look { uint4 g[2], s[2]; };
+  __device__ static Look lookup(const Raw& r, int stage, const uint32_t* lds) {
+    const uint8_t* grid = (const uint8_t*)lds;
+    const uint8_t* sign = (const uint8_t*)(lds + MSQ_IQ2XXS_GRID_N * 4);
+    Look k;
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+      const int l = 2 * stage + i;
+      k.g[i] = *(const uint4*)(grid + (((r.a0 >> (8 * l)) & 0xFFu) << 4));
+      k.s[i] = *(const uint4*)(sign + (((r.a1 >> (7 * l)) & 127u) << 4));
+    }
+    return k;
+  }
+  __device__ static float partial(const Raw& r, const Look& k, const X& x, int stage, float acc) {
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+      const int l = 2 * stage + i;
+      acc = dot2(k.g[i].x ^ k.s[i].x, x.v[4 * l + 0], acc);
+      acc = dot2(k.g[i].y ^ k.s[i].y, x.v[4 * l + 1], acc);
+      acc = dot2(k.g[i].z ^ k.s[i].z, x.v[4 * l + 2], acc);
+      acc = dot2(k.g[i].w ^ k.s[i].w, x.v[4 * l + 3], acc);
+    }
+    if (stage == 1) acc *= half_bits_to_float(r.d) * (0.5f + (float)(r.a1 >> 28)) * 0.25f;
+    return acc;
+  }
 };
 
 // ---- Q8_0: {fp16 d; int8 qs[32]}, 34 bytes / 32 weights; unit = one block, activations kept in fp32
@@ -325,8 +439,9 @@ struct DecQ8_0 {
     for (int i = 0; i < 8; i++) { const float4 f = p[i]; r.v[4 * i] = f.x; r.v[4 * i + 1] = f.y; r.v[4 * i + 2] = f.z; r.v[4 * i + 3] = f.w; }
     return r;
   }
-  __device__ static Raw load(const uint8_t* row, uint32_t u) {
-    const uint8_t* b = row + u * 34u;
+  template <class P>
+  __device__ static Raw load(P row, uint32_t u) {
+    const P b = row + u * 34u;
     const u128_a2 a = ld128(b + 2), c = ld128(b + 18);
     return {{a.x, a.y, a.z, a.w, c.x, c.y, c.z, c.w}, ld16(b)};
   }
@@ -361,8 +476,9 @@ struct DecIQ4NL {
     }
     return r;
   }
-  __device__ static Raw load(const uint8_t* row, uint32_t u) {
-    const uint8_t* b = row + u * 18u;
+  template <class P>
+  __device__ static Raw load(P row, uint32_t u) {
+    const P b = row + u * 18u;
     const u128_a2 a = ld128(b + 2);
     return {{a.x, a.y, a.z, a.w}, ld16(b)};
   }
@@ -396,8 +512,9 @@ struct DecQ6K {
     }
     return r;
   }
-  __device__ static Raw load(const uint8_t* row, uint32_t u) {
-    const uint8_t* b = row + (u >> 3) * 210u;
+  template <class P>
+  __device__ static Raw load(P row, uint32_t u) {
+    const P b = row + (u >> 3) * 210u;
     const uint32_t j = u & 7u, h = j >> 2, l0 = 8u * (j & 3u);
     const u64_a2 a = ld64(b + 64 * h + l0), c = ld64(b + 64 * h + 32 + l0), q = ld64(b + 128 + 32 * h + l0);
     const u64_a2 s = ld64(b + 192 + 8 * h);
@@ -445,8 +562,9 @@ struct DecQ5K {
     r.sx[1] = sum_h2(r.v + 8, 8);
     return r;
   }
-  __device__ static Raw load(const uint8_t* row, uint32_t u) {
-    const uint8_t* b = row + (u >> 3) * 176u;
+  template <class P>
+  __device__ static Raw load(P row, uint32_t u) {
+    const P b = row + (u >> 3) * 176u;
     const uint32_t j = u & 7u, g = j >> 1, l0 = 16u * (j & 1u), is = 2u * g;
     const u128_a2 l = ld128(b + 48 + 32 * g + l0), h = ld128(b + 16 + l0);
     // scale bytes is, is+1 (pa), is+4, is+5 (pb) and, for the upper groups, is-4, is-3 (pc)
@@ -491,7 +609,8 @@ struct DecDense {
     r.v[0] = a.x; r.v[1] = a.y; r.v[2] = a.z; r.v[3] = a.w; r.v[4] = b.x; r.v[5] = b.y; r.v[6] = b.z; r.v[7] = b.w;
     return r;
   }
-  __device__ static Raw load(const uint8_t* row, uint32_t u) {
+  template <class P>
+  __device__ static Raw load(P row, uint32_t u) {
     Raw r;
     if constexpr (QT == MSQ_F32) {
       const u128_a2 a = ld128(row + 32u * u), b = ld128(row + 32u * u + 16);

@@ -57,8 +57,9 @@ struct FragIQ1S {
   static constexpr int LDS_WORDS = MSQ_IQ1S_GRID_N * 4;
   __device__ static void fill_lds(uint32_t* lds, int tid, int nt) { copy_words16(lds, g_tbl_iq1s.w, LDS_WORDS, tid, nt); }
   __device__ static uint32_t col_of(uint32_t q, uint32_t p) { return 8u * q + p; }
-  __device__ static FragOut get(const uint8_t* row, uint32_t step, uint32_t q, const uint32_t* tbl) {
-    const uint8_t* b = row + (step >> 3) * 50u;
+  template <class P>
+  __device__ static FragOut get(P row, uint32_t step, uint32_t q, const uint32_t* tbl) {
+    const P b = row + (step >> 3) * 50u;
     const uint32_t ib = step & 7u;
     const uint32_t qh = ld16(b + 34 + 2 * ib);
     const uint32_t idx = ld8(b + 2 + 4 * ib + q) | (((qh >> (3 * q)) & 7u) << 8);
@@ -78,9 +79,10 @@ struct FragIQ2XXS {
   static constexpr int LDS_WORDS = MSQ_IQ2XXS_GRID_N * 4 + 128 * 4;
   __device__ static void fill_lds(uint32_t* lds, int tid, int nt) { DecIQ2XXS::fill_lds(lds, tid, nt); }
   __device__ static uint32_t col_of(uint32_t q, uint32_t p) { return 8u * q + p; }
-  __device__ static FragOut get(const uint8_t* row, uint32_t step, uint32_t q, const uint32_t* tbl) {
-    const uint8_t* b = row + (step >> 3) * 66u;
-    const uint8_t* a8 = b + 2 + 8 * (step & 7u);
+  template <class P>
+  __device__ static FragOut get(P row, uint32_t step, uint32_t q, const uint32_t* tbl) {
+    const P b = row + (step >> 3) * 66u;
+    const P a8 = b + 2 + 8 * (step & 7u);
     const uint32_t a1 = ld32(a8 + 4);
     const uint4 g = ((const uint4*)tbl)[ld8(a8 + q)];
     const uint4 s = ((const uint4*)(tbl + MSQ_IQ2XXS_GRID_N * 4))[(a1 >> (7 * q)) & 127u];
@@ -97,8 +99,9 @@ struct FragQ8_0 {
   static constexpr int LDS_WORDS = 0;
   __device__ static void fill_lds(uint32_t*, int, int) {}
   __device__ static uint32_t col_of(uint32_t q, uint32_t p) { return 8u * q + p; }
-  __device__ static FragOut get(const uint8_t* row, uint32_t step, uint32_t q, const uint32_t*) {
-    const uint8_t* b = row + step * 34u;
+  template <class P>
+  __device__ static FragOut get(P row, uint32_t step, uint32_t q, const uint32_t*) {
+    const P b = row + step * 34u;
     const u64_a2 v = ld64(b + 2 + 8 * q);
     const uint32_t lo = v.x ^ 0x80808080u, hi = v.y ^ 0x80808080u;  // bytes become q + 128
     const uint32_t bias = 0xE480E480u;                              // -1152 in both halves
@@ -118,8 +121,9 @@ struct FragIQ4NL {
   static constexpr int LDS_WORDS = 256;
   __device__ static void fill_lds(uint32_t* lds, int tid, int nt) { copy_words16(lds, g_tbl_iq4nl.w, 256, tid, nt); }
   __device__ static uint32_t col_of(uint32_t q, uint32_t p) { return 4u * q + (p >> 1) + 16u * (p & 1u); }
-  __device__ static FragOut get(const uint8_t* row, uint32_t step, uint32_t q, const uint32_t* tbl) {
-    const uint8_t* b = row + step * 18u;
+  template <class P>
+  __device__ static FragOut get(P row, uint32_t step, uint32_t q, const uint32_t* tbl) {
+    const P b = row + step * 18u;
     const uint32_t v = ld32(b + 2 + 4 * q);
     FragOut o;
     o.h[0] = tbl[v & 0xFFu]; o.h[1] = tbl[(v >> 8) & 0xFFu]; o.h[2] = tbl[(v >> 16) & 0xFFu]; o.h[3] = tbl[v >> 24];
@@ -136,8 +140,9 @@ struct FragQ6K {
   static constexpr int LDS_WORDS = 0;
   __device__ static void fill_lds(uint32_t*, int, int) {}
   __device__ static uint32_t col_of(uint32_t q, uint32_t p) { return 8u * q + p; }
-  __device__ static FragOut get(const uint8_t* row, uint32_t step, uint32_t q, const uint32_t*) {
-    const uint8_t* b = row + (step >> 3) * 210u;
+  template <class P>
+  __device__ static FragOut get(P row, uint32_t step, uint32_t q, const uint32_t*) {
+    const P b = row + (step >> 3) * 210u;
     const uint32_t e0 = 32u * (step & 7u) + 8u * q, h = e0 >> 7, k = (e0 & 127u) >> 5, l0 = e0 & 31u;
     const u64_a2 ql = ld64(b + 64 * h + 32 * (k & 1u) + l0), qh = ld64(b + 128 + 32 * h + l0);
     const uint32_t sh4 = 4u * (k >> 1), sh2 = 2u * k;
@@ -151,8 +156,9 @@ struct FragQ6K {
     o.add = 0.f;
     return o;
   }
-  __device__ static void get_scales(const uint8_t* row, uint32_t step, float& sa, float& sb) {
-    const uint8_t* b = row + (step >> 3) * 210u;
+  template <class P>
+  __device__ static void get_scales(P row, uint32_t step, float& sa, float& sb) {
+    const P b = row + (step >> 3) * 210u;
     const uint32_t e0 = 32u * (step & 7u), h = e0 >> 7, k = (e0 & 127u) >> 5;
     const uint32_t sc = ld16(b + 192 + 8 * h + 2 * k);
     const float d = half_bits_to_float(ld16(b + 208));
@@ -166,14 +172,15 @@ struct FragQ5K {
   static constexpr int LDS_WORDS = 0;
   __device__ static void fill_lds(uint32_t*, int, int) {}
   __device__ static uint32_t col_of(uint32_t q, uint32_t p) { return 8u * q + p; }
-  __device__ static FragOut get(const uint8_t* row, uint32_t step, uint32_t q, const uint32_t*) {
-    const uint8_t* b = row + (step >> 3) * 176u;
+  template <class P>
+  __device__ static FragOut get(P row, uint32_t step, uint32_t q, const uint32_t*) {
+    const P b = row + (step >> 3) * 176u;
     const uint32_t is = step & 7u, g = is >> 1, run = is & 1u, l0 = 8u * q;
     const u64_a2 ql = ld64(b + 48 + 32 * g + l0), qh = ld64(b + 16 + l0);
     const uint32_t q0 = ((ql.x >> (4 * run)) & 0x0F0F0F0Fu) | (((qh.x >> is) & 0x01010101u) << 4);
     const uint32_t q1 = ((ql.y >> (4 * run)) & 0x0F0F0F0Fu) | (((qh.y >> is) & 0x01010101u) << 4);
     const uint32_t bias = 0xE400E400u;  // -1024 in both halves
-    const uint8_t* s = b + 4;
+    const P s = b + 4;
     uint32_t sc, mn;
     if (is < 4) { sc = ld8(s + is) & 63u; mn = ld8(s + is + 4) & 63u; }
     else { sc = (ld8(s + is + 4) & 0xFu) | ((ld8(s + is - 4) >> 6) << 4); mn = (ld8(s + is + 4) >> 4) | ((ld8(s + is) >> 6) << 4); }
@@ -193,7 +200,8 @@ struct FragDense16 {
   static constexpr int LDS_WORDS = 0;
   __device__ static void fill_lds(uint32_t*, int, int) {}
   __device__ static uint32_t col_of(uint32_t q, uint32_t p) { return 8u * q + p; }
-  __device__ static FragOut get(const uint8_t* row, uint32_t step, uint32_t q, const uint32_t*) {
+  template <class P>
+  __device__ static FragOut get(P row, uint32_t step, uint32_t q, const uint32_t*) {
     const u128_a2 v = ld128(row + 64u * step + 16u * q);
     FragOut o;
     o.h[0] = v.x; o.h[1] = v.y; o.h[2] = v.z; o.h[3] = v.w;

@@ -13,12 +13,14 @@
 // order and run the epilogue.
 #pragma once
 #include "msq_device.cuh"
+#ifndef MSQ_EXP
+#define MSQ_EXP 0
+#endif
 
 namespace msq {
 
 constexpr int kMaxRouted = 6;
 constexpr int kMoeChunkRows = 128;  // rows a workgroup finishes between two synchronisations
-constexpr bool kStagedGateUp = false;  // stream gate/up weights through LDS staging (coalesced 128-bit loads)
 
 struct MoeArgs {
   const float* x;        // [dim]
@@ -55,6 +57,10 @@ constexpr int rows_in_flight(int matrices) {
 }
 
 __device__ __forceinline__ uint32_t uniform(uint32_t v) { return (uint32_t)__builtin_amdgcn_readfirstlane((int)v); }
+__device__ __forceinline__ const void* uniform(const void* p) {
+  const uint64_t v = (uint64_t)p;
+  return (const void*)((uint64_t)uniform((uint32_t)v) | ((uint64_t)uniform((uint32_t)(v >> 32)) << 32));
+}
 
 // gate + up + SwiGLU over the virtual rows [wg * per, ...) of one kind of expert (routed: e * inter + r; shared: r).
 template <class D, int RPW>
@@ -76,13 +82,13 @@ __device__ __forceinline__ void moe_gu_run_direct(const MoeArgs& a, uint32_t* sm
   const uint32_t PSTRIDE = 4 * KS + 1;  // partial sums per (row, matrix): 4 sixteen-lane rows per K-split wave, padded
 
   // address of virtual row v of the gate (which = 0) or up (1) matrices
-  auto row_ptr = [&](uint32_t v, int which) -> const uint8_t* {
+  auto row_ptr = [&](uint32_t v, int which) -> gptr_t {
     const uint32_t e = shared ? 0u : v / a.inter, r = v - e * a.inter;
     const uint8_t* base;
     if (shared) base = which ? a.sup : a.sgate;
     else if (a.table) base = (const uint8_t*)a.table[3 * e + which];
     else base = which ? a.up[e] : a.gate[e];
-    return base + (size_t)r * row_bytes;
+    return as_global(base) + (size_t)r * row_bytes;
   };
 
   typename D::X xr;
@@ -154,92 +160,111 @@ __device__ __forceinline__ void moe_gu_run_direct(const MoeArgs& a, uint32_t* sm
   }
 }
 
-// Same computation with the weights streamed through LDS staging (decoders with SLICE_BYTES > 0): per row pair a wave
-// issues two coalesced 128-bit loads (its K slice of the gate row and of the up row), DEPTH row pairs ahead.
+// Same computation for the codebook decoders (those with lookup() / partial() stages), arranged for memory-level
+// parallelism: a wave keeps the block bytes of NR row pairs in flight in a register ring -- a slot is refilled with the
+// row pair NR places ahead as soon as its bytes have been consumed -- so that about NR x 2 x (slice of a row) bytes per
+// wave are outstanding at any time, which is what it takes to keep HBM busy at batch 1. The refills are range-checked
+// buffer loads issued unconditionally (an empty descriptor past the end of the wave's run), so every wait in the loop
+// names an exact number of loads that may stay in flight. Table lookups run one decoder stage ahead of the dot
+// products (two alternating lookup buffers), so LDS latency overlaps the math as well.
 template <class D>
-__device__ __forceinline__ void moe_gu_run_staged(const MoeArgs& a, uint32_t* smem, const bool shared, const uint32_t wg) {
-  constexpr int DEPTH = 4;
+__device__ __forceinline__ void moe_gu_run_ring(const MoeArgs& a, uint32_t* smem, const bool shared, const uint32_t wg) {
+  constexpr int NR = 8;  // row pairs in flight per wave
+  constexpr int NS = D::STAGES;
   uint32_t* tbl = smem;
+  float* part = (float*)(smem + D::LDS_WORDS);
   const uint32_t tid = threadIdx.x, lane = tid & 63u;
   const uint32_t wave = uniform(tid >> 6), nwaves = blockDim.x >> 6;
   const uint32_t KS = a.ks, ks = wave % KS, rw = wave / KS, RW = nwaves / KS;
   const uint32_t PSTRIDE = 4 * KS + 1;
-  float* part = (float*)(smem + D::LDS_WORDS);
-  uint8_t* stage_g = (uint8_t*)(part + kMoeChunkRows * 2 * PSTRIDE) + (size_t)wave * 2 * kStageBytes;
-  uint8_t* stage_u = stage_g + kStageBytes;
   const uint32_t units = a.dim / D::UNIT;
   const uint32_t row_bytes = shared ? a.rb_gu_s : a.rb_gu_r;
+  const uint32_t mat_bytes = a.inter * row_bytes;
   const uint32_t total = (shared ? 1u : a.n_routed) * a.inter;
   const uint32_t per = shared ? a.rows_per_wg_s : a.rows_per_wg_r;
   const uint32_t wg_begin = wg * per, wg_end = min(total, wg_begin + per);
 
   const uint32_t u0 = ks * 64u + lane;
   const bool valid = u0 < units;
-  const uint32_t unit = valid ? u0 : units - 1;           // activations: idle lanes shadow the last unit
-  const uint32_t lunit = valid ? lane : (units - 1) & 63u;  // unit inside the staged slice
-  const uint32_t slice_off = ks * (uint32_t)D::SLICE_BYTES;
-  const uint32_t slice_bytes = min((uint32_t)D::SLICE_BYTES, row_bytes - slice_off);
-
-  auto row_ptr = [&](uint32_t v, int which) -> const uint8_t* {
-    const uint32_t e = shared ? 0u : v / a.inter, r = v - e * a.inter;
-    const uint8_t* base;
-    if (shared) base = which ? a.sup : a.sgate;
-    else if (a.table) base = (const uint8_t*)a.table[3 * e + which];
-    else base = which ? a.up[e] : a.gate[e];
-    return base + (size_t)r * row_bytes + slice_off;
-  };
+  const uint32_t unit = valid ? u0 : units - 1;  // lanes past the row shadow the last unit; their activations are zero
+  const typename D::Off off = D::offsets(unit);
 
   typename D::X xr;
   bool first = true;
   for (uint32_t c0 = wg_begin; c0 < wg_end; c0 += kMoeChunkRows) {
     const uint32_t c1 = min(wg_end, c0 + kMoeChunkRows), n = c1 - c0;
-    const uint32_t run = (n + RW - 1) / RW;
+    const uint32_t run = uniform((n + RW - 1) / RW);  // divisions run on the vector unit: bring the results back
     const uint32_t w0 = min(c0 + rw * run, c1), w1 = min(w0 + run, c1);
-    uint4 pg[DEPTH], pu[DEPTH];
-    uint32_t sg[DEPTH], su[DEPTH];  // shift of each in-flight slice inside its first 16-byte granule
-#pragma unroll
-    for (int s = 0; s < DEPTH; s++) {
-      if (w0 + s < w1) {
-        const uint8_t *g = row_ptr(w0 + s, 0), *u = row_ptr(w0 + s, 1);
-        pg[s] = slice_load(g, slice_bytes, lane); sg[s] = (uint32_t)((uintptr_t)g & 15u);
-        pu[s] = slice_load(u, slice_bytes, lane); su[s] = (uint32_t)((uintptr_t)u & 15u);
-      }
+
+    // cursor of the next row pair to fetch: expert pe, row pr of it, matrix bases pg / pu (all wave-uniform)
+    uint32_t pv = uniform(w0), pe = 0, pr = pv;
+    const void *pg = nullptr, *pu = nullptr;
+    auto set_expert = [&]() {
+      if (shared) { pg = a.sgate; pu = a.sup; }
+      else if (a.table) { pg = (const void*)a.table[3 * pe]; pu = (const void*)a.table[3 * pe + 1]; }
+      else { pg = a.gate[pe]; pu = a.up[pe]; }
+      pg = uniform(pg); pu = uniform(pu);  // buffer descriptors live in scalar registers
+    };
+    if (w0 < w1) {
+      if (!shared) { pe = uniform(w0 / a.inter); pr = uniform(w0 - pe * a.inter); }
+      set_expert();
     }
+    typename D::Raw rg[NR], ru[NR];
+    auto fetch = [&](int s) {  // loads of row pair pv into slot s (nothing is read once pv has passed w1), then advance
+      const uint32_t bytes = pv < w1 ? mat_bytes : 0u;
+      const uint32_t soff = pr * row_bytes;
+      rg[s] = D::fetch(make_rsrc(pg, bytes), off, soff);
+      ru[s] = D::fetch(make_rsrc(pu, bytes), off, soff);
+      pv++; pr++;
+      if (!shared && pr == a.inter && pv < w1) { pr = 0; pe++; set_expert(); }
+    };
+#pragma unroll
+    for (int s = 0; s < NR; s++) fetch(s);
     if (first) {  // tables and activations arrive while the first weight rows are in flight
       D::fill_lds(tbl, (int)tid, (int)blockDim.x);
       xr = D::load_x(a.x, unit);
+      if (!valid) xr = typename D::X{};
       __syncthreads();
       first = false;
     }
-    for (uint32_t r0 = w0; r0 < w1; r0 += DEPTH) {
-      float acc[2 * DEPTH];
+    typename D::Look lk[2];  // stage t of a row pair uses lk[t & 1]; 2 NS stages per row pair keep the parity fixed
+    if (w0 < w1) lk[0] = D::lookup(rg[0], 0, tbl);
+    for (uint32_t r0 = w0; r0 < w1; r0 += NR) {
 #pragma unroll
-      for (int s = 0; s < DEPTH; s++) {
-        if (r0 + s < w1) {  // wave-uniform
-          slice_stage(stage_g, pg[s], lane);
-          slice_stage(stage_u, pu[s], lane);
-          const uint32_t shg = sg[s], shu = su[s];
-          if (r0 + s + DEPTH < w1) {  // refill the slot: DEPTH row pairs stay in flight
-            const uint8_t *g = row_ptr(r0 + s + DEPTH, 0), *u = row_ptr(r0 + s + DEPTH, 1);
-            pg[s] = slice_load(g, slice_bytes, lane); sg[s] = (uint32_t)((uintptr_t)g & 15u);
-            pu[s] = slice_load(u, slice_bytes, lane); su[s] = (uint32_t)((uintptr_t)u & 15u);
+      for (int half = 0; half < 2; half++) {
+        float acc[NR];  // value 2 j + m: row pair j of this half, m = 0 gate, 1 up
+#pragma unroll
+        for (int j = 0; j < NR / 2; j++) {
+          const int s = half * (NR / 2) + j;
+          const uint32_t row = r0 + s;
+          float g = 0.f, u = 0.f;
+          if (row < w1) {  // wave-uniform; no global loads inside, so the loads in flight stay countable
+            const bool more = row + 1 < w1;
+#pragma unroll
+            for (int t = 0; t < 2 * NS; t++) {
+              const bool up = t >= NS;
+              const int st = up ? t - NS : t;
+              // issue the next stage's table reads, then consume this stage's
+              if (t + 1 < 2 * NS) lk[(t + 1) & 1] = D::lookup(t + 1 >= NS ? ru[s] : rg[s], t + 1 >= NS ? t + 1 - NS : t + 1, tbl);
+              else if (more) lk[0] = D::lookup(rg[(s + 1) % NR], 0, tbl);
+              if (up) { u = D::partial(ru[s], lk[t & 1], xr, st, u); asm volatile("" : "+v"(u)); }
+              else { g = D::partial(rg[s], lk[t & 1], xr, st, g); asm volatile("" : "+v"(g)); }
+            }
           }
-          const typename D::Raw rg = D::load(stage_g + shg, lunit), ru = D::load(stage_u + shu, lunit);
-          const float g = dec_dot<D>(rg, xr, tbl, unit), u = dec_dot<D>(ru, xr, tbl, unit);
-          acc[2 * s] = valid ? g : 0.f;
-          acc[2 * s + 1] = valid ? u : 0.f;
-        } else {
-          acc[2 * s] = 0.f; acc[2 * s + 1] = 0.f;
+          acc[2 * j] = g;
+          acc[2 * j + 1] = u;
+          fetch(s);  // the slot is free again: fetch the row pair NR places ahead
         }
-        asm volatile("" ::: "memory");  // one row pair's table lookups live at a time (register pressure)
-      }
-      row16_fold<2 * DEPTH>(acc, lane);
-      {
-        const uint32_t k = group8_sel<2 * DEPTH>(lane), j = k >> 1, m = k & 1u;
-        if (!(lane & 8u) && r0 + j < w1) part[((r0 + j - c0) * 2 + m) * PSTRIDE + ks * 4 + (lane >> 4)] = acc[0];
+        const uint32_t rb = r0 + half * (NR / 2);
+        if (rb < w1) {
+          row16_fold<NR>(acc, lane);
+          const uint32_t k = group8_sel<NR>(lane), j = k >> 1, m = k & 1u;
+          if (!(lane & 8u) && rb + j < w1) part[((rb + j - c0) * 2 + m) * PSTRIDE + ks * 4 + (lane >> 4)] = acc[0];
+        }
       }
     }
     __syncthreads();
+    // thread q sums the partials of (row q / 2, matrix q % 2); gate and up then meet in the even lane
     for (uint32_t q0 = 0; q0 < 2 * n; q0 += blockDim.x) {
       const uint32_t q = q0 + tid;
       float sum = 0.f;
@@ -259,7 +284,7 @@ __device__ __forceinline__ void moe_gu_run_staged(const MoeArgs& a, uint32_t* sm
 
 template <class D>
 __device__ __forceinline__ void moe_gu_run(const MoeArgs& a, uint32_t* smem, const bool shared, const uint32_t wg) {
-  if constexpr (kStagedGateUp && D::SLICE_BYTES > 0) moe_gu_run_staged<D>(a, smem, shared, wg);
+  if constexpr (requires { D::STAGES; }) moe_gu_run_ring<D>(a, smem, shared, wg);
   else moe_gu_run_direct<D, rows_in_flight<D>(2)>(a, smem, shared, wg);
 }
 
@@ -297,8 +322,9 @@ __global__ __launch_bounds__(1024) void moe_down_kernel(const MoeArgs a) {
   const uint32_t units_r = a.inter / DR::UNIT, units_s = a.inter / DS::UNIT;
   const bool valid_r = NE && u0 < units_r, valid_s = a.run_shared && u0 < units_s;
   const uint32_t unit_r = u0 < units_r ? u0 : units_r - 1, unit_s = u0 < units_s ? u0 : units_s - 1;
-  const uint8_t* Dr = nullptr;
-  if (NE) Dr = a.table ? (const uint8_t*)a.table[3 * e + 2] : a.down[e];
+  gptr_t Dr = nullptr;
+  if (NE) Dr = as_global(a.table ? (const uint8_t*)a.table[3 * e + 2] : a.down[e]);
+  const gptr_t Dsh = as_global(a.sdown);
 
   const uint32_t wg_begin = blockIdx.x * a.rows_per_wg, wg_end = min(a.dim, wg_begin + a.rows_per_wg);
   typename DR::X xr;
@@ -348,8 +374,8 @@ __global__ __launch_bounds__(1024) void moe_down_kernel(const MoeArgs a) {
       // the row-group's waves with K-slice ks take the shared expert's rows w0 + e, w0 + e + E, ...
       for (uint32_t r0 = w0 + e; r0 < w1; r0 += 2 * E) {
         const uint32_t r1 = r0 + E;
-        const typename DS::Raw ra = DS::load(a.sdown + (size_t)r0 * a.rb_d_s, unit_s);
-        const typename DS::Raw rb = DS::load(a.sdown + (size_t)min(r1, w1 - 1) * a.rb_d_s, unit_s);
+        const typename DS::Raw ra = DS::load(Dsh + (size_t)r0 * a.rb_d_s, unit_s);
+        const typename DS::Raw rb = DS::load(Dsh + (size_t)min(r1, w1 - 1) * a.rb_d_s, unit_s);
         const float va = dec_dot<DS>(ra, xs, tbl_s, unit_s), vb = dec_dot<DS>(rb, xs, tbl_s, unit_s);
         float acc[2] = {valid_s ? va : 0.f, valid_s ? vb : 0.f};
         row16_fold<2>(acc, lane);

@@ -125,7 +125,7 @@ int moe_decode_impl(hipStream_t st, const MsqMoeDecodeArgs* p, const MsqBuffer* 
     const int threads = 64 * rw * ks;
     a.ks = (uint32_t)ks;
     a.run_routed = n_gu_r > 0; a.run_shared = gu_s;
-    const size_t part_bytes = (size_t)kMoeChunkRows * 2 * (4 * ks + 1) * 4 + (size_t)(threads / 64) * 2 * kStageBytes;
+    const size_t part_bytes = (size_t)kMoeChunkRows * 2 * (4 * ks + 1) * 4;
     // persistent workgroups, dealt to the routed experts and the shared expert in proportion to their bytes
     const long rows_r = (long)n_gu_r * inter, rows_s = gu_s ? inter : 0;
     const long total = std::max<long>(2, (long)cus * std::max(1, env_gu_wgs));

@@ -14,6 +14,8 @@
 // B fragments; weights stay exact (fp16 payloads, fp32 scales applied to the MFMA result). The K-split partial tiles
 // meet in LDS and are added in wave order, so results do not depend on scheduling.
 #pragma once
+#include <type_traits>
+
 #include "msq_mfma.cuh"
 
 namespace msq {
@@ -38,7 +40,7 @@ struct PfArgs {
 
 constexpr int kPfStageGranules = 3;  // 16-byte granules per thread per matrix the staging path can hold (48 KiB / 1024 threads)
 
-template <class F, bool GU>
+template <class F, bool GU, bool STAGED>
 __global__ __launch_bounds__(1024) void moe_pf_gemm_kernel(const PfArgs a) {
   constexpr int NM = GU ? 2 : 1;
   extern __shared__ __attribute__((aligned(16))) uint32_t smem[];
@@ -59,9 +61,9 @@ __global__ __launch_bounds__(1024) void moe_pf_gemm_kernel(const PfArgs a) {
   const uint32_t e = a.tiles[2 * mt], t0 = a.tiles[2 * mt + 1];
   const uint32_t base = a.offs[e] + t0;                       // first entry (row of A / H / Z) of the token tile
   const uint32_t mtok = min(16u, a.offs[e + 1] - base);
-  const uint8_t* W[NM];
-  if (GU) { W[0] = (const uint8_t*)a.ptrs[3 * e]; W[NM - 1] = (const uint8_t*)a.ptrs[3 * e + 1]; }
-  else W[0] = (const uint8_t*)a.ptrs[3 * e + 2];
+  gptr_t W[NM];
+  if (GU) { W[0] = as_global((const void*)a.ptrs[3 * e]); W[NM - 1] = as_global((const void*)a.ptrs[3 * e + 1]); }
+  else W[0] = as_global((const void*)a.ptrs[3 * e + 2]);
 
   // A fragments of this wave's K steps: token m16 of the tile, chunk q
   uint32_t xa[kMvnMaxSteps][4];
@@ -83,7 +85,7 @@ __global__ __launch_bounds__(1024) void moe_pf_gemm_kernel(const PfArgs a) {
   auto issue = [&](uint32_t tile) {
 #pragma unroll
     for (int m = 0; m < NM; m++) {
-      const uint8_t* start = W[m] + (size_t)tile * tile_bytes;
+      const gptr_t start = W[m] + (size_t)tile * tile_bytes;
       const uint32_t shift = (uint32_t)((uintptr_t)start & 15u);
       // the last tile of a matrix may be short: never read beyond the last row's granule
       const uint32_t rows_here = min(16u, a.N - tile * 16u);
@@ -91,19 +93,19 @@ __global__ __launch_bounds__(1024) void moe_pf_gemm_kernel(const PfArgs a) {
 #pragma unroll
       for (int g = 0; g < kPfStageGranules; g++) {
         const uint32_t gi = tid + g * nthreads;
-        uint4 v = {0u, 0u, 0u, 0u};
-        if (16u * gi < valid) v = *(const uint4*)(start - shift + 16u * gi);
-        pf[m][g] = v;
+        u32x4 v = {0u, 0u, 0u, 0u};
+        if (16u * gi < valid) v = *(const MSQ_GLOBAL u32x4*)(start - shift + 16u * gi);
+        pf[m][g] = uint4{v.x, v.y, v.z, v.w};
       }
     }
   };
-  if (a.staged && tile_first < tile_last) issue(tile_first);
+  if (STAGED && tile_first < tile_last) issue(tile_first);
   __syncthreads();  // tables ready
 
   const uint32_t ones[4] = {0x3C003C00u, 0x3C003C00u, 0x3C003C00u, 0x3C003C00u};
   for (uint32_t tile = tile_first; tile < tile_last; tile++) {
-    const uint8_t* wr[NM];
-    if (a.staged) {
+    std::conditional_t<STAGED, const uint8_t*, gptr_t> wr[NM];
+    if constexpr (STAGED) {
 #pragma unroll
       for (int m = 0; m < NM; m++) {
 #pragma unroll

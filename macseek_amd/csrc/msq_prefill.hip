@@ -33,10 +33,12 @@ int launch_gemm_t(hipStream_t st, PfArgs a, int cus) {
   a.nchunks = (ntile_rows + a.chunk_tiles - 1) / a.chunk_tiles;
   static bool attr_set = false;  // per instantiation: allow more than 64 KiB of dynamic LDS
   if (!attr_set) {
-    MSQ_HIP(hipFuncSetAttribute((const void*)moe_pf_gemm_kernel<F, GU>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+    MSQ_HIP(hipFuncSetAttribute((const void*)moe_pf_gemm_kernel<F, GU, true>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+    MSQ_HIP(hipFuncSetAttribute((const void*)moe_pf_gemm_kernel<F, GU, false>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
     attr_set = true;
   }
-  hipLaunchKernelGGL((moe_pf_gemm_kernel<F, GU>), dim3(a.ntiles * a.nchunks), dim3(threads), lds, st, a);
+  if (a.staged) hipLaunchKernelGGL((moe_pf_gemm_kernel<F, GU, true>), dim3(a.ntiles * a.nchunks), dim3(threads), lds, st, a);
+  else hipLaunchKernelGGL((moe_pf_gemm_kernel<F, GU, false>), dim3(a.ntiles * a.nchunks), dim3(threads), lds, st, a);
   MSQ_HIP(hipGetLastError());
   return MSQ_OK;
 }
