@@ -336,14 +336,20 @@ struct DecIQ1S {
     return k;
   }
   __device__ static float partial(const Raw& r, const Look& k, const X& x, int, float) {
-    float acc = 0.f;
+    // two interleaved chains: a dependent dot2 issues every 8 cycles, an independent one every 4
+    float acc = 0.f, acc1 = 0.f;
 #pragma unroll
-    for (int l = 0; l < 4; l++) {
+    for (int l = 0; l < 4; l += 2) {
       acc = dot2(k.g[l].x, x.v[4 * l + 0], acc);
+      acc1 = dot2(k.g[l + 1].x, x.v[4 * l + 4], acc1);
       acc = dot2(k.g[l].y, x.v[4 * l + 1], acc);
+      acc1 = dot2(k.g[l + 1].y, x.v[4 * l + 5], acc1);
       acc = dot2(k.g[l].z, x.v[4 * l + 2], acc);
+      acc1 = dot2(k.g[l + 1].z, x.v[4 * l + 6], acc1);
       acc = dot2(k.g[l].w, x.v[4 * l + 3], acc);
+      acc1 = dot2(k.g[l + 1].w, x.v[4 * l + 7], acc1);
     }
+    acc += acc1;
     const float dl = half_bits_to_float(r.d) * (float)(2u * ((r.qh >> 12) & 7u) + 1u);
     const float delta = (r.qh & 0x8000u) ? -0.125f : 0.125f;
     return dl * (acc + delta * x.sx);
@@ -413,14 +419,19 @@ struct DecIQ2XXS {
     return k;
   }
   __device__ static float partial(const Raw& r, const Look& k, const X& x, int stage, float acc) {
-#pragma unroll
-    for (int i = 0; i < 2; i++) {
-      const int l = 2 * stage + i;
-      acc = dot2(k.g[i].x ^ k.s[i].x, x.v[4 * l + 0], acc);
-      acc = dot2(k.g[i].y ^ k.s[i].y, x.v[4 * l + 1], acc);
-      acc = dot2(k.g[i].z ^ k.s[i].z, x.v[4 * l + 2], acc);
-      acc = dot2(k.g[i].w ^ k.s[i].w, x.v[4 * l + 3], acc);
+    float acc1 = 0.f;  // second chain: dependent dot2s issue at half rate
+    {
+      const int l = 2 * stage;
+      acc = dot2(k.g[0].x ^ k.s[0].x, x.v[4 * l + 0], acc);
+      acc1 = dot2(k.g[1].x ^ k.s[1].x, x.v[4 * l + 4], acc1);
+      acc = dot2(k.g[0].y ^ k.s[0].y, x.v[4 * l + 1], acc);
+      acc1 = dot2(k.g[1].y ^ k.s[1].y, x.v[4 * l + 5], acc1);
+      acc = dot2(k.g[0].z ^ k.s[0].z, x.v[4 * l + 2], acc);
+      acc1 = dot2(k.g[1].z ^ k.s[1].z, x.v[4 * l + 6], acc1);
+      acc = dot2(k.g[0].w ^ k.s[0].w, x.v[4 * l + 3], acc);
+      acc1 = dot2(k.g[1].w ^ k.s[1].w, x.v[4 * l + 7], acc1);
     }
+    acc += acc1;
     if (stage == 1) acc *= half_bits_to_float(r.d) * (0.5f + (float)(r.a1 >> 28)) * 0.25f;
     return acc;
   }

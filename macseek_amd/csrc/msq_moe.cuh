@@ -16,6 +16,12 @@
 #ifndef MSQ_EXP
 #define MSQ_EXP 0
 #endif
+#ifndef MSQ_NR
+#define MSQ_NR 4
+#endif
+#ifndef MSQ_NRD
+#define MSQ_NRD 4
+#endif
 
 namespace msq {
 
@@ -169,7 +175,7 @@ __device__ __forceinline__ void moe_gu_run_direct(const MoeArgs& a, uint32_t* sm
 // products (two alternating lookup buffers), so LDS latency overlaps the math as well.
 template <class D>
 __device__ __forceinline__ void moe_gu_run_ring(const MoeArgs& a, uint32_t* smem, const bool shared, const uint32_t wg) {
-  constexpr int NR = 8;  // row pairs in flight per wave
+  constexpr int NR = MSQ_NR;  // row pairs in flight per wave
   constexpr int NS = D::STAGES;
   uint32_t* tbl = smem;
   float* part = (float*)(smem + D::LDS_WORDS);
@@ -191,6 +197,16 @@ __device__ __forceinline__ void moe_gu_run_ring(const MoeArgs& a, uint32_t* smem
 
   typename D::X xr;
   bool first = true;
+#if MSQ_EXP == 5
+  return;
+#endif
+#if MSQ_EXP == 6
+  D::fill_lds(tbl, (int)tid, (int)blockDim.x);
+  xr = D::load_x(a.x, unit);
+  __syncthreads();
+  if (xr.sx == 1.2345f) a.h[0] = tbl[tid];
+  return;
+#endif
   for (uint32_t c0 = wg_begin; c0 < wg_end; c0 += kMoeChunkRows) {
     const uint32_t c1 = min(wg_end, c0 + kMoeChunkRows), n = c1 - c0;
     const uint32_t run = uniform((n + RW - 1) / RW);  // divisions run on the vector unit: bring the results back
@@ -227,6 +243,12 @@ __device__ __forceinline__ void moe_gu_run_ring(const MoeArgs& a, uint32_t* smem
       __syncthreads();
       first = false;
     }
+#if MSQ_EXP == 7
+    { uint32_t sm_ = 0;
+      for (int s_ = 0; s_ < NR; s_++) { uint32_t w_[sizeof(typename D::Raw) / 4]; __builtin_memcpy(w_, &rg[s_], sizeof(w_)); sm_ += w_[0]; __builtin_memcpy(w_, &ru[s_], sizeof(w_)); sm_ += w_[0]; }
+      if (sm_ == 0x12345u && xr.sx == 1.2345f) a.h[0] = 1.f;
+      return; }
+#endif
     typename D::Look lk[2];  // stage t of a row pair uses lk[t & 1]; 2 NS stages per row pair keep the parity fixed
     if (w0 < w1) lk[0] = D::lookup(rg[0], 0, tbl);
     for (uint32_t r0 = w0; r0 < w1; r0 += NR) {
@@ -296,11 +318,60 @@ __global__ __launch_bounds__(1024) void moe_gu_kernel(const MoeArgs a) {
 }
 
 // down: workgroup = RW row-groups x (NE expert-waves x KS K-split waves). In a row-group, wave (e, ks) owns routed
-// expert e's K-slice ks of the row-group's rows; afterwards the same waves share out the shared expert's rows.
-// Per row the partial sums are added in the fixed order (expert 0 ks 0.., expert 1 .., shared ks 0..).
+// expert e's K-slice ks of the row-group's rows; the shared expert's rows are dealt over the same waves (wave e takes
+// rows e, e + E, ...). Per row the partial sums are added in the fixed order (expert 0 ks 0.., expert 1 .., shared ks 0..).
+// Codebook decoders stream their rows through register rings of range-checked buffer loads (see moe_gu_run_ring): the
+// first rows of both the routed and the shared matrix are requested before the tables and activations are staged.
+template <class D, int NR, class F>
+__device__ __forceinline__ void down_rows_ring(const uint32_t* tbl, const typename D::X& x, const uint32_t lane, uint32_t first,
+                                                const uint32_t step, const uint32_t end, typename D::Raw (&ring)[NR], F&& fetch,
+                                                float* part_col, const uint32_t pstride, const uint32_t c0) {
+  // rows first, first + step, ... < end; ring[s] already holds row first + s * step; fetch(s) refills slot s
+  constexpr int NS = D::STAGES;
+  typename D::Look lk[2];
+  if (first < end) lk[0] = D::lookup(ring[0], 0, tbl);
+  for (uint32_t r0 = first; r0 < end; r0 += NR * step) {
+#pragma unroll
+    for (int half = 0; half < NR / 4; half++) {
+      float acc[4];
+#pragma unroll
+      for (int j = 0; j < 4; j++) {
+        const int s = half * 4 + j;
+        const uint32_t row = r0 + s * step;
+        float v = 0.f;
+#if MSQ_EXP == 12
+        if (row < end) { uint32_t w_[sizeof(typename D::Raw) / 4]; __builtin_memcpy(w_, &ring[s], sizeof(w_)); v = (float)(w_[0] + w_[1]); }
+        else
+#endif
+        if (row < end) {  // wave-uniform; no global loads inside
+          const bool more = row + step < end;
+#pragma unroll
+          for (int t = 0; t < NS; t++) {
+            const int cur = (s * NS + t) & 1;
+            if (t + 1 < NS) lk[cur ^ 1] = D::lookup(ring[s], t + 1, tbl);
+            else if (more) lk[cur ^ 1] = D::lookup(ring[(s + 1) % NR], 0, tbl);
+            v = D::partial(ring[s], lk[cur], x, t, v);
+            asm volatile("" : "+v"(v));
+          }
+        }
+        acc[j] = v;
+        fetch(s);
+      }
+      const uint32_t rb = r0 + half * 4 * step;
+      if (rb < end) {
+        row16_fold<4>(acc, lane);
+        const uint32_t r = rb + group8_sel<4>(lane) * step;
+        if (!(lane & 8u) && r < end) part_col[(r - c0) * pstride + (lane >> 4)] = acc[0];
+      }
+    }
+  }
+}
+
 template <class DR, class DS>
 __global__ __launch_bounds__(1024) void moe_down_kernel(const MoeArgs a) {
+  constexpr bool RING_R = requires { DR::STAGES; }, RING_S = requires { DS::STAGES; };
   constexpr int RPW = rows_in_flight<DR>(1);
+  constexpr int NR = MSQ_NRD, NSH = 4;  // ring depth: routed rows, shared rows
   extern __shared__ __attribute__((aligned(16))) uint32_t smem[];
   constexpr int TBL = DR::LDS_WORDS + DS::LDS_WORDS;
   uint32_t* tbl_r = smem;
@@ -313,8 +384,8 @@ __global__ __launch_bounds__(1024) void moe_down_kernel(const MoeArgs a) {
   const uint32_t NE = a.run_routed ? a.n_routed : 0u;       // routed experts computed here
   const uint32_t E = max(NE, 1u);
   const uint32_t wpg = E * KS;                              // waves per row-group
-  const uint32_t RW = nwaves / wpg, rg = wave / wpg, wl = wave % wpg;
-  const uint32_t e = wl / KS, ks = wl % KS;
+  const uint32_t RW = nwaves / wpg, rg = uniform(wave / wpg), wl = uniform(wave % wpg);
+  const uint32_t e = uniform(wl / KS), ks = uniform(wl % KS);
   const uint32_t slots = 4 * (NE * KS + (a.run_shared ? KS : 0u));  // partial sums per row: 4 per contributing wave
   const uint32_t PSTRIDE = slots + 1;
 
@@ -322,9 +393,12 @@ __global__ __launch_bounds__(1024) void moe_down_kernel(const MoeArgs a) {
   const uint32_t units_r = a.inter / DR::UNIT, units_s = a.inter / DS::UNIT;
   const bool valid_r = NE && u0 < units_r, valid_s = a.run_shared && u0 < units_s;
   const uint32_t unit_r = u0 < units_r ? u0 : units_r - 1, unit_s = u0 < units_s ? u0 : units_s - 1;
-  gptr_t Dr = nullptr;
-  if (NE) Dr = as_global(a.table ? (const uint8_t*)a.table[3 * e + 2] : a.down[e]);
-  const gptr_t Dsh = as_global(a.sdown);
+  const void* Dr_ = nullptr;
+  if (NE) Dr_ = uniform(a.table ? (const void*)a.table[3 * e + 2] : (const void*)a.down[e]);
+  const gptr_t Dr = as_global(Dr_), Dsh = as_global(a.sdown);
+
+  const auto off_r = [&] { if constexpr (RING_R) return DR::offsets(unit_r); else return 0; }();
+  const auto off_s = [&] { if constexpr (RING_S) return DS::offsets(unit_s); else return 0; }();
 
   const uint32_t wg_begin = blockIdx.x * a.rows_per_wg, wg_end = min(a.dim, wg_begin + a.rows_per_wg);
   typename DR::X xr;
@@ -332,55 +406,99 @@ __global__ __launch_bounds__(1024) void moe_down_kernel(const MoeArgs a) {
   bool first = true;
   for (uint32_t c0 = wg_begin; c0 < wg_end; c0 += kMoeChunkRows) {
     const uint32_t c1 = min(wg_end, c0 + kMoeChunkRows), n = c1 - c0;
-    const uint32_t run = (n + RW - 1) / RW;
-    const uint32_t w0 = min(c0 + rg * run, c1), w1 = min(w0 + run, c1);
-    typename DR::Raw cur[RPW], nxt[RPW];
-    if (NE && w0 < w1) {
+    const uint32_t run = uniform((n + RW - 1) / RW);
+    const uint32_t w0 = uniform(min(c0 + rg * run, c1)), w1 = uniform(min(w0 + run, c1));
+
+    // ---- request the first rows of both matrices
+    typename DR::Raw cur[RING_R ? 1 : RPW], nxt[RING_R ? 1 : RPW];
+    uint32_t pv = w0;  // routed ring cursor
+    typename DR::Raw rr[NR];
+    typename DS::Raw rs[NSH];
+    uint32_t sv = w0 + e;  // shared ring cursor
+    auto fetch_r = [&](int s) {
+      if constexpr (RING_R) {
+        rr[s] = DR::fetch(make_rsrc(Dr_, (NE && pv < w1) ? a.dim * a.rb_d_r : 0u), off_r, pv * a.rb_d_r);
+        pv++;
+      }
+    };
+    auto fetch_s = [&](int s) {
+      if constexpr (RING_S) {
+        rs[s] = DS::fetch(make_rsrc(a.sdown, (a.run_shared && sv < w1) ? a.dim * a.rb_d_s : 0u), off_s, sv * a.rb_d_s);
+        sv += E;
+      }
+    };
+    if constexpr (RING_R) {
+#pragma unroll
+      for (int s = 0; s < NR; s++) fetch_r(s);
+    } else if (NE && w0 < w1) {
 #pragma unroll
       for (int j = 0; j < RPW; j++) cur[j] = DR::load(Dr + (size_t)min(w0 + j, w1 - 1) * a.rb_d_r, unit_r);
     }
+    if constexpr (RING_S) {
+#pragma unroll
+      for (int s = 0; s < NSH; s++) fetch_s(s);
+    }
     if (first) {
-      if (NE) { DR::fill_lds(tbl_r, (int)tid, (int)blockDim.x); xr = DR::load_x(a.h + (size_t)e * a.inter, unit_r); }
-      if (a.run_shared) { DS::fill_lds(tbl_s, (int)tid, (int)blockDim.x); xs = DS::load_x(a.h + (size_t)a.n_routed * a.inter, unit_s); }
+      if (NE) {
+        DR::fill_lds(tbl_r, (int)tid, (int)blockDim.x);
+        xr = DR::load_x(a.h + (size_t)e * a.inter, unit_r);
+        if (!valid_r) xr = typename DR::X{};
+      }
+      if (a.run_shared) {
+        DS::fill_lds(tbl_s, (int)tid, (int)blockDim.x);
+        xs = DS::load_x(a.h + (size_t)a.n_routed * a.inter, unit_s);
+        if (!valid_s) xs = typename DS::X{};
+      }
       __syncthreads();
       first = false;
     }
+#if MSQ_EXP == 11
+    if (xr.sx == 1.2345f) a.y[0] = 1.f;
+    return;
+#endif
+    // ---- routed expert e, rows w0 .. w1
     if (NE) {
-      for (uint32_t r0 = w0; r0 < w1; r0 += RPW) {
-        const bool more = r0 + RPW < w1;
-        if (more) {
+      if constexpr (RING_R) {
+        down_rows_ring<DR, NR>(tbl_r, xr, lane, w0, 1u, w1, rr, fetch_r, part + 4 * (e * KS + ks), PSTRIDE, c0);
+      } else {
+        for (uint32_t r0 = w0; r0 < w1; r0 += RPW) {
+          const bool more = r0 + RPW < w1;
+          if (more) {
 #pragma unroll
-          for (int j = 0; j < RPW; j++) nxt[j] = DR::load(Dr + (size_t)min(r0 + RPW + j, w1 - 1) * a.rb_d_r, unit_r);
-        }
-        float acc[RPW];
+            for (int j = 0; j < RPW; j++) nxt[j] = DR::load(Dr + (size_t)min(r0 + RPW + j, w1 - 1) * a.rb_d_r, unit_r);
+          }
+          float acc[RPW];
 #pragma unroll
-        for (int j = 0; j < RPW; j++) {
-          const float v = dec_dot<DR>(cur[j], xr, tbl_r, unit_r);
-          acc[j] = valid_r ? v : 0.f;
-          asm volatile("" ::: "memory");
-        }
-        row16_fold<RPW>(acc, lane);
-        {
-          const uint32_t j = group8_sel<RPW>(lane);
-          if (!(lane & 8u) && r0 + j < w1) part[(r0 + j - c0) * PSTRIDE + 4 * (e * KS + ks) + (lane >> 4)] = acc[0];
-        }
-        if (more) {
+          for (int j = 0; j < RPW; j++) {
+            acc[j] = dec_dot<DR>(cur[j], xr, tbl_r, unit_r);  // lanes past the row hold zero activations
+            asm volatile("" ::: "memory");
+          }
+          row16_fold<RPW>(acc, lane);
+          {
+            const uint32_t j = group8_sel<RPW>(lane);
+            if (!(lane & 8u) && r0 + j < w1) part[(r0 + j - c0) * PSTRIDE + 4 * (e * KS + ks) + (lane >> 4)] = acc[0];
+          }
+          if (more) {
 #pragma unroll
-          for (int j = 0; j < RPW; j++) cur[j] = nxt[j];
+            for (int j = 0; j < RPW; j++) cur[j] = nxt[j];
+          }
         }
       }
     }
+    // ---- shared expert: the row-group's waves with K-slice ks take rows w0 + e, w0 + e + E, ...
     if (a.run_shared) {
-      // the row-group's waves with K-slice ks take the shared expert's rows w0 + e, w0 + e + E, ...
-      for (uint32_t r0 = w0 + e; r0 < w1; r0 += 2 * E) {
-        const uint32_t r1 = r0 + E;
-        const typename DS::Raw ra = DS::load(Dsh + (size_t)r0 * a.rb_d_s, unit_s);
-        const typename DS::Raw rb = DS::load(Dsh + (size_t)min(r1, w1 - 1) * a.rb_d_s, unit_s);
-        const float va = dec_dot<DS>(ra, xs, tbl_s, unit_s), vb = dec_dot<DS>(rb, xs, tbl_s, unit_s);
-        float acc[2] = {valid_s ? va : 0.f, valid_s ? vb : 0.f};
-        row16_fold<2>(acc, lane);
-        const uint32_t r = group8_sel<2>(lane) ? r1 : r0;
-        if (!(lane & 8u) && r < w1) part[(r - c0) * PSTRIDE + 4 * (NE * KS + ks) + (lane >> 4)] = acc[0];
+      if constexpr (RING_S) {
+        down_rows_ring<DS, NSH>(tbl_s, xs, lane, w0 + e, E, w1, rs, fetch_s, part + 4 * (NE * KS + ks), PSTRIDE, c0);
+      } else {
+        for (uint32_t r0 = w0 + e; r0 < w1; r0 += 2 * E) {
+          const uint32_t r1 = r0 + E;
+          const typename DS::Raw ra = DS::load(Dsh + (size_t)r0 * a.rb_d_s, unit_s);
+          const typename DS::Raw rb = DS::load(Dsh + (size_t)min(r1, w1 - 1) * a.rb_d_s, unit_s);
+          float acc[2] = {dec_dot<DS>(ra, xs, tbl_s, unit_s), dec_dot<DS>(rb, xs, tbl_s, unit_s)};
+          row16_fold<2>(acc, lane);
+          const uint32_t r = group8_sel<2>(lane) ? r1 : r0;
+          if (!(lane & 8u) && r < w1) part[(r - c0) * PSTRIDE + 4 * (NE * KS + ks) + (lane >> 4)] = acc[0];
+        }
       }
     }
     __syncthreads();
