@@ -16,6 +16,9 @@
 #ifndef MSQ_EXP
 #define MSQ_EXP 0
 #endif
+#ifndef MSQ_NOPIPE
+#define MSQ_NOPIPE 0
+#endif
 #ifndef MSQ_NR
 #define MSQ_NR 4
 #endif
@@ -250,7 +253,9 @@ __device__ __forceinline__ void moe_gu_run_ring(const MoeArgs& a, uint32_t* smem
       return; }
 #endif
     typename D::Look lk[2];  // stage t of a row pair uses lk[t & 1]; 2 NS stages per row pair keep the parity fixed
+#if !MSQ_NOPIPE
     if (w0 < w1) lk[0] = D::lookup(rg[0], 0, tbl);
+#endif
     for (uint32_t r0 = w0; r0 < w1; r0 += NR) {
 #pragma unroll
       for (int half = 0; half < 2; half++) {
@@ -267,8 +272,13 @@ __device__ __forceinline__ void moe_gu_run_ring(const MoeArgs& a, uint32_t* smem
               const bool up = t >= NS;
               const int st = up ? t - NS : t;
               // issue the next stage's table reads, then consume this stage's
+#if MSQ_NOPIPE
+              lk[t & 1] = D::lookup(up ? ru[s] : rg[s], st, tbl);
+              (void)more;
+#else
               if (t + 1 < 2 * NS) lk[(t + 1) & 1] = D::lookup(t + 1 >= NS ? ru[s] : rg[s], t + 1 >= NS ? t + 1 - NS : t + 1, tbl);
               else if (more) lk[0] = D::lookup(rg[(s + 1) % NR], 0, tbl);
+#endif
               if (up) { u = D::partial(ru[s], lk[t & 1], xr, st, u); asm volatile("" : "+v"(u)); }
               else { g = D::partial(rg[s], lk[t & 1], xr, st, g); asm volatile("" : "+v"(g)); }
             }
