@@ -211,4 +211,67 @@ struct FragDense16 {
   }
 };
 
+// ================================================================================================ block fragments
+// For the 256-weight codebook formats the large-token GEMM uses a second decomposition: weight = block_scale * n with
+// n a small integer (or a multiple of 1/8) that fp16 holds exactly -- the sub-block factor (2 s + 1) is folded into the
+// payload. A wave then accumulates a whole 256-column block in the matrix cores and applies the fp32 block scale once
+// per block instead of once per K step. Lane (row n, chunk q) owns the sub-blocks 2 q and 2 q + 1 of its row's block
+// (16 contiguous bytes of IQ2_XXS), so no lane loads a byte twice; step j (0..7) of a block therefore covers, for chunk
+// q, the 8 columns col_of(q, j) .. + 7 of the block, and the activation operand is read with the same mapping.
+//   Raw / load(block pointer, q)    the lane's bytes of one block
+//   scale(raw)                      fp32 block scale
+//   frag(raw, j, tbl, h)            payloads of step j
+__device__ __forceinline__ uint32_t pk_mul_f16(uint32_t a, uint32_t b) {
+  const h2_t r = as_h2(a) * as_h2(b);
+  return __builtin_bit_cast(uint32_t, r);
+}
+// both halves = (fp16)v for an integer 0 <= v < 1024, without a conversion: 0x6400 | v is 1024 + v
+__device__ __forceinline__ uint32_t pk_small_int_f16(uint32_t v) {
+  return pk_add_f16(0x64006400u | v | (v << 16), 0xE400E400u);
+}
+__device__ __forceinline__ uint32_t blk_col_of(uint32_t q, uint32_t j) { return 64u * q + 32u * (j >> 2) + 8u * (j & 3u); }
+
+struct BlkIQ2XXS {
+  static constexpr int LDS_WORDS = FragIQ2XXS::LDS_WORDS, BLOCK_BYTES = 66;
+  __device__ static void fill_lds(uint32_t* lds, int tid, int nt) { FragIQ2XXS::fill_lds(lds, tid, nt); }
+  struct Raw { uint32_t w[4]; uint32_t d; };  // {a0, a1} of sub-block 2 q, then of 2 q + 1; fp16 bits of d
+  template <class P>
+  __device__ static Raw load(P blk, uint32_t q) {
+    const u128_a2 v = ld128(blk + 2 + 16 * q);
+    return {{v.x, v.y, v.z, v.w}, ld16(blk)};
+  }
+  __device__ static float scale(const Raw& r) { return half_bits_to_float(r.d) * 0.125f; }  // db = d (2 s + 1) / 8
+  __device__ static void frag(const Raw& r, int j, const uint32_t* tbl, uint32_t (&h)[4]) {
+    const uint32_t a0 = r.w[2 * (j >> 2)], a1 = r.w[2 * (j >> 2) + 1];
+    const int l = j & 3;
+    const uint4 g = ((const uint4*)tbl)[(a0 >> (8 * l)) & 0xFFu];
+    const uint4 s = ((const uint4*)(tbl + MSQ_IQ2XXS_GRID_N * 4))[(a1 >> (7 * l)) & 127u];
+    const uint32_t m2 = pk_small_int_f16(((a1 >> 27) & 0x1Eu) | 1u);  // 2 s + 1 <= 31; grid <= 43: products are exact
+    h[0] = pk_mul_f16(g.x ^ s.x, m2); h[1] = pk_mul_f16(g.y ^ s.y, m2);
+    h[2] = pk_mul_f16(g.z ^ s.z, m2); h[3] = pk_mul_f16(g.w ^ s.w, m2);
+  }
+};
+
+struct BlkIQ1S {
+  static constexpr int LDS_WORDS = FragIQ1S::LDS_WORDS, BLOCK_BYTES = 50;
+  __device__ static void fill_lds(uint32_t* lds, int tid, int nt) { FragIQ1S::fill_lds(lds, tid, nt); }
+  struct Raw { uint32_t qs[2]; uint32_t qh; uint32_t d; };  // qs bytes 8 q .. 8 q + 7; qh[2 q] | qh[2 q + 1] << 16
+  template <class P>
+  __device__ static Raw load(P blk, uint32_t q) {
+    const u64_a2 v = ld64(blk + 2 + 8 * q);
+    return {{v.x, v.y}, ld32(blk + 34 + 4 * q), ld16(blk)};
+  }
+  __device__ static float scale(const Raw& r) { return half_bits_to_float(r.d); }  // w = d (2 s + 1) (g + delta)
+  __device__ static void frag(const Raw& r, int j, const uint32_t* tbl, uint32_t (&h)[4]) {
+    const uint32_t qs = r.qs[j >> 2], qh = (j >> 2) ? r.qh >> 16 : r.qh & 0xFFFFu;
+    const int l = j & 3;
+    const uint32_t idx = ((qs >> (8 * l)) & 0xFFu) | (((qh >> (3 * l)) & 7u) << 8);
+    const uint4 g = ((const uint4*)tbl)[idx];
+    const uint32_t d2 = (qh & 0x8000u) ? 0xB000B000u : 0x30003000u;          // -+ 1/8 in both halves
+    const uint32_t m2 = pk_small_int_f16(((qh >> 11) & 0xEu) | 1u);          // 2 s + 1 <= 15; |g + delta| <= 9/8
+    h[0] = pk_mul_f16(pk_add_f16(g.x, d2), m2); h[1] = pk_mul_f16(pk_add_f16(g.y, d2), m2);
+    h[2] = pk_mul_f16(pk_add_f16(g.z, d2), m2); h[3] = pk_mul_f16(pk_add_f16(g.w, d2), m2);
+  }
+};
+
 }  // namespace msq

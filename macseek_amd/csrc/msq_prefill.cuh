@@ -177,6 +177,158 @@ __global__ __launch_bounds__(1024) void moe_pf_gemm_kernel(const PfArgs a) {
   }
 }
 
+// ------------------------------------------------------------------------------------------------ block GEMM
+// Grouped GEMM for the 256-weight codebook formats (block fragments, see msq_mfma.cuh). A work item is one expert's
+// block of up to 64 entries (token tiles t < T <= 4) times a chunk of weight rows; the item's 8 waves own different
+// weight-row tiles and walk K block by block (256 columns): the activation block [64][256] fp16 is staged in LDS for
+// all waves (double-buffered, one barrier per block), every wave decodes the fragments of its own rows once per block
+// and reuses each of them for all T token tiles, accumulates the block in the matrix cores and applies the fp32 block
+// scale once. Weights are decoded exactly once per (item, row): no lane loads a weight byte twice.
+struct PfBlkArgs {
+  const uint16_t* A;        // fp16 activations [entries][K]
+  const uint64_t* ptrs;     // per expert: gate, up, down addresses
+  const uint32_t* offs;     // per expert: first entry
+  const uint32_t* items;    // per item: expert, first entry of the block inside the expert, entries in the block
+  const float* wt;          // per routed entry: routing weight
+  uint16_t* H;              // gate/up output [entries][N] fp16
+  float* Z;                 // down output [entries][N] fp32
+  uint32_t nitems, total;
+  uint32_t K, N, row_bytes, nblocks;
+  uint32_t row_chunks;      // chunks of 8 * RT * 16 weight rows
+};
+
+constexpr int kPfBlkTokens = 64, kPfBlkThreads = 512, kPfBlkPitch = 256 * 2 + 16;
+constexpr int kPfBlkRowsGU = 8 * 2 * 16, kPfBlkRowsDown = 8 * 4 * 16;  // weight rows per work item
+
+template <class B, bool GU>
+__global__ __launch_bounds__(kPfBlkThreads) void moe_pf_block_kernel(const PfBlkArgs a) {
+  constexpr int NM = GU ? 2 : 1, RT = GU ? 2 : 4, R = RT * NM, TMAX = kPfBlkTokens / 16, PITCH = kPfBlkPitch;
+  extern __shared__ __attribute__((aligned(16))) uint32_t smem[];
+  uint32_t* tbl = smem;
+  uint8_t* abuf = (uint8_t*)(smem + B::LDS_WORDS);  // [2][64 tokens][PITCH]
+  const uint32_t tid = threadIdx.x, lane = tid & 63u;
+  const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
+  const uint32_t n16 = lane & 15u, q = lane >> 4;
+
+  // consecutive workgroups land on different XCDs: the row chunks of one item stay on one XCD (shared L2 for its
+  // activations), and items -- sorted by size -- are dealt round-robin over the XCDs
+  const uint32_t xcd = blockIdx.x & 7u, slot = blockIdx.x >> 3;
+  const uint32_t item = (slot / a.row_chunks) * 8u + xcd, rc = slot % a.row_chunks;
+  if (item >= a.nitems) return;
+  const uint32_t e = a.items[3 * item], t0 = a.items[3 * item + 1], cnt = a.items[3 * item + 2];
+  const uint32_t base = a.offs[e] + t0;
+  const uint32_t T = (cnt + 15u) / 16u;
+
+  gptr_t wrow[R];
+  uint32_t row_of[RT];
+#pragma unroll
+  for (int jt = 0; jt < RT; jt++) {
+    row_of[jt] = ((rc * 8u + wave) * RT + jt) * 16u + n16;
+    const uint32_t row = min(row_of[jt], a.N - 1);
+#pragma unroll
+    for (int m = 0; m < NM; m++)
+      wrow[jt * NM + m] = as_global((const void*)a.ptrs[3 * e + (GU ? m : 2)]) + (size_t)row * a.row_bytes;
+  }
+
+  // activation chunk loader: thread owns granule (token 16 i + tid / 32, 16-byte column tid % 32) of every token tile
+  const uint32_t atok = tid >> 5, acol = tid & 31u;
+  uint4 pa[TMAX];
+  auto a_issue = [&](uint32_t kc) {
+#pragma unroll
+    for (int i = 0; i < TMAX; i++) {
+      const uint32_t tok = 16u * i + atok;
+      pa[i] = uint4{0u, 0u, 0u, 0u};
+      if (tok < cnt) pa[i] = *(const uint4*)(a.A + (size_t)(base + tok) * a.K + kc * 256u + acol * 8u);
+    }
+  };
+  auto a_store = [&](uint32_t buf) {
+#pragma unroll
+    for (int i = 0; i < TMAX; i++)
+      if ((uint32_t)i < T) *(uint4*)(abuf + buf * (kPfBlkTokens * PITCH) + (16u * i + atok) * PITCH + acol * 16u) = pa[i];
+  };
+
+  typename B::Raw cur[R], nxt[R];
+#pragma unroll
+  for (int r = 0; r < R; r++) cur[r] = B::load(wrow[r], q);
+  a_issue(0);
+  B::fill_lds(tbl, (int)tid, (int)blockDim.x);
+  a_store(0);
+  __syncthreads();
+
+  f4_t acc[TMAX][R];
+#pragma unroll
+  for (int t = 0; t < TMAX; t++)
+#pragma unroll
+    for (int r = 0; r < R; r++) acc[t][r] = f4_t{0.f, 0.f, 0.f, 0.f};
+
+  for (uint32_t kc = 0; kc < a.nblocks; kc++) {
+    const uint32_t buf = kc & 1u;
+    const bool more = kc + 1 < a.nblocks;
+    if (more) {
+#pragma unroll
+      for (int r = 0; r < R; r++) nxt[r] = B::load(wrow[r] + (size_t)(kc + 1) * B::BLOCK_BYTES, q);
+      a_issue(kc + 1);
+    }
+    f4_t blk[TMAX][R];
+#pragma unroll
+    for (int t = 0; t < TMAX; t++)
+#pragma unroll
+      for (int r = 0; r < R; r++) blk[t][r] = f4_t{0.f, 0.f, 0.f, 0.f};
+    const uint8_t* arow = abuf + buf * (kPfBlkTokens * PITCH) + n16 * PITCH;
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+      uint32_t h[R][4];
+#pragma unroll
+      for (int r = 0; r < R; r++) B::frag(cur[r], j, tbl, h[r]);
+#pragma unroll
+      for (int t = 0; t < TMAX; t++) {
+        if ((uint32_t)t < T) {  // wave-uniform
+          const uint4 av = *(const uint4*)(arow + t * 16 * PITCH + 2u * blk_col_of(q, j));
+          const uint32_t af[4] = {av.x, av.y, av.z, av.w};
+#pragma unroll
+          for (int r = 0; r < R; r++) blk[t][r] = mfma_f16(af, h[r], blk[t][r]);
+        }
+      }
+    }
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+      const float sc = B::scale(cur[r]);
+#pragma unroll
+      for (int t = 0; t < TMAX; t++)
+        if ((uint32_t)t < T) acc[t][r] += sc * blk[t][r];
+    }
+    if (more) {
+      a_store(buf ^ 1u);
+#pragma unroll
+      for (int r = 0; r < R; r++) cur[r] = nxt[r];
+    }
+    __syncthreads();
+  }
+
+#pragma unroll
+  for (int t = 0; t < TMAX; t++) {
+    if ((uint32_t)t >= T) continue;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      const uint32_t tok = 16u * t + 4u * q + i;
+      if (tok >= cnt) continue;
+      const uint32_t entry = base + tok;
+#pragma unroll
+      for (int jt = 0; jt < RT; jt++) {
+        if (row_of[jt] >= a.N) continue;
+        if constexpr (GU) {
+          const float g = fminf(acc[t][2 * jt][i], 10.f), u = fminf(fmaxf(acc[t][2 * jt + 1][i], -10.f), 10.f);
+          const float w = entry < a.total ? a.wt[entry] : 1.f;
+          const float hv = g / (1.f + expf(-g)) * u * w;
+          a.H[(size_t)entry * a.N + row_of[jt]] = __builtin_bit_cast(uint16_t, (_Float16)hv);
+        } else {
+          a.Z[(size_t)entry * a.N + row_of[jt]] = acc[t][jt][i];
+        }
+      }
+    }
+  }
+}
+
 // Xg[i] = fp16(X[src(i)]): i < total gathers token tok[i]; rows total .. total + n - 1 are the tokens themselves
 template <bool X_BF16>
 __global__ __launch_bounds__(256) void moe_pf_gather_kernel(const void* __restrict__ X, uint16_t* __restrict__ Xg,

@@ -1,5 +1,6 @@
 // C ABI: prefill MoE (see include/msq.h; reference host code src/kernels/quant.mm:372-612).
 #include <algorithm>
+#include <array>
 #include <cstdlib>
 #include <vector>
 
@@ -12,7 +13,8 @@ namespace {
 size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
 size_t header_bytes(int total, int n, int n_exp) {
   const size_t tiles = (size_t)n_exp + total / 16 + n / 16 + 4;  // token tiles of up to 16 entries
-  return align256(24 * (size_t)(n_exp + 1) + 4 * (size_t)(n_exp + 2) + 8 * tiles);
+  const size_t items = (size_t)n_exp + total / kPfBlkTokens + n / kPfBlkTokens + 4;  // blocks of up to 64 entries
+  return align256(24 * (size_t)(n_exp + 1) + 4 * (size_t)(n_exp + 2) + 8 * tiles + 12 * items);
 }
 bool routed_ok(int t) { return t == MSQ_IQ1_S || t == MSQ_IQ2_XXS; }
 bool shared_ok(int t) { return t == MSQ_Q6_K || t == MSQ_Q8_0 || t == MSQ_IQ2_XXS || t == MSQ_IQ1_S; }
@@ -42,6 +44,27 @@ int launch_gemm_t(hipStream_t st, PfArgs a, int cus) {
   MSQ_HIP(hipGetLastError());
   return MSQ_OK;
 }
+template <class B, bool GU>
+int launch_block_t(hipStream_t st, PfBlkArgs a) {
+  const size_t lds = (size_t)B::LDS_WORDS * 4 + 2 * (size_t)kPfBlkTokens * kPfBlkPitch;
+  const uint32_t rows_per_item = GU ? kPfBlkRowsGU : kPfBlkRowsDown;
+  a.row_chunks = (a.N + rows_per_item - 1) / rows_per_item;
+  static bool attr_set = false;  // per instantiation: allow more than 64 KiB of dynamic LDS
+  if (!attr_set) {
+    MSQ_HIP(hipFuncSetAttribute((const void*)moe_pf_block_kernel<B, GU>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+    attr_set = true;
+  }
+  const uint32_t grid = ((a.nitems + 7) / 8) * 8 * a.row_chunks;
+  hipLaunchKernelGGL((moe_pf_block_kernel<B, GU>), dim3(grid), dim3(kPfBlkThreads), lds, st, a);
+  MSQ_HIP(hipGetLastError());
+  return MSQ_OK;
+}
+bool block_path(int t) { return t == MSQ_IQ1_S || t == MSQ_IQ2_XXS; }
+template <bool GU>
+int launch_block(int t, hipStream_t st, const PfBlkArgs& a) {
+  return t == MSQ_IQ1_S ? launch_block_t<BlkIQ1S, GU>(st, a) : launch_block_t<BlkIQ2XXS, GU>(st, a);
+}
+
 template <bool GU>
 int launch_gemm(int t, hipStream_t st, const PfArgs& a, int cus) {
   switch (t) {
@@ -133,10 +156,27 @@ int msq_moe_prefill(void* stream, const MsqMoePrefillArgs* p) {
     for (int t0 = 0; t0 < p->offs[j + 1] - p->offs[j]; t0 += 16) { tiles[2 * nt_routed] = (uint32_t)j; tiles[2 * nt_routed + 1] = (uint32_t)t0; nt_routed++; }
   if (p->has_shared)
     for (int t0 = 0; t0 < n; t0 += 16) { tiles[2 * (nt_routed + nt_shared)] = (uint32_t)ne; tiles[2 * (nt_routed + nt_shared) + 1] = (uint32_t)t0; nt_shared++; }
+  // work items of the block GEMM: blocks of up to 64 entries, largest first (they take longest)
+  uint32_t* items = tiles + 2 * (size_t)(nt_routed + nt_shared);
+  uint32_t ni_routed = 0, ni_shared = 0;
+  {
+    std::vector<std::array<uint32_t, 3>> v;
+    for (int j = 0; j < ne; j++)
+      for (int t0 = 0; t0 < p->offs[j + 1] - p->offs[j]; t0 += kPfBlkTokens)
+        v.push_back({(uint32_t)j, (uint32_t)t0, (uint32_t)std::min(kPfBlkTokens, p->offs[j + 1] - p->offs[j] - t0)});
+    std::stable_sort(v.begin(), v.end(), [](const auto& x, const auto& y) { return x[2] > y[2]; });
+    for (const auto& it : v) { std::copy(it.begin(), it.end(), items + 3 * (size_t)ni_routed); ni_routed++; }
+    if (p->has_shared)
+      for (int t0 = 0; t0 < n; t0 += kPfBlkTokens) {
+        uint32_t* it = items + 3 * (size_t)(ni_routed + ni_shared);
+        it[0] = (uint32_t)ne; it[1] = (uint32_t)t0; it[2] = (uint32_t)std::min(kPfBlkTokens, n - t0);
+        ni_shared++;
+      }
+  }
   uint8_t* sc = bptr_mut(&p->scratch);
   // pageable source: the copy is staged by the runtime before this call returns, and ordered on the stream
-  MSQ_HIP(hipMemcpyAsync(sc, hdr.data(), 24 * (size_t)(ne + 1) + 4 * (size_t)(ne + 2) + 8 * (size_t)(nt_routed + nt_shared),
-                         hipMemcpyHostToDevice, st));
+  MSQ_HIP(hipMemcpyAsync(sc, hdr.data(), 24 * (size_t)(ne + 1) + 4 * (size_t)(ne + 2) + 8 * (size_t)(nt_routed + nt_shared) +
+                             12 * (size_t)(ni_routed + ni_shared), hipMemcpyHostToDevice, st));
   const size_t rows = (size_t)total + n;
   uint16_t* Xg = (uint16_t*)(sc + hbytes);
   uint16_t* H = (uint16_t*)((uint8_t*)Xg + align256(rows * dim * 2));
@@ -144,6 +184,7 @@ int msq_moe_prefill(void* stream, const MsqMoePrefillArgs* p) {
   const uint64_t* d_ptrs = (const uint64_t*)sc;
   const uint32_t* d_offs = (const uint32_t*)(sc + 24 * (size_t)(ne + 1));
   const uint32_t* d_tiles = d_offs + (ne + 2);
+  const uint32_t* d_items = d_tiles + 2 * (size_t)(nt_routed + nt_shared);
 
   // 1) gather + convert
   const uint32_t grows = (uint32_t)(total + (p->has_shared ? n : 0));
@@ -162,15 +203,28 @@ int msq_moe_prefill(void* stream, const MsqMoePrefillArgs* p) {
     const uint32_t ks = std::min<uint32_t>(16u, a.nsteps);
     a.steps_per_wave = (a.nsteps + ks - 1) / ks;
   };
+  PfBlkArgs b{};
+  b.H = H; b.Z = Z; b.wt = a.wt; b.ptrs = d_ptrs; b.offs = d_offs; b.total = (uint32_t)total;
+  // one GEMM over the routed experts or over the shared expert: block kernel for the codebook formats, else the
+  // token-tile kernel
+  auto gemm = [&](auto gu_tag, int type, bool shared, const uint16_t* A, uint32_t K, uint32_t N, size_t row_bytes) -> int {
+    constexpr bool GU = decltype(gu_tag)::value;
+    if (block_path(type)) {
+      b.A = A; b.K = K; b.N = N; b.nblocks = K / 256; b.row_bytes = (uint32_t)row_bytes;
+      b.items = d_items + (shared ? 3 * (size_t)ni_routed : 0); b.nitems = shared ? ni_shared : ni_routed;
+      return launch_block<GU>(type, st, b);
+    }
+    a.A = A; a.N = N; steps(K); a.row_bytes = (uint32_t)row_bytes;
+    a.tiles = d_tiles + (shared ? 2 * (size_t)nt_routed : 0); a.ntiles = shared ? nt_shared : nt_routed;
+    return launch_gemm<GU>(type, st, a, cus);
+  };
   int rc;
   // 2) gate + up + SwiGLU -> H
-  a.A = Xg; a.N = (uint32_t)inter; steps((uint32_t)dim);
-  if (nt_routed && !(skip & 2)) { a.tiles = d_tiles; a.ntiles = nt_routed; a.row_bytes = (uint32_t)rb_gu; if ((rc = launch_gemm<true>(p->t_gate_up, st, a, cus))) return rc; }
-  if (nt_shared && !(skip & 4)) { a.tiles = d_tiles + 2 * nt_routed; a.ntiles = nt_shared; a.row_bytes = (uint32_t)rb_sgu; if ((rc = launch_gemm<true>(p->t_shared, st, a, cus))) return rc; }
+  if (nt_routed && !(skip & 2) && (rc = gemm(std::true_type{}, p->t_gate_up, false, Xg, (uint32_t)dim, (uint32_t)inter, rb_gu))) return rc;
+  if (nt_shared && !(skip & 4) && (rc = gemm(std::true_type{}, p->t_shared, true, Xg, (uint32_t)dim, (uint32_t)inter, rb_sgu))) return rc;
   // 3) down -> Z
-  a.A = H; a.N = (uint32_t)dim; steps((uint32_t)inter);
-  if (nt_routed && !(skip & 8)) { a.tiles = d_tiles; a.ntiles = nt_routed; a.row_bytes = (uint32_t)rb_d; if ((rc = launch_gemm<false>(p->t_down, st, a, cus))) return rc; }
-  if (nt_shared && !(skip & 16)) { a.tiles = d_tiles + 2 * nt_routed; a.ntiles = nt_shared; a.row_bytes = (uint32_t)rb_sd; if ((rc = launch_gemm<false>(p->t_shared, st, a, cus))) return rc; }
+  if (nt_routed && !(skip & 8) && (rc = gemm(std::false_type{}, p->t_down, false, H, (uint32_t)inter, (uint32_t)dim, rb_d))) return rc;
+  if (nt_shared && !(skip & 16) && (rc = gemm(std::false_type{}, p->t_shared, true, H, (uint32_t)inter, (uint32_t)dim, rb_sd))) return rc;
   // 4) ordered reduction into Y
   if ((nt_routed || nt_shared) && !(skip & 32)) {
     const dim3 grid((dim / 4 + 255) / 256, (unsigned)n), block(256);
