@@ -220,7 +220,8 @@ struct FragDense16 {
 // q, the 8 columns col_of(q, j) .. + 7 of the block, and the activation operand is read with the same mapping.
 //   Raw / load(block pointer, q)    the lane's bytes of one block
 //   scale(raw)                      fp32 block scale
-//   frag(raw, j, tbl, h)            payloads of step j
+//   lookup(raw, j, tbl, col)        table reads of step j (col = lane % 16), issued ahead of their use
+//   finish(raw, j, look, h)         payloads of step j
 __device__ __forceinline__ uint32_t pk_mul_f16(uint32_t a, uint32_t b) {
   const h2_t r = as_h2(a) * as_h2(b);
   return __builtin_bit_cast(uint32_t, r);
@@ -231,9 +232,20 @@ __device__ __forceinline__ uint32_t pk_small_int_f16(uint32_t v) {
 }
 __device__ __forceinline__ uint32_t blk_col_of(uint32_t q, uint32_t j) { return 64u * q + 32u * (j >> 2) + 8u * (j & 3u); }
 
+// IQ2_XXS keeps 16 copies of its two small tables in LDS, copy c in the 16-byte bank column c of each 256-byte row:
+// a 16-lane group whose lanes read "their" column (c = lane % 16) touches every bank exactly once whatever the
+// entries are, so the random lookups run at the conflict-free rate.
 struct BlkIQ2XXS {
-  static constexpr int LDS_WORDS = FragIQ2XXS::LDS_WORDS, BLOCK_BYTES = 66;
-  __device__ static void fill_lds(uint32_t* lds, int tid, int nt) { FragIQ2XXS::fill_lds(lds, tid, nt); }
+  static constexpr int LDS_WORDS = (MSQ_IQ2XXS_GRID_N + 128) * 16 * 4, BLOCK_BYTES = 66;
+  __device__ static void fill_lds(uint32_t* lds, int tid, int nt) {
+    const uint4* grid = (const uint4*)g_tbl_iq2xxs.w;
+    const uint4* sign = (const uint4*)g_tbl_sign.w;
+    uint4* dst = (uint4*)lds;
+    for (int i = tid; i < (MSQ_IQ2XXS_GRID_N + 128) * 16; i += nt) {
+      const int e = i >> 4;
+      dst[i] = e < MSQ_IQ2XXS_GRID_N ? grid[e] : sign[e - MSQ_IQ2XXS_GRID_N];
+    }
+  }
   struct Raw { uint32_t w[4]; uint32_t d; };  // {a0, a1} of sub-block 2 q, then of 2 q + 1; fp16 bits of d
   template <class P>
   __device__ static Raw load(P blk, uint32_t q) {
@@ -241,14 +253,18 @@ struct BlkIQ2XXS {
     return {{v.x, v.y, v.z, v.w}, ld16(blk)};
   }
   __device__ static float scale(const Raw& r) { return half_bits_to_float(r.d) * 0.125f; }  // db = d (2 s + 1) / 8
-  __device__ static void frag(const Raw& r, int j, const uint32_t* tbl, uint32_t (&h)[4]) {
+  struct Look { uint4 g, s; };
+  __device__ static Look lookup(const Raw& r, int j, const uint32_t* tbl, uint32_t col) {
     const uint32_t a0 = r.w[2 * (j >> 2)], a1 = r.w[2 * (j >> 2) + 1];
     const int l = j & 3;
-    const uint4 g = ((const uint4*)tbl)[(a0 >> (8 * l)) & 0xFFu];
-    const uint4 s = ((const uint4*)(tbl + MSQ_IQ2XXS_GRID_N * 4))[(a1 >> (7 * l)) & 127u];
+    const uint4* t4 = (const uint4*)tbl;
+    return {t4[(((a0 >> (8 * l)) & 0xFFu) << 4) | col], t4[MSQ_IQ2XXS_GRID_N * 16 + ((((a1 >> (7 * l)) & 127u) << 4) | col)]};
+  }
+  __device__ static void finish(const Raw& r, int j, const Look& k, uint32_t (&h)[4]) {
+    const uint32_t a1 = r.w[2 * (j >> 2) + 1];
     const uint32_t m2 = pk_small_int_f16(((a1 >> 27) & 0x1Eu) | 1u);  // 2 s + 1 <= 31; grid <= 43: products are exact
-    h[0] = pk_mul_f16(g.x ^ s.x, m2); h[1] = pk_mul_f16(g.y ^ s.y, m2);
-    h[2] = pk_mul_f16(g.z ^ s.z, m2); h[3] = pk_mul_f16(g.w ^ s.w, m2);
+    h[0] = pk_mul_f16(k.g.x ^ k.s.x, m2); h[1] = pk_mul_f16(k.g.y ^ k.s.y, m2);
+    h[2] = pk_mul_f16(k.g.z ^ k.s.z, m2); h[3] = pk_mul_f16(k.g.w ^ k.s.w, m2);
   }
 };
 
@@ -262,15 +278,18 @@ struct BlkIQ1S {
     return {{v.x, v.y}, ld32(blk + 34 + 4 * q), ld16(blk)};
   }
   __device__ static float scale(const Raw& r) { return half_bits_to_float(r.d); }  // w = d (2 s + 1) (g + delta)
-  __device__ static void frag(const Raw& r, int j, const uint32_t* tbl, uint32_t (&h)[4]) {
+  struct Look { uint4 g; };
+  __device__ static Look lookup(const Raw& r, int j, const uint32_t* tbl, uint32_t) {
     const uint32_t qs = r.qs[j >> 2], qh = (j >> 2) ? r.qh >> 16 : r.qh & 0xFFFFu;
     const int l = j & 3;
-    const uint32_t idx = ((qs >> (8 * l)) & 0xFFu) | (((qh >> (3 * l)) & 7u) << 8);
-    const uint4 g = ((const uint4*)tbl)[idx];
+    return {((const uint4*)tbl)[((qs >> (8 * l)) & 0xFFu) | (((qh >> (3 * l)) & 7u) << 8)]};
+  }
+  __device__ static void finish(const Raw& r, int j, const Look& k, uint32_t (&h)[4]) {
+    const uint32_t qh = (j >> 2) ? r.qh >> 16 : r.qh & 0xFFFFu;
     const uint32_t d2 = (qh & 0x8000u) ? 0xB000B000u : 0x30003000u;          // -+ 1/8 in both halves
     const uint32_t m2 = pk_small_int_f16(((qh >> 11) & 0xEu) | 1u);          // 2 s + 1 <= 15; |g + delta| <= 9/8
-    h[0] = pk_mul_f16(pk_add_f16(g.x, d2), m2); h[1] = pk_mul_f16(pk_add_f16(g.y, d2), m2);
-    h[2] = pk_mul_f16(pk_add_f16(g.z, d2), m2); h[3] = pk_mul_f16(pk_add_f16(g.w, d2), m2);
+    h[0] = pk_mul_f16(pk_add_f16(k.g.x, d2), m2); h[1] = pk_mul_f16(pk_add_f16(k.g.y, d2), m2);
+    h[2] = pk_mul_f16(pk_add_f16(k.g.z, d2), m2); h[3] = pk_mul_f16(pk_add_f16(k.g.w, d2), m2);
   }
 };
 

@@ -179,11 +179,12 @@ __global__ __launch_bounds__(1024) void moe_pf_gemm_kernel(const PfArgs a) {
 
 // ------------------------------------------------------------------------------------------------ block GEMM
 // Grouped GEMM for the 256-weight codebook formats (block fragments, see msq_mfma.cuh). A work item is one expert's
-// block of up to 64 entries (token tiles t < T <= 4) times a chunk of weight rows; the item's 8 waves own different
-// weight-row tiles and walk K block by block (256 columns): the activation block [64][256] fp16 is staged in LDS for
-// all waves (double-buffered, one barrier per block), every wave decodes the fragments of its own rows once per block
-// and reuses each of them for all T token tiles, accumulates the block in the matrix cores and applies the fp32 block
-// scale once. Weights are decoded exactly once per (item, row): no lane loads a weight byte twice.
+// block of up to 48 entries (T <= 3 token tiles) times a chunk of weight rows; the item's 8 waves own different
+// weight-row tiles and walk K block by block (256 columns): the activation block [48][256] fp16 is staged in LDS for
+// all waves, every wave decodes the fragments of its own rows once per block and reuses each of them for all T token
+// tiles, accumulates the block in the matrix cores and applies the fp32 block scale once. Weights are decoded exactly
+// once per (item, row), no lane loads a weight byte twice, and the next block's bytes are in flight during a block.
+// Table lookups run one fragment pair ahead of the pair being multiplied.
 struct PfBlkArgs {
   const uint16_t* A;        // fp16 activations [entries][K]
   const uint64_t* ptrs;     // per expert: gate, up, down addresses
@@ -197,27 +198,18 @@ struct PfBlkArgs {
   uint32_t row_chunks;      // chunks of 8 * RT * 16 weight rows
 };
 
-constexpr int kPfBlkTokens = 64, kPfBlkThreads = 512, kPfBlkPitch = 256 * 2 + 16;
+constexpr int kPfBlkTokens = 48, kPfBlkThreads = 512, kPfBlkPitch = 256 * 2 + 16;
 constexpr int kPfBlkRowsGU = 8 * 2 * 16, kPfBlkRowsDown = 8 * 4 * 16;  // weight rows per work item
 
-template <class B, bool GU>
-__global__ __launch_bounds__(kPfBlkThreads) void moe_pf_block_kernel(const PfBlkArgs a) {
-  constexpr int NM = GU ? 2 : 1, RT = GU ? 2 : 4, R = RT * NM, TMAX = kPfBlkTokens / 16, PITCH = kPfBlkPitch;
-  extern __shared__ __attribute__((aligned(16))) uint32_t smem[];
+template <class B, bool GU, int T>
+__device__ __forceinline__ void pf_block_run(const PfBlkArgs& a, uint32_t* smem, uint32_t e, uint32_t base, uint32_t cnt, uint32_t rc) {
+  constexpr int NM = GU ? 2 : 1, RT = GU ? 2 : 4, R = RT * NM, PITCH = kPfBlkPitch;
+  static_assert(R == 4, "fragment pairs below assume four fragments per step");
   uint32_t* tbl = smem;
-  uint8_t* abuf = (uint8_t*)(smem + B::LDS_WORDS);  // [2][64 tokens][PITCH]
+  uint8_t* abuf = (uint8_t*)(smem + B::LDS_WORDS);  // [T * 16 tokens][PITCH]
   const uint32_t tid = threadIdx.x, lane = tid & 63u;
   const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
   const uint32_t n16 = lane & 15u, q = lane >> 4;
-
-  // consecutive workgroups land on different XCDs: the row chunks of one item stay on one XCD (shared L2 for its
-  // activations), and items -- sorted by size -- are dealt round-robin over the XCDs
-  const uint32_t xcd = blockIdx.x & 7u, slot = blockIdx.x >> 3;
-  const uint32_t item = (slot / a.row_chunks) * 8u + xcd, rc = slot % a.row_chunks;
-  if (item >= a.nitems) return;
-  const uint32_t e = a.items[3 * item], t0 = a.items[3 * item + 1], cnt = a.items[3 * item + 2];
-  const uint32_t base = a.offs[e] + t0;
-  const uint32_t T = (cnt + 15u) / 16u;
 
   gptr_t wrow[R];
   uint32_t row_of[RT];
@@ -232,19 +224,18 @@ __global__ __launch_bounds__(kPfBlkThreads) void moe_pf_block_kernel(const PfBlk
 
   // activation chunk loader: thread owns granule (token 16 i + tid / 32, 16-byte column tid % 32) of every token tile
   const uint32_t atok = tid >> 5, acol = tid & 31u;
-  uint4 pa[TMAX];
+  uint4 pa[T];
   auto a_issue = [&](uint32_t kc) {
 #pragma unroll
-    for (int i = 0; i < TMAX; i++) {
+    for (int i = 0; i < T; i++) {
       const uint32_t tok = 16u * i + atok;
       pa[i] = uint4{0u, 0u, 0u, 0u};
       if (tok < cnt) pa[i] = *(const uint4*)(a.A + (size_t)(base + tok) * a.K + kc * 256u + acol * 8u);
     }
   };
-  auto a_store = [&](uint32_t buf) {
+  auto a_store = [&]() {
 #pragma unroll
-    for (int i = 0; i < TMAX; i++)
-      if ((uint32_t)i < T) *(uint4*)(abuf + buf * (kPfBlkTokens * PITCH) + (16u * i + atok) * PITCH + acol * 16u) = pa[i];
+    for (int i = 0; i < T; i++) *(uint4*)(abuf + (16u * i + atok) * PITCH + acol * 16u) = pa[i];
   };
 
   typename B::Raw cur[R], nxt[R];
@@ -252,53 +243,62 @@ __global__ __launch_bounds__(kPfBlkThreads) void moe_pf_block_kernel(const PfBlk
   for (int r = 0; r < R; r++) cur[r] = B::load(wrow[r], q);
   a_issue(0);
   B::fill_lds(tbl, (int)tid, (int)blockDim.x);
-  a_store(0);
+  a_store();
   __syncthreads();
 
-  f4_t acc[TMAX][R];
+  f4_t acc[T][R];
 #pragma unroll
-  for (int t = 0; t < TMAX; t++)
+  for (int t = 0; t < T; t++)
 #pragma unroll
     for (int r = 0; r < R; r++) acc[t][r] = f4_t{0.f, 0.f, 0.f, 0.f};
+  const f4_t zero = {0.f, 0.f, 0.f, 0.f};
+  const uint8_t* arow = abuf + n16 * PITCH;
 
   for (uint32_t kc = 0; kc < a.nblocks; kc++) {
-    const uint32_t buf = kc & 1u;
     const bool more = kc + 1 < a.nblocks;
     if (more) {
 #pragma unroll
       for (int r = 0; r < R; r++) nxt[r] = B::load(wrow[r] + (size_t)(kc + 1) * B::BLOCK_BYTES, q);
       a_issue(kc + 1);
     }
-    f4_t blk[TMAX][R];
+    f4_t blk[T][R];
+    typename B::Look lk[2][2];  // pair p = 2 j + half uses lk[p & 1]: fragments 2 half, 2 half + 1 of step j
+    lk[0][0] = B::lookup(cur[0], 0, tbl, n16);
+    lk[0][1] = B::lookup(cur[1], 0, tbl, n16);
+    uint32_t af[T][4];
 #pragma unroll
-    for (int t = 0; t < TMAX; t++)
+    for (int p = 0; p < 16; p++) {
+      const int j = p >> 1, r0 = 2 * (p & 1);
+      if (!(p & 1)) {  // activations of step j, read with the fragments' column mapping
 #pragma unroll
-      for (int r = 0; r < R; r++) blk[t][r] = f4_t{0.f, 0.f, 0.f, 0.f};
-    const uint8_t* arow = abuf + buf * (kPfBlkTokens * PITCH) + n16 * PITCH;
-#pragma unroll
-    for (int j = 0; j < 8; j++) {
-      uint32_t h[R][4];
-#pragma unroll
-      for (int r = 0; r < R; r++) B::frag(cur[r], j, tbl, h[r]);
-#pragma unroll
-      for (int t = 0; t < TMAX; t++) {
-        if ((uint32_t)t < T) {  // wave-uniform
+        for (int t = 0; t < T; t++) {
           const uint4 av = *(const uint4*)(arow + t * 16 * PITCH + 2u * blk_col_of(q, j));
-          const uint32_t af[4] = {av.x, av.y, av.z, av.w};
-#pragma unroll
-          for (int r = 0; r < R; r++) blk[t][r] = mfma_f16(af, h[r], blk[t][r]);
+          af[t][0] = av.x; af[t][1] = av.y; af[t][2] = av.z; af[t][3] = av.w;
         }
+      }
+      if (p + 1 < 16) {  // table reads of the next pair
+        const int jn = (p + 1) >> 1, rn = 2 * ((p + 1) & 1);
+        lk[(p + 1) & 1][0] = B::lookup(cur[rn], jn, tbl, n16);
+        lk[(p + 1) & 1][1] = B::lookup(cur[rn + 1], jn, tbl, n16);
+      }
+      uint32_t h[2][4];
+      B::finish(cur[r0], j, lk[p & 1][0], h[0]);
+      B::finish(cur[r0 + 1], j, lk[p & 1][1], h[1]);
+#pragma unroll
+      for (int t = 0; t < T; t++) {
+        blk[t][r0] = mfma_f16(af[t], h[0], j == 0 ? zero : blk[t][r0]);
+        blk[t][r0 + 1] = mfma_f16(af[t], h[1], j == 0 ? zero : blk[t][r0 + 1]);
       }
     }
 #pragma unroll
     for (int r = 0; r < R; r++) {
       const float sc = B::scale(cur[r]);
 #pragma unroll
-      for (int t = 0; t < TMAX; t++)
-        if ((uint32_t)t < T) acc[t][r] += sc * blk[t][r];
+      for (int t = 0; t < T; t++) acc[t][r] += sc * blk[t][r];
     }
+    __syncthreads();  // every wave is done with this block's activations
     if (more) {
-      a_store(buf ^ 1u);
+      a_store();
 #pragma unroll
       for (int r = 0; r < R; r++) cur[r] = nxt[r];
     }
@@ -306,8 +306,7 @@ __global__ __launch_bounds__(kPfBlkThreads) void moe_pf_block_kernel(const PfBlk
   }
 
 #pragma unroll
-  for (int t = 0; t < TMAX; t++) {
-    if ((uint32_t)t >= T) continue;
+  for (int t = 0; t < T; t++) {
 #pragma unroll
     for (int i = 0; i < 4; i++) {
       const uint32_t tok = 16u * t + 4u * q + i;
@@ -327,6 +326,21 @@ __global__ __launch_bounds__(kPfBlkThreads) void moe_pf_block_kernel(const PfBlk
       }
     }
   }
+}
+
+template <class B, bool GU>
+__global__ __launch_bounds__(kPfBlkThreads) void moe_pf_block_kernel(const PfBlkArgs a) {
+  extern __shared__ __attribute__((aligned(16))) uint32_t smem[];
+  // consecutive workgroups land on different XCDs: the row chunks of one item stay on one XCD (shared L2 for its
+  // activations), and items -- sorted by size -- are dealt round-robin over the XCDs
+  const uint32_t xcd = blockIdx.x & 7u, slot = blockIdx.x >> 3;
+  const uint32_t item = (slot / a.row_chunks) * 8u + xcd, rc = slot % a.row_chunks;
+  if (item >= a.nitems) return;
+  const uint32_t e = a.items[3 * item], t0 = a.items[3 * item + 1], cnt = a.items[3 * item + 2];
+  const uint32_t base = a.offs[e] + t0;
+  if (cnt <= 16) pf_block_run<B, GU, 1>(a, smem, e, base, cnt, rc);
+  else if (cnt <= 32) pf_block_run<B, GU, 2>(a, smem, e, base, cnt, rc);
+  else pf_block_run<B, GU, 3>(a, smem, e, base, cnt, rc);
 }
 
 // Xg[i] = fp16(X[src(i)]): i < total gathers token tok[i]; rows total .. total + n - 1 are the tokens themselves

@@ -46,7 +46,7 @@ int launch_gemm_t(hipStream_t st, PfArgs a, int cus) {
 }
 template <class B, bool GU>
 int launch_block_t(hipStream_t st, PfBlkArgs a) {
-  const size_t lds = (size_t)B::LDS_WORDS * 4 + 2 * (size_t)kPfBlkTokens * kPfBlkPitch;
+  const size_t lds = (size_t)B::LDS_WORDS * 4 + (size_t)kPfBlkTokens * kPfBlkPitch;
   const uint32_t rows_per_item = GU ? kPfBlkRowsGU : kPfBlkRowsDown;
   a.row_chunks = (a.N + rows_per_item - 1) / rows_per_item;
   static bool attr_set = false;  // per instantiation: allow more than 64 KiB of dynamic LDS
