@@ -230,6 +230,20 @@ __device__ __forceinline__ uint32_t pk_mul_f16(uint32_t a, uint32_t b) {
 __device__ __forceinline__ uint32_t pk_small_int_f16(uint32_t v) {
   return pk_add_f16(0x64006400u | v | (v << 16), 0xE400E400u);
 }
+// N dwords from a global address that is only 2-byte aligned, fetched with 4-byte-aligned loads: wide loads that are
+// not dword aligned run at about a third of the rate of aligned ones. N aligned dwords plus the one that follows (the
+// last one again when the address is aligned, so nothing past the data is touched), then a funnel shift.
+template <int N>
+__device__ __forceinline__ void ld_dwords_2aligned(gptr_t p, uint32_t (&out)[N]) {
+  typedef uint32_t __attribute__((ext_vector_type(N), aligned(4))) vec_t;
+  const uintptr_t a = (uintptr_t)p;
+  const uint32_t odd = (uint32_t)a & 2u;
+  const MSQ_GLOBAL uint32_t* w = (const MSQ_GLOBAL uint32_t*)(a - odd);
+  const vec_t v = *(const MSQ_GLOBAL vec_t*)w;
+  const uint32_t tail = w[odd ? N : N - 1];
+#pragma unroll
+  for (int i = 0; i < N; i++) out[i] = __builtin_amdgcn_alignbit(i + 1 < N ? v[i + 1] : tail, v[i], odd * 8u);
+}
 __device__ __forceinline__ uint32_t blk_col_of(uint32_t q, uint32_t j) { return 64u * q + 32u * (j >> 2) + 8u * (j & 3u); }
 
 // IQ2_XXS keeps 16 copies of its two small tables in LDS, copy c in the 16-byte bank column c of each 256-byte row:
@@ -247,10 +261,11 @@ struct BlkIQ2XXS {
     }
   }
   struct Raw { uint32_t w[4]; uint32_t d; };  // {a0, a1} of sub-block 2 q, then of 2 q + 1; fp16 bits of d
-  template <class P>
-  __device__ static Raw load(P blk, uint32_t q) {
-    const u128_a2 v = ld128(blk + 2 + 16 * q);
-    return {{v.x, v.y, v.z, v.w}, ld16(blk)};
+  __device__ static Raw load(gptr_t blk, uint32_t q) {
+    Raw r;
+    ld_dwords_2aligned<4>(blk + 2 + 16 * q, r.w);
+    r.d = ld16(blk);
+    return r;
   }
   __device__ static float scale(const Raw& r) { return half_bits_to_float(r.d) * 0.125f; }  // db = d (2 s + 1) / 8
   struct Look { uint4 g, s; };
@@ -272,10 +287,14 @@ struct BlkIQ1S {
   static constexpr int LDS_WORDS = FragIQ1S::LDS_WORDS, BLOCK_BYTES = 50;
   __device__ static void fill_lds(uint32_t* lds, int tid, int nt) { FragIQ1S::fill_lds(lds, tid, nt); }
   struct Raw { uint32_t qs[2]; uint32_t qh; uint32_t d; };  // qs bytes 8 q .. 8 q + 7; qh[2 q] | qh[2 q + 1] << 16
-  template <class P>
-  __device__ static Raw load(P blk, uint32_t q) {
-    const u64_a2 v = ld64(blk + 2 + 8 * q);
-    return {{v.x, v.y}, ld32(blk + 34 + 4 * q), ld16(blk)};
+  __device__ static Raw load(gptr_t blk, uint32_t q) {
+    Raw r;
+    uint32_t qh[1];
+    ld_dwords_2aligned<2>(blk + 2 + 8 * q, r.qs);
+    ld_dwords_2aligned<1>(blk + 34 + 4 * q, qh);
+    r.qh = qh[0];
+    r.d = ld16(blk);
+    return r;
   }
   __device__ static float scale(const Raw& r) { return half_bits_to_float(r.d); }  // w = d (2 s + 1) (g + delta)
   struct Look { uint4 g; };

@@ -17,6 +17,9 @@
 #include <type_traits>
 
 #include "msq_mfma.cuh"
+#ifndef MSQ_EXP
+#define MSQ_EXP 0
+#endif
 
 namespace msq {
 
@@ -179,7 +182,7 @@ __global__ __launch_bounds__(1024) void moe_pf_gemm_kernel(const PfArgs a) {
 
 // ------------------------------------------------------------------------------------------------ block GEMM
 // Grouped GEMM for the 256-weight codebook formats (block fragments, see msq_mfma.cuh). A work item is one expert's
-// block of up to 48 entries (T <= 3 token tiles) times a chunk of weight rows; the item's 8 waves own different
+// block of up to 48 entries (T <= 3 token tiles) times a chunk of weight rows; the item's waves own different
 // weight-row tiles and walk K block by block (256 columns): the activation block [48][256] fp16 is staged in LDS for
 // all waves, every wave decodes the fragments of its own rows once per block and reuses each of them for all T token
 // tiles, accumulates the block in the matrix cores and applies the fp32 block scale once. Weights are decoded exactly
@@ -195,55 +198,79 @@ struct PfBlkArgs {
   float* Z;                 // down output [entries][N] fp32
   uint32_t nitems, total;
   uint32_t K, N, row_bytes, nblocks;
-  uint32_t row_chunks;      // chunks of 8 * RT * 16 weight rows
+  uint32_t row_chunks;      // chunks of pf_blk_rows() weight rows
 };
 
-constexpr int kPfBlkTokens = 48, kPfBlkThreads = 512, kPfBlkPitch = 256 * 2 + 16;
-constexpr int kPfBlkRowsGU = 8 * 2 * 16, kPfBlkRowsDown = 8 * 4 * 16;  // weight rows per work item
+constexpr int kPfBlkTokens = 48, kPfBlkPitch = 256 * 2 + 16;
+// waves per workgroup by token tiles per item: the one-tile variant needs few registers and runs four waves per SIMD
+// (it is the one that streams weights fastest and has the least matrix work to hide latency behind)
+constexpr int pf_blk_waves(int T) { return T == 1 ? 16 : 8; }
+// weight-row tiles per wave (the one-tile variant takes half as many to stay within its registers)
+constexpr int pf_blk_rt(bool gu, int T) { return (gu ? 2 : 4) / (T == 1 ? 2 : 1); }
+constexpr int pf_blk_rows(bool gu, int T) { return pf_blk_waves(T) * pf_blk_rt(gu, T) * 16; }  // weight rows per work item
+template <class B>
+constexpr size_t pf_blk_lds() { return (size_t)B::LDS_WORDS * 4 + 2 * (size_t)kPfBlkTokens * kPfBlkPitch; }
 
 template <class B, bool GU, int T>
-__device__ __forceinline__ void pf_block_run(const PfBlkArgs& a, uint32_t* smem, uint32_t e, uint32_t base, uint32_t cnt, uint32_t rc) {
-  constexpr int NM = GU ? 2 : 1, RT = GU ? 2 : 4, R = RT * NM, PITCH = kPfBlkPitch;
-  static_assert(R == 4, "fragment pairs below assume four fragments per step");
+__global__ __launch_bounds__(64 * pf_blk_waves(T)) void moe_pf_block_kernel(const PfBlkArgs a) {
+  constexpr int WAVES = pf_blk_waves(T), NT = 64 * WAVES;
+  constexpr int NM = GU ? 2 : 1, RT = pf_blk_rt(GU, T), R = RT * NM, PITCH = kPfBlkPitch;
+  constexpr int ABUF = kPfBlkTokens * PITCH;
+  constexpr int PPS = R / 2, NP = 8 * PPS;  // fragment pairs per K step, per block
+  static_assert(R == 2 || R == 4, "fragments are processed in pairs");
+  extern __shared__ __attribute__((aligned(16))) uint32_t smem[];
   uint32_t* tbl = smem;
-  uint8_t* abuf = (uint8_t*)(smem + B::LDS_WORDS);  // [T * 16 tokens][PITCH]
+  uint8_t* abuf = (uint8_t*)(smem + B::LDS_WORDS);  // [2][T * 16 tokens][PITCH]
   const uint32_t tid = threadIdx.x, lane = tid & 63u;
   const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
   const uint32_t n16 = lane & 15u, q = lane >> 4;
+
+  // consecutive workgroups land on different XCDs: the row chunks of one item stay on one XCD (shared L2 for its
+  // activations), and items are dealt round-robin over the XCDs
+  const uint32_t xcd = blockIdx.x & 7u, slot = blockIdx.x >> 3;
+  const uint32_t item = (slot / a.row_chunks) * 8u + xcd, rc = slot % a.row_chunks;
+  if (item >= a.nitems) return;
+  const uint32_t e = a.items[3 * item], t0 = a.items[3 * item + 1], cnt = a.items[3 * item + 2];
+  const uint32_t base = a.offs[e] + t0;
 
   gptr_t wrow[R];
   uint32_t row_of[RT];
 #pragma unroll
   for (int jt = 0; jt < RT; jt++) {
-    row_of[jt] = ((rc * 8u + wave) * RT + jt) * 16u + n16;
+    row_of[jt] = ((rc * WAVES + wave) * RT + jt) * 16u + n16;
     const uint32_t row = min(row_of[jt], a.N - 1);
 #pragma unroll
     for (int m = 0; m < NM; m++)
       wrow[jt * NM + m] = as_global((const void*)a.ptrs[3 * e + (GU ? m : 2)]) + (size_t)row * a.row_bytes;
   }
 
-  // activation chunk loader: thread owns granule (token 16 i + tid / 32, 16-byte column tid % 32) of every token tile
-  const uint32_t atok = tid >> 5, acol = tid & 31u;
-  uint4 pa[T];
+  // activation chunk loader: T * 512 granules of 16 bytes (token g / 32, column g % 32) over the workgroup's threads
+  constexpr int AG = (T * 512 + NT - 1) / NT;
+  u32x4 pa[AG];  // (a plain vector type: the HIP struct type keeps the array in scratch memory)
   auto a_issue = [&](uint32_t kc) {
 #pragma unroll
-    for (int i = 0; i < T; i++) {
-      const uint32_t tok = 16u * i + atok;
-      pa[i] = uint4{0u, 0u, 0u, 0u};
-      if (tok < cnt) pa[i] = *(const uint4*)(a.A + (size_t)(base + tok) * a.K + kc * 256u + acol * 8u);
+    for (int i = 0; i < AG; i++) {
+      // rows past the block's last entry repeat it (their products are never stored): no branch around the load, so
+      // the number of loads in flight stays known to every wait that follows
+      const uint32_t g = min(tid + i * NT, T * 512u - 1u);
+      const uint32_t tok = min(g >> 5, cnt - 1);
+      pa[i] = *(const u32x4*)(a.A + (size_t)(base + tok) * a.K + kc * 256u + (g & 31u) * 8u);
     }
   };
-  auto a_store = [&]() {
+  auto a_store = [&](uint32_t buf) {
 #pragma unroll
-    for (int i = 0; i < T; i++) *(uint4*)(abuf + (16u * i + atok) * PITCH + acol * 16u) = pa[i];
+    for (int i = 0; i < AG; i++) {
+      const uint32_t g = tid + i * NT;
+      if (g < T * 512u) *(u32x4*)(abuf + buf * ABUF + (g >> 5) * PITCH + (g & 31u) * 16u) = pa[i];
+    }
   };
 
   typename B::Raw cur[R], nxt[R];
 #pragma unroll
   for (int r = 0; r < R; r++) cur[r] = B::load(wrow[r], q);
   a_issue(0);
-  B::fill_lds(tbl, (int)tid, (int)blockDim.x);
-  a_store();
+  B::fill_lds(tbl, (int)tid, NT);
+  a_store(0);
   __syncthreads();
 
   f4_t acc[T][R];
@@ -252,32 +279,48 @@ __device__ __forceinline__ void pf_block_run(const PfBlkArgs& a, uint32_t* smem,
 #pragma unroll
     for (int r = 0; r < R; r++) acc[t][r] = f4_t{0.f, 0.f, 0.f, 0.f};
   const f4_t zero = {0.f, 0.f, 0.f, 0.f};
-  const uint8_t* arow = abuf + n16 * PITCH;
 
   for (uint32_t kc = 0; kc < a.nblocks; kc++) {
-    const bool more = kc + 1 < a.nblocks;
-    if (more) {
-#pragma unroll
-      for (int r = 0; r < R; r++) nxt[r] = B::load(wrow[r] + (size_t)(kc + 1) * B::BLOCK_BYTES, q);
-      a_issue(kc + 1);
-    }
+    const uint32_t kn = kc + 1 < a.nblocks ? kc + 1 : kc;  // the last block fetches itself again: no branch around the loads
+    const uint8_t* arow = abuf + (kc & 1u) * ABUF + n16 * PITCH;
     f4_t blk[T][R];
-    typename B::Look lk[2][2];  // pair p = 2 j + half uses lk[p & 1]: fragments 2 half, 2 half + 1 of step j
-    lk[0][0] = B::lookup(cur[0], 0, tbl, n16);
-    lk[0][1] = B::lookup(cur[1], 0, tbl, n16);
+    // table reads run one fragment pair ahead where registers allow (pair p = 2 j + half uses lk[p & 1]: fragments
+    // 2 half, 2 half + 1 of step j): the one-tile variant has four waves per SIMD to hide them behind instead, the
+    // three-tile variant six matrix instructions per pair
+    constexpr bool AHEAD = T == 2;
+    typename B::Look lk[2][2];
+    if (AHEAD) {
+      lk[0][0] = B::lookup(cur[0], 0, tbl, n16);
+      lk[0][1] = B::lookup(cur[1], 0, tbl, n16);
+    }
     uint32_t af[T][4];
 #pragma unroll
-    for (int p = 0; p < 16; p++) {
-      const int j = p >> 1, r0 = 2 * (p & 1);
-      if (!(p & 1)) {  // activations of step j, read with the fragments' column mapping
+    for (int p = 0; p < NP; p++) {
+      const int j = p / PPS, r0 = 2 * (p % PPS);
+      // the next block's bytes are requested a few at a time between the fragment pairs: requested all at once by
+      // all waves right after the barrier, they queue up in the texture addresser and hold the waves at issue
+      if (p == 1) {
+        __builtin_amdgcn_sched_barrier(0);  // keep the requests here: the scheduler would sink them to their first use
+        a_issue(kn);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      if (p % 2 == 0 && p >= 2 && p / 2 - 1 < R) {
+        __builtin_amdgcn_sched_barrier(0);
+        nxt[p / 2 - 1] = B::load(wrow[p / 2 - 1] + (size_t)kn * B::BLOCK_BYTES, q);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      if (p % PPS == 0 && T < 3) {  // activations of step j, read with the fragments' column mapping
 #pragma unroll
         for (int t = 0; t < T; t++) {
           const uint4 av = *(const uint4*)(arow + t * 16 * PITCH + 2u * blk_col_of(q, j));
           af[t][0] = av.x; af[t][1] = av.y; af[t][2] = av.z; af[t][3] = av.w;
         }
       }
-      if (p + 1 < 16) {  // table reads of the next pair
-        const int jn = (p + 1) >> 1, rn = 2 * ((p + 1) & 1);
+      if (!AHEAD) {
+        lk[p & 1][0] = B::lookup(cur[r0], j, tbl, n16);
+        lk[p & 1][1] = B::lookup(cur[r0 + 1], j, tbl, n16);
+      } else if (p + 1 < NP) {  // table reads of the next pair
+        const int jn = (p + 1) / PPS, rn = 2 * ((p + 1) % PPS);
         lk[(p + 1) & 1][0] = B::lookup(cur[rn], jn, tbl, n16);
         lk[(p + 1) & 1][1] = B::lookup(cur[rn + 1], jn, tbl, n16);
       }
@@ -286,8 +329,13 @@ __device__ __forceinline__ void pf_block_run(const PfBlkArgs& a, uint32_t* smem,
       B::finish(cur[r0 + 1], j, lk[p & 1][1], h[1]);
 #pragma unroll
       for (int t = 0; t < T; t++) {
-        blk[t][r0] = mfma_f16(af[t], h[0], j == 0 ? zero : blk[t][r0]);
-        blk[t][r0 + 1] = mfma_f16(af[t], h[1], j == 0 ? zero : blk[t][r0 + 1]);
+        if (T >= 3) {  // short of registers: each tile's activations are read right before their use
+          const uint4 av = *(const uint4*)(arow + t * 16 * PITCH + 2u * blk_col_of(q, j));
+          af[0][0] = av.x; af[0][1] = av.y; af[0][2] = av.z; af[0][3] = av.w;
+        }
+        const uint32_t(&x)[4] = af[T >= 3 ? 0 : t];
+        blk[t][r0] = mfma_f16(x, h[0], j == 0 ? zero : blk[t][r0]);
+        blk[t][r0 + 1] = mfma_f16(x, h[1], j == 0 ? zero : blk[t][r0 + 1]);
       }
     }
 #pragma unroll
@@ -296,15 +344,22 @@ __device__ __forceinline__ void pf_block_run(const PfBlkArgs& a, uint32_t* smem,
 #pragma unroll
       for (int t = 0; t < T; t++) acc[t][r] += sc * blk[t][r];
     }
-    __syncthreads();  // every wave is done with this block's activations
-    if (more) {
-      a_store();
+    // the other activation buffer was last read one block ago, before the previous barrier: free to refill
+    a_store((kc & 1u) ^ 1u);
 #pragma unroll
-      for (int r = 0; r < R; r++) cur[r] = nxt[r];
-    }
+    for (int r = 0; r < R; r++) cur[r] = nxt[r];
     __syncthreads();
   }
 
+  float wts[T][4];  // routing weights of the lane's entries, fetched together ahead of the epilogue's math
+#pragma unroll
+  for (int t = 0; t < T; t++)
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      const uint32_t entry = base + min(16u * t + 4u * q + i, cnt - 1);
+      wts[t][i] = GU && entry < a.total ? a.wt[entry] : 1.f;
+    }
+  __builtin_amdgcn_sched_barrier(0);  // all requests first: sunk to their uses they would be waited for one by one
 #pragma unroll
   for (int t = 0; t < T; t++) {
 #pragma unroll
@@ -317,8 +372,7 @@ __device__ __forceinline__ void pf_block_run(const PfBlkArgs& a, uint32_t* smem,
         if (row_of[jt] >= a.N) continue;
         if constexpr (GU) {
           const float g = fminf(acc[t][2 * jt][i], 10.f), u = fminf(fmaxf(acc[t][2 * jt + 1][i], -10.f), 10.f);
-          const float w = entry < a.total ? a.wt[entry] : 1.f;
-          const float hv = g / (1.f + expf(-g)) * u * w;
+          const float hv = g / (1.f + expf(-g)) * u * wts[t][i];
           a.H[(size_t)entry * a.N + row_of[jt]] = __builtin_bit_cast(uint16_t, (_Float16)hv);
         } else {
           a.Z[(size_t)entry * a.N + row_of[jt]] = acc[t][jt][i];
@@ -326,21 +380,6 @@ __device__ __forceinline__ void pf_block_run(const PfBlkArgs& a, uint32_t* smem,
       }
     }
   }
-}
-
-template <class B, bool GU>
-__global__ __launch_bounds__(kPfBlkThreads) void moe_pf_block_kernel(const PfBlkArgs a) {
-  extern __shared__ __attribute__((aligned(16))) uint32_t smem[];
-  // consecutive workgroups land on different XCDs: the row chunks of one item stay on one XCD (shared L2 for its
-  // activations), and items -- sorted by size -- are dealt round-robin over the XCDs
-  const uint32_t xcd = blockIdx.x & 7u, slot = blockIdx.x >> 3;
-  const uint32_t item = (slot / a.row_chunks) * 8u + xcd, rc = slot % a.row_chunks;
-  if (item >= a.nitems) return;
-  const uint32_t e = a.items[3 * item], t0 = a.items[3 * item + 1], cnt = a.items[3 * item + 2];
-  const uint32_t base = a.offs[e] + t0;
-  if (cnt <= 16) pf_block_run<B, GU, 1>(a, smem, e, base, cnt, rc);
-  else if (cnt <= 32) pf_block_run<B, GU, 2>(a, smem, e, base, cnt, rc);
-  else pf_block_run<B, GU, 3>(a, smem, e, base, cnt, rc);
 }
 
 // Xg[i] = fp16(X[src(i)]): i < total gathers token tok[i]; rows total .. total + n - 1 are the tokens themselves

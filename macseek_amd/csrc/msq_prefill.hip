@@ -44,25 +44,38 @@ int launch_gemm_t(hipStream_t st, PfArgs a, int cus) {
   MSQ_HIP(hipGetLastError());
   return MSQ_OK;
 }
-template <class B, bool GU>
-int launch_block_t(hipStream_t st, PfBlkArgs a) {
-  const size_t lds = (size_t)B::LDS_WORDS * 4 + (size_t)kPfBlkTokens * kPfBlkPitch;
-  const uint32_t rows_per_item = GU ? kPfBlkRowsGU : kPfBlkRowsDown;
+template <class B, bool GU, int T>
+int launch_block_tt(hipStream_t st, PfBlkArgs a) {
+  if (!a.nitems) return MSQ_OK;
+  const uint32_t rows_per_item = pf_blk_rows(GU, T);
   a.row_chunks = (a.N + rows_per_item - 1) / rows_per_item;
   static bool attr_set = false;  // per instantiation: allow more than 64 KiB of dynamic LDS
   if (!attr_set) {
-    MSQ_HIP(hipFuncSetAttribute((const void*)moe_pf_block_kernel<B, GU>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+    MSQ_HIP(hipFuncSetAttribute((const void*)moe_pf_block_kernel<B, GU, T>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
     attr_set = true;
   }
   const uint32_t grid = ((a.nitems + 7) / 8) * 8 * a.row_chunks;
-  hipLaunchKernelGGL((moe_pf_block_kernel<B, GU>), dim3(grid), dim3(kPfBlkThreads), lds, st, a);
+  hipLaunchKernelGGL((moe_pf_block_kernel<B, GU, T>), dim3(grid), dim3(64 * pf_blk_waves(T)), pf_blk_lds<B>(), st, a);
   MSQ_HIP(hipGetLastError());
   return MSQ_OK;
 }
+// items are sorted by size, largest first: n3 items of three token tiles, then n2 of two, then the one-tile items
+template <class B, bool GU>
+int launch_block_t(hipStream_t st, PfBlkArgs a, uint32_t n3, uint32_t n2) {
+  const uint32_t* items = a.items;
+  const uint32_t n = a.nitems;
+  int rc;
+  a.items = items; a.nitems = n3;
+  if ((rc = launch_block_tt<B, GU, 3>(st, a))) return rc;
+  a.items = items + 3 * (size_t)n3; a.nitems = n2;
+  if ((rc = launch_block_tt<B, GU, 2>(st, a))) return rc;
+  a.items = items + 3 * (size_t)(n3 + n2); a.nitems = n - n3 - n2;
+  return launch_block_tt<B, GU, 1>(st, a);
+}
 bool block_path(int t) { return t == MSQ_IQ1_S || t == MSQ_IQ2_XXS; }
 template <bool GU>
-int launch_block(int t, hipStream_t st, const PfBlkArgs& a) {
-  return t == MSQ_IQ1_S ? launch_block_t<BlkIQ1S, GU>(st, a) : launch_block_t<BlkIQ2XXS, GU>(st, a);
+int launch_block(int t, hipStream_t st, const PfBlkArgs& a, uint32_t n3, uint32_t n2) {
+  return t == MSQ_IQ1_S ? launch_block_t<BlkIQ1S, GU>(st, a, n3, n2) : launch_block_t<BlkIQ2XXS, GU>(st, a, n3, n2);
 }
 
 template <bool GU>
@@ -159,18 +172,24 @@ int msq_moe_prefill(void* stream, const MsqMoePrefillArgs* p) {
   // work items of the block GEMM: blocks of up to 64 entries, largest first (they take longest)
   uint32_t* items = tiles + 2 * (size_t)(nt_routed + nt_shared);
   uint32_t ni_routed = 0, ni_shared = 0;
+  uint32_t n3_routed = 0, n2_routed = 0, n3_shared = 0, n2_shared = 0;  // items of three / two token tiles
   {
     std::vector<std::array<uint32_t, 3>> v;
     for (int j = 0; j < ne; j++)
       for (int t0 = 0; t0 < p->offs[j + 1] - p->offs[j]; t0 += kPfBlkTokens)
         v.push_back({(uint32_t)j, (uint32_t)t0, (uint32_t)std::min(kPfBlkTokens, p->offs[j + 1] - p->offs[j] - t0)});
     std::stable_sort(v.begin(), v.end(), [](const auto& x, const auto& y) { return x[2] > y[2]; });
-    for (const auto& it : v) { std::copy(it.begin(), it.end(), items + 3 * (size_t)ni_routed); ni_routed++; }
+    for (const auto& it : v) {
+      std::copy(it.begin(), it.end(), items + 3 * (size_t)ni_routed);
+      ni_routed++;
+      n3_routed += it[2] > 32; n2_routed += it[2] > 16 && it[2] <= 32;
+    }
     if (p->has_shared)
       for (int t0 = 0; t0 < n; t0 += kPfBlkTokens) {
         uint32_t* it = items + 3 * (size_t)(ni_routed + ni_shared);
         it[0] = (uint32_t)ne; it[1] = (uint32_t)t0; it[2] = (uint32_t)std::min(kPfBlkTokens, n - t0);
         ni_shared++;
+        n3_shared += it[2] > 32; n2_shared += it[2] > 16 && it[2] <= 32;
       }
   }
   uint8_t* sc = bptr_mut(&p->scratch);
@@ -212,7 +231,7 @@ int msq_moe_prefill(void* stream, const MsqMoePrefillArgs* p) {
     if (block_path(type)) {
       b.A = A; b.K = K; b.N = N; b.nblocks = K / 256; b.row_bytes = (uint32_t)row_bytes;
       b.items = d_items + (shared ? 3 * (size_t)ni_routed : 0); b.nitems = shared ? ni_shared : ni_routed;
-      return launch_block<GU>(type, st, b);
+      return launch_block<GU>(type, st, b, shared ? n3_shared : n3_routed, shared ? n2_shared : n2_routed);
     }
     a.A = A; a.N = N; steps(K); a.row_bytes = (uint32_t)row_bytes;
     a.tiles = d_tiles + (shared ? 2 * (size_t)nt_routed : 0); a.ntiles = shared ? nt_shared : nt_routed;
