@@ -269,11 +269,15 @@ struct BlkIQ2XXS {
   }
   __device__ static float scale(const Raw& r) { return half_bits_to_float(r.d) * 0.125f; }  // db = d (2 s + 1) / 8
   struct Look { uint4 g, s; };
+  // byte offsets in the replicated tables: entry << 8 | column << 4
   __device__ static Look lookup(const Raw& r, int j, const uint32_t* tbl, uint32_t col) {
     const uint32_t a0 = r.w[2 * (j >> 2)], a1 = r.w[2 * (j >> 2) + 1];
     const int l = j & 3;
-    const uint4* t4 = (const uint4*)tbl;
-    return {t4[(((a0 >> (8 * l)) & 0xFFu) << 4) | col], t4[MSQ_IQ2XXS_GRID_N * 16 + ((((a1 >> (7 * l)) & 127u) << 4) | col)]};
+    const uint32_t cg = col << 4, cs = cg | (MSQ_IQ2XXS_GRID_N * 256u);
+    const uint32_t g8 = l == 0 ? a0 << 8 : l == 1 ? a0 : a0 >> (8 * l - 8);    // grid index byte at bits 8..15
+    const uint32_t s8 = 7 * l < 8 ? a1 << (8 - 7 * l) : a1 >> (7 * l - 8);     // sign index at bits 8..14
+    const uint8_t* t8 = (const uint8_t*)tbl;
+    return {*(const uint4*)(t8 + ((g8 & 0xFF00u) | cg)), *(const uint4*)(t8 + ((s8 & 0x7F00u) | cs))};
   }
   __device__ static void finish(const Raw& r, int j, const Look& k, uint32_t (&h)[4]) {
     const uint32_t a1 = r.w[2 * (j >> 2) + 1];

@@ -202,17 +202,17 @@ struct PfBlkArgs {
 };
 
 constexpr int kPfBlkTokens = 48, kPfBlkPitch = 256 * 2 + 16;
-// waves per workgroup by token tiles per item: the one-tile variant needs few registers and runs four waves per SIMD
-// (it is the one that streams weights fastest and has the least matrix work to hide latency behind)
-constexpr int pf_blk_waves(int T) { return T == 1 ? 16 : 8; }
-// weight-row tiles per wave (the one-tile variant takes half as many to stay within its registers)
-constexpr int pf_blk_rt(bool gu, int T) { return (gu ? 2 : 4) / (T == 1 ? 2 : 1); }
+// waves per workgroup by token tiles per item: four per SIMD for the one-tile variant, three for the others
+constexpr int pf_blk_waves(int) { return 16; }
+// weight-row tiles per wave: two fragments per K step (gate + up of one tile, or two tiles of the down matrix) keep
+// the register count low enough for three or four waves per SIMD, which is what overlaps decode, matrix and LDS work
+constexpr int pf_blk_rt(bool gu, int) { return gu ? 1 : 2; }
 constexpr int pf_blk_rows(bool gu, int T) { return pf_blk_waves(T) * pf_blk_rt(gu, T) * 16; }  // weight rows per work item
 template <class B>
 constexpr size_t pf_blk_lds() { return (size_t)B::LDS_WORDS * 4 + 2 * (size_t)kPfBlkTokens * kPfBlkPitch; }
 
 template <class B, bool GU, int T>
-__global__ __launch_bounds__(64 * pf_blk_waves(T)) void moe_pf_block_kernel(const PfBlkArgs a) {
+__device__ __forceinline__ void pf_block_body(const PfBlkArgs& a) {
   constexpr int WAVES = pf_blk_waves(T), NT = 64 * WAVES;
   constexpr int NM = GU ? 2 : 1, RT = pf_blk_rt(GU, T), R = RT * NM, PITCH = kPfBlkPitch;
   constexpr int ABUF = kPfBlkTokens * PITCH;
@@ -309,7 +309,7 @@ __global__ __launch_bounds__(64 * pf_blk_waves(T)) void moe_pf_block_kernel(cons
         nxt[p / 2 - 1] = B::load(wrow[p / 2 - 1] + (size_t)kn * B::BLOCK_BYTES, q);
         __builtin_amdgcn_sched_barrier(0);
       }
-      if (p % PPS == 0 && T < 3) {  // activations of step j, read with the fragments' column mapping
+      if (p % PPS == 0) {  // activations of step j, read with the fragments' column mapping
 #pragma unroll
         for (int t = 0; t < T; t++) {
           const uint4 av = *(const uint4*)(arow + t * 16 * PITCH + 2u * blk_col_of(q, j));
@@ -329,13 +329,8 @@ __global__ __launch_bounds__(64 * pf_blk_waves(T)) void moe_pf_block_kernel(cons
       B::finish(cur[r0 + 1], j, lk[p & 1][1], h[1]);
 #pragma unroll
       for (int t = 0; t < T; t++) {
-        if (T >= 3) {  // short of registers: each tile's activations are read right before their use
-          const uint4 av = *(const uint4*)(arow + t * 16 * PITCH + 2u * blk_col_of(q, j));
-          af[0][0] = av.x; af[0][1] = av.y; af[0][2] = av.z; af[0][3] = av.w;
-        }
-        const uint32_t(&x)[4] = af[T >= 3 ? 0 : t];
-        blk[t][r0] = mfma_f16(x, h[0], j == 0 ? zero : blk[t][r0]);
-        blk[t][r0 + 1] = mfma_f16(x, h[1], j == 0 ? zero : blk[t][r0 + 1]);
+        blk[t][r0] = mfma_f16(af[t], h[0], j == 0 ? zero : blk[t][r0]);
+        blk[t][r0 + 1] = mfma_f16(af[t], h[1], j == 0 ? zero : blk[t][r0 + 1]);
       }
     }
 #pragma unroll
@@ -379,6 +374,20 @@ __global__ __launch_bounds__(64 * pf_blk_waves(T)) void moe_pf_block_kernel(cons
         }
       }
     }
+  }
+}
+
+// Kernel variants: T = 1 takes the items of one token tile (16 waves); T = 3 takes the larger ones, two or three
+// tiles each (8 waves), so that they share one launch and its tail.
+template <class B, bool GU, int T>
+__global__ __launch_bounds__(64 * pf_blk_waves(T)) void moe_pf_block_kernel(const PfBlkArgs a) {
+  if constexpr (T == 1) {
+    pf_block_body<B, GU, 1>(a);
+  } else {
+    const uint32_t item = ((blockIdx.x >> 3) / a.row_chunks) * 8u + (blockIdx.x & 7u);
+    if (item >= a.nitems) return;
+    if (a.items[3 * item + 2] > 32) pf_block_body<B, GU, 3>(a);
+    else pf_block_body<B, GU, 2>(a);
   }
 }
 

@@ -65,10 +65,8 @@ int launch_block_t(hipStream_t st, PfBlkArgs a, uint32_t n3, uint32_t n2) {
   const uint32_t* items = a.items;
   const uint32_t n = a.nitems;
   int rc;
-  a.items = items; a.nitems = n3;
+  a.items = items; a.nitems = n3 + n2;
   if ((rc = launch_block_tt<B, GU, 3>(st, a))) return rc;
-  a.items = items + 3 * (size_t)n3; a.nitems = n2;
-  if ((rc = launch_block_tt<B, GU, 2>(st, a))) return rc;
   a.items = items + 3 * (size_t)(n3 + n2); a.nitems = n - n3 - n2;
   return launch_block_tt<B, GU, 1>(st, a);
 }
