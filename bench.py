@@ -29,6 +29,11 @@ METRIC = "MoE decode matvec GB/s (% of HBM peak) + prefill MoE GEMM TFLOP/s (% M
 HBM_PEAK_GBPS = 8000.0
 
 
+# HBM bytes per launch of the decode gate/up kernel, from the FETCH_SIZE / WRITE_SIZE counter runs of this workload
+# (KiB per dispatch, scaled by what the same counters read for a 1 GiB copy: x2.000 and x1.000): 42.87 MB + 0.06 MB
+GU_TRAFFIC_BYTES = 42935015
+
+
 def cores():
     try:
         n = len(os.sched_getaffinity(0))
@@ -209,7 +214,7 @@ def bench_moe_decode(torch, args):
                                "top-6 of a seeded softmax router + 1 shared IQ2_XXS expert, SwiGLU; fresh top-6 per step",
                    "bytes_per_step": step_bytes, "experts": NE, "top_k": TOPK, "dim": DIM, "inter": INTER},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBPS,
-                     "traffic": None, "kernel": "moe_gu_kernel<DecIQ1S,DecIQ2XXS>", "bytes_per_launch": gu_bytes,
+                     "traffic": GU_TRAFFIC_BYTES, "kernel": "moe_gu_kernel<DecIQ1S,DecIQ2XXS>", "bytes_per_launch": gu_bytes,
                      "avg_launch_us": gu_graph * 1e3,
                      "timing": "HIP event pair around one graph replay of %d back-to-back launches of this kernel" % n_ev,
                      "eager_event_pair_us": {"mean": gu_mean * 1e3, "median": gu_med * 1e3, "min": gu_min * 1e3},
@@ -353,10 +358,11 @@ def bench_moe_prefill(torch, steps, warmup, with_cpu=True):
                    "tokens_per_expert_median": float(np.median(counts[used])), "flops_per_step": flops,
                    "weight_bytes_touched": int(len(used)) * per_exp},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": achieved / MFMA_PEAK_TFLOPS,
-                     "traffic": None, "kernel": "moe_pf_gemm_kernel<FragIQ2XXS,gate/up>", "flops_per_launch": gu_flops,
+                     "traffic": None, "kernel": "moe_pf_block_kernel<BlkIQ2XXS, gate/up> (two launches: multi-tile items, one-tile items)",
+                     "flops_per_launch": gu_flops,
                      "avg_launch_us": gu_mean * 1e3, "min_launch_us": gu_min * 1e3,
                      "weight_GBps": int(len(used)) * 2 * gu_b / (gu_mean * 1e-3) / 1e9,
-                     "second_kernel": {"kernel": "moe_pf_gemm_kernel<FragIQ2XXS,down>", "avg_launch_us": dn_mean * 1e3,
+                     "second_kernel": {"kernel": "moe_pf_block_kernel<BlkIQ2XXS, down> (two launches)", "avg_launch_us": dn_mean * 1e3,
                                        "achieved": 2.0 * DIM * INTER * total / (dn_mean * 1e-3) / 1e12}},
         "pct_of_mfma_peak": 100 * value / MFMA_PEAK_TFLOPS,
     }
@@ -381,13 +387,68 @@ def bench_moe_prefill(torch, steps, warmup, with_cpu=True):
     return out
 
 
+# ------------------------------------------------------------------------------------------------ stream / copy references
+def bench_stream(torch, args):
+    """Plain streaming reads (msq_bw_probe: every lane sums 128-bit loads) at a few sizes: what this device delivers to
+    a kernel that does nothing but read, next to the 8 TB/s the rooflines are priced against."""
+    from macseek_amd import _lib
+    from macseek_amd import quant as q
+    L = _lib.load()
+    dev = torch.device("cuda:0")
+    arena = torch.randint(0, 256, (3 << 30,), dtype=torch.uint8, device=dev)
+    sink = torch.zeros(4096, dtype=torch.uint8, device=dev)
+    sb = q.Buffer.of(sink).c()
+    rows = []
+    for mb in (21, 42, 63, 256, 1024):
+        nbytes = mb << 20
+        ncopies = (3 << 30) // nbytes  # successive launches read different memory: nothing is served from a cache
+        bufs = [q.Buffer.of(arena).sub(i * nbytes, nbytes).c() for i in range(ncopies)]
+
+        def launch(i):
+            rc = L.msq_bw_probe(C.c_void_p(torch.cuda.current_stream().cuda_stream), C.byref(bufs[i % ncopies]), nbytes, C.byref(sb))
+            if rc != 0:
+                raise RuntimeError(L.msq_last_error().decode())
+        ms = graph_ms_per_launch(torch, launch, min(200, max(20, 3 * ncopies)))
+        rows.append({"MiB": mb, "us_per_launch": ms * 1e3, "GBps": nbytes / (ms * 1e-3) / 1e9})
+    best = max(r["GBps"] for r in rows)
+    return {"value": best, "ms_per_step": rows[-1]["us_per_launch"] * 1e-3, "dtype": "u8",
+            "config": {"workload": "streaming read probe (bw_probe_kernel), sizes in MiB, launches back to back in a graph", "sizes": rows},
+            "roofline": {"bound": "hbm", "achieved": best, "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": best / HBM_PEAK_GBPS,
+                         "traffic": None, "kernel": "bw_probe_kernel"},
+            "cpu_baseline": None, "pct_of_hbm_peak": 100 * best / HBM_PEAK_GBPS}
+
+
+def bench_copy_calibration(torch, args):
+    """A device-to-device copy of known size (1 GiB read, 1 GiB written per launch): the reference that the FETCH_SIZE /
+    WRITE_SIZE counters of a profiling run are scaled by."""
+    dev = torch.device("cuda:0")
+    n = 1 << 30
+    src = torch.randint(0, 256, (n,), dtype=torch.uint8, device=dev)
+    dst = torch.empty_like(src)
+    for _ in range(3):
+        dst.copy_(src)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    reps = 10
+    for _ in range(reps):
+        dst.copy_(src)
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / reps
+    gbps = 2 * n / (ms * 1e-3) / 1e9
+    return {"value": gbps, "ms_per_step": ms, "dtype": "u8",
+            "config": {"workload": "device-to-device copy, 1 GiB read + 1 GiB written per launch (counter calibration)", "bytes_read": n, "bytes_written": n},
+            "roofline": {"bound": "hbm", "achieved": gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": gbps / HBM_PEAK_GBPS, "traffic": 2 * n,
+                         "kernel": "torch elementwise copy"},
+            "cpu_baseline": None, "pct_of_hbm_peak": 100 * gbps / HBM_PEAK_GBPS}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=500)
     ap.add_argument("--warmup", type=int, default=100)
     ap.add_argument("--workload", default="moe_decode",
-                    choices=["moe_decode", "moe_prefill", "matvec_iq1s", "matvec_iq2xxs", "q8_0"])
+                    choices=["moe_decode", "moe_prefill", "matvec_iq1s", "matvec_iq2xxs", "q8_0", "stream", "copy_calibration"])
     ap.add_argument("--gpu-only", action="store_true",
                     help="profiling runs: skip the CPU baseline leg and the prefill appendix of the default workload")
     args = ap.parse_args()
@@ -414,6 +475,10 @@ def main():
         return
     if args.workload == "moe_decode":
         r = bench_moe_decode(torch, args)
+    elif args.workload == "stream":
+        r = bench_stream(torch, args)
+    elif args.workload == "copy_calibration":
+        r = bench_copy_calibration(torch, args)
     elif args.workload == "matvec_iq1s":
         r = bench_matvec(torch, args, q.QType.IQ1_S, 4096, 7168, 0.01, "BASELINE configs[1]: single-expert decode matvec IQ1_S 4096x7168, batch 1")
     elif args.workload == "matvec_iq2xxs":
