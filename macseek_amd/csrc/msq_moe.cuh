@@ -377,8 +377,9 @@ __device__ __forceinline__ void down_rows_ring(const uint32_t* tbl, const typena
   }
 }
 
-template <class DR, class DS>
-__global__ __launch_bounds__(1024) void moe_down_kernel(const MoeArgs a) {
+// MAXT: largest workgroup the instantiation is launched with (768 threads leave 170 registers per lane, 1024 only 128)
+template <class DR, class DS, int MAXT>
+__global__ __launch_bounds__(MAXT) void moe_down_kernel(const MoeArgs a) {
   constexpr bool RING_R = requires { DR::STAGES; }, RING_S = requires { DS::STAGES; };
   constexpr int RPW = rows_in_flight<DR>(1);
   constexpr int NR = MSQ_NRD, NSH = 4;  // ring depth: routed rows, shared rows

@@ -17,7 +17,8 @@ void launch_gu_t(dim3 g, dim3 b, size_t lds, hipStream_t st, const MoeArgs& a) {
 }
 template <class DR, class DS>
 void launch_down_t(dim3 g, dim3 b, size_t lds, hipStream_t st, const MoeArgs& a) {
-  hipLaunchKernelGGL((moe_down_kernel<DR, DS>), g, b, lds, st, a);
+  if (b.x <= 768) hipLaunchKernelGGL((moe_down_kernel<DR, DS, 768>), g, b, lds, st, a);
+  else hipLaunchKernelGGL((moe_down_kernel<DR, DS, 1024>), g, b, lds, st, a);
 }
 // launch-shape knobs for experiments (the reference exposes MACSEEK_MOE_* the same way, quant.mm:274-276)
 int env_int(const char* name, int dflt) {
