@@ -13,18 +13,6 @@
 // order and run the epilogue.
 #pragma once
 #include "msq_device.cuh"
-#ifndef MSQ_EXP
-#define MSQ_EXP 0
-#endif
-#ifndef MSQ_NOPIPE
-#define MSQ_NOPIPE 0
-#endif
-#ifndef MSQ_NR
-#define MSQ_NR 4
-#endif
-#ifndef MSQ_NRD
-#define MSQ_NRD 4
-#endif
 
 namespace msq {
 
@@ -178,7 +166,7 @@ __device__ __forceinline__ void moe_gu_run_direct(const MoeArgs& a, uint32_t* sm
 // products (two alternating lookup buffers), so LDS latency overlaps the math as well.
 template <class D>
 __device__ __forceinline__ void moe_gu_run_ring(const MoeArgs& a, uint32_t* smem, const bool shared, const uint32_t wg) {
-  constexpr int NR = MSQ_NR;  // row pairs in flight per wave
+  constexpr int NR = 4;  // row pairs in flight per wave
   constexpr int NS = D::STAGES;
   uint32_t* tbl = smem;
   float* part = (float*)(smem + D::LDS_WORDS);
@@ -200,16 +188,6 @@ __device__ __forceinline__ void moe_gu_run_ring(const MoeArgs& a, uint32_t* smem
 
   typename D::X xr;
   bool first = true;
-#if MSQ_EXP == 5
-  return;
-#endif
-#if MSQ_EXP == 6
-  D::fill_lds(tbl, (int)tid, (int)blockDim.x);
-  xr = D::load_x(a.x, unit);
-  __syncthreads();
-  if (xr.sx == 1.2345f) a.h[0] = tbl[tid];
-  return;
-#endif
   for (uint32_t c0 = wg_begin; c0 < wg_end; c0 += kMoeChunkRows) {
     const uint32_t c1 = min(wg_end, c0 + kMoeChunkRows), n = c1 - c0;
     const uint32_t run = uniform((n + RW - 1) / RW);  // divisions run on the vector unit: bring the results back
@@ -246,16 +224,8 @@ __device__ __forceinline__ void moe_gu_run_ring(const MoeArgs& a, uint32_t* smem
       __syncthreads();
       first = false;
     }
-#if MSQ_EXP == 7
-    { uint32_t sm_ = 0;
-      for (int s_ = 0; s_ < NR; s_++) { uint32_t w_[sizeof(typename D::Raw) / 4]; __builtin_memcpy(w_, &rg[s_], sizeof(w_)); sm_ += w_[0]; __builtin_memcpy(w_, &ru[s_], sizeof(w_)); sm_ += w_[0]; }
-      if (sm_ == 0x12345u && xr.sx == 1.2345f) a.h[0] = 1.f;
-      return; }
-#endif
     typename D::Look lk[2];  // stage t of a row pair uses lk[t & 1]; 2 NS stages per row pair keep the parity fixed
-#if !MSQ_NOPIPE
     if (w0 < w1) lk[0] = D::lookup(rg[0], 0, tbl);
-#endif
     for (uint32_t r0 = w0; r0 < w1; r0 += NR) {
 #pragma unroll
       for (int half = 0; half < 2; half++) {
@@ -272,13 +242,8 @@ __device__ __forceinline__ void moe_gu_run_ring(const MoeArgs& a, uint32_t* smem
               const bool up = t >= NS;
               const int st = up ? t - NS : t;
               // issue the next stage's table reads, then consume this stage's
-#if MSQ_NOPIPE
-              lk[t & 1] = D::lookup(up ? ru[s] : rg[s], st, tbl);
-              (void)more;
-#else
               if (t + 1 < 2 * NS) lk[(t + 1) & 1] = D::lookup(t + 1 >= NS ? ru[s] : rg[s], t + 1 >= NS ? t + 1 - NS : t + 1, tbl);
               else if (more) lk[0] = D::lookup(rg[(s + 1) % NR], 0, tbl);
-#endif
               if (up) { u = D::partial(ru[s], lk[t & 1], xr, st, u); asm volatile("" : "+v"(u)); }
               else { g = D::partial(rg[s], lk[t & 1], xr, st, g); asm volatile("" : "+v"(g)); }
             }
@@ -349,10 +314,6 @@ __device__ __forceinline__ void down_rows_ring(const uint32_t* tbl, const typena
         const int s = half * 4 + j;
         const uint32_t row = r0 + s * step;
         float v = 0.f;
-#if MSQ_EXP == 12
-        if (row < end) { uint32_t w_[sizeof(typename D::Raw) / 4]; __builtin_memcpy(w_, &ring[s], sizeof(w_)); v = (float)(w_[0] + w_[1]); }
-        else
-#endif
         if (row < end) {  // wave-uniform; no global loads inside
           const bool more = row + step < end;
 #pragma unroll
@@ -382,7 +343,7 @@ template <class DR, class DS, int MAXT>
 __global__ __launch_bounds__(MAXT) void moe_down_kernel(const MoeArgs a) {
   constexpr bool RING_R = requires { DR::STAGES; }, RING_S = requires { DS::STAGES; };
   constexpr int RPW = rows_in_flight<DR>(1);
-  constexpr int NR = MSQ_NRD, NSH = 4;  // ring depth: routed rows, shared rows
+  constexpr int NR = 4, NSH = 4;  // ring depth: routed rows, shared rows
   extern __shared__ __attribute__((aligned(16))) uint32_t smem[];
   constexpr int TBL = DR::LDS_WORDS + DS::LDS_WORDS;
   uint32_t* tbl_r = smem;
@@ -463,10 +424,6 @@ __global__ __launch_bounds__(MAXT) void moe_down_kernel(const MoeArgs a) {
       __syncthreads();
       first = false;
     }
-#if MSQ_EXP == 11
-    if (xr.sx == 1.2345f) a.y[0] = 1.f;
-    return;
-#endif
     // ---- routed expert e, rows w0 .. w1
     if (NE) {
       if constexpr (RING_R) {

@@ -17,9 +17,6 @@
 #include <type_traits>
 
 #include "msq_mfma.cuh"
-#ifndef MSQ_EXP
-#define MSQ_EXP 0
-#endif
 
 namespace msq {
 
