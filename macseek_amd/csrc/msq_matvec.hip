@@ -53,13 +53,21 @@ bool mv_shape(int t, int rows, int cols, int groups, const MsqMvCfg* cfg, MvShap
     while (iters < 4 && units > 64 * ks * iters) iters *= 2;
   }
   if (ks > 16 || units > 64 * ks * iters) return false;
-  int rw = std::max(1, 8 / ks);
+  // the codebook formats stage a table of up to 32 KB per workgroup: one 16-wave workgroup per CU, each wave a run of
+  // rows long enough for its register ring; the others run several small workgroups per CU
+  const bool table = t == MSQ_IQ1_S || t == MSQ_IQ2_XXS;
+  int rw = std::max(1, (table ? 16 : 8) / ks);
   if (cfg && cfg->rsg > 0) rw = cfg->rsg;
   if (rw * ks > 16) rw = std::max(1, 16 / ks);
   const int rpg = rows / groups;
-  // rows per wave per tile: enough tiles to fill the chip a few times over, at most 8 rows per wave
-  int rpw = 8;
-  while (rpw > 1 && (long)rows / (rw * rpw) < 2048) rpw /= 2;
+  int rpw;
+  if (table) {  // about one tile per CU
+    const long per_cu = ((long)rows + device_info().cus - 1) / device_info().cus;
+    rpw = (int)std::min<long>(64, std::max<long>(1, (per_cu + rw - 1) / rw));
+  } else {  // rows per wave per tile: enough tiles to fill the chip a few times over, at most 8 rows per wave
+    rpw = 8;
+    while (rpw > 1 && (long)rows / (rw * rpw) < 2048) rpw /= 2;
+  }
   if (cfg && cfg->nr > 0) rpw = std::min(cfg->nr, 64);
   if (groups > 1) {  // every tile must stay inside one block-diagonal group
     while (rpw > 1 && rpg % (rw * rpw)) rpw /= 2;
@@ -82,6 +90,13 @@ int launch_mv(hipStream_t st, const MvShape& s, MvArgs& a) {
   // persistent workgroups: as many as can be resident, never more than there are tiles
   const int wg_per_cu = std::max(1, std::min(2048 / threads, (int)((160 * 1024) / std::max<size_t>(lds, 1))));
   const int grid = (int)std::min<long>(a.ntiles, (long)device_info().cus * wg_per_cu);
+  if constexpr (requires { D::STAGES; }) {  // codebook formats: ring kernel (one unit per lane, matrix below 4 GiB)
+    if (s.iters == 1 && (uint64_t)a.rows * a.row_bytes < (1ull << 32)) {
+      hipLaunchKernelGGL((mv_ring_kernel<D>), dim3(grid), dim3(threads), lds, st, a);
+      MSQ_HIP(hipGetLastError());
+      return MSQ_OK;
+    }
+  }
   switch (s.iters) {
     case 1: hipLaunchKernelGGL((mv_kernel<D, 1>), dim3(grid), dim3(threads), lds, st, a); break;
     case 2: hipLaunchKernelGGL((mv_kernel<D, 2>), dim3(grid), dim3(threads), lds, st, a); break;

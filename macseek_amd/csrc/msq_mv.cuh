@@ -6,6 +6,8 @@
 // the only HBM stream. Workgroups are persistent (grid-stride over row tiles) so codebook tables are staged into LDS
 // once per workgroup. K-split partial sums meet in LDS and are added in a fixed order.
 #pragma once
+#include <array>
+
 #include "msq_device.cuh"
 
 namespace msq {
@@ -85,6 +87,102 @@ __global__ __launch_bounds__(1024) void mv_kernel(const MvArgs a) {
           float s = 0.f;
           for (uint32_t k = 0; k < KS; k++) s += part[tid * KS + k];
           a.y[row] = a.accumulate ? a.y[row] + s : s;
+        }
+      }
+      __syncthreads();
+    }
+  }
+}
+
+// The same matvec with one unit per lane, arranged like the MoE decode kernels: a wave keeps the block bytes of NR rows
+// in flight in a register ring that is refilled unconditionally (codebook decoders: range-checked buffer loads with an
+// empty descriptor past the end of the wave's rows; the others: the last row again), the first NR rows before the
+// tables and activations are staged; codebook table lookups run one decoder stage ahead of the dot products. With a handful of rows
+// per wave per launch it is the latency of the first loads, not bandwidth, that such a launch spends its time on.
+template <class D>
+__global__ __launch_bounds__(1024) void mv_ring_kernel(const MvArgs a) {
+  constexpr bool BUFFER = requires { D::STAGES; };  // codebook decoders: buffer loads and staged table lookups
+  constexpr int NR = 4;
+  extern __shared__ __attribute__((aligned(16))) uint32_t smem[];
+  uint32_t* tbl = smem;
+  float* part = (float*)(smem + D::LDS_WORDS);
+
+  const uint32_t tid = threadIdx.x, lane = tid & 63u, nwaves = blockDim.x >> 6;
+  const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
+  const uint32_t KS = a.ks, ks = wave % KS, rw = wave / KS, RW = nwaves / KS;
+  const uint32_t tile_rows = RW * a.rpw;
+  const uint32_t u0 = ks * 64u + lane;
+  const bool valid = u0 < a.units;
+  const uint32_t unit = valid ? u0 : a.units - 1;  // lanes past the row shadow the last unit with zero activations
+  const auto off = [&] { if constexpr (BUFFER) return D::offsets(unit); else return 0; }();
+  const uint32_t mat_bytes = a.rows * a.row_bytes;  // buffer loads: < 4 GiB (host-checked)
+
+  typename D::X xr;
+  uint32_t cur_group = 0xFFFFFFFFu;
+  bool first = true;
+  for (uint32_t tile = blockIdx.x; tile < a.ntiles; tile += gridDim.x) {
+    const uint32_t tile_row0 = tile * tile_rows;
+    const uint32_t row0 = tile_row0 + rw * a.rpw, row1 = min(row0 + a.rpw, a.rows);
+    uint32_t pv = row0;
+    typename D::Raw ring[NR];
+    auto fetch = [&](int s) {
+      if constexpr (BUFFER) ring[s] = D::fetch(make_rsrc(a.W, pv < row1 ? mat_bytes : 0u), off, pv * a.row_bytes);
+      else ring[s] = D::load(as_global(a.W) + (size_t)min(pv, a.rows - 1) * a.row_bytes, unit);  // past the end: the last row again
+      pv++;
+    };
+#pragma unroll
+    for (int s = 0; s < NR; s++) fetch(s);
+    if (first) {
+      D::fill_lds(tbl, (int)tid, (int)blockDim.x);
+      first = false;
+      if (D::LDS_WORDS) __syncthreads();
+    }
+    const uint32_t group = tile_row0 / a.rows_per_group;  // a tile never straddles two groups (host guarantees)
+    if (group != cur_group) {
+      xr = D::load_x(a.x + (size_t)group * a.x_group_stride, unit);
+      if (!valid) xr = typename D::X{};
+      cur_group = group;
+    }
+    auto lk = [&] { if constexpr (BUFFER) return std::array<typename D::Look, 2>{}; else return 0; }();
+    if constexpr (BUFFER) { if (row0 < row1) lk[0] = D::lookup(ring[0], 0, tbl); }
+    for (uint32_t r0 = row0; r0 < row1; r0 += NR) {
+#pragma unroll
+      for (int s = 0; s < NR; s++) {
+        const uint32_t row = r0 + s;
+        if (row < row1) {  // wave-uniform; no global loads inside
+          float v = 0.f;
+          if constexpr (BUFFER) {
+            constexpr int NS = D::STAGES;
+            const bool more = row + 1 < row1;
+#pragma unroll
+            for (int t = 0; t < NS; t++) {
+              const int cur = (s * NS + t) & 1;
+              if (t + 1 < NS) lk[cur ^ 1] = D::lookup(ring[s], t + 1, tbl);
+              else if (more) lk[cur ^ 1] = D::lookup(ring[(s + 1) % NR], 0, tbl);
+              v = D::partial(ring[s], lk[cur], xr, t, v);
+              asm volatile("" : "+v"(v));
+            }
+          } else {
+            v = dec_dot<D>(ring[s], xr, tbl, unit);
+          }
+          v = wave_sum(valid ? v : 0.f);
+          if (KS == 1) {
+            if (lane == 0) a.y[row] = a.accumulate ? a.y[row] + v : v;
+          } else if (lane == 0) {
+            part[(row - tile_row0) * KS + ks] = v;
+          }
+        }
+        fetch(s);
+      }
+    }
+    if (KS > 1) {
+      __syncthreads();
+      if (tid < tile_rows) {
+        const uint32_t row = tile_row0 + tid;
+        if (row < a.rows) {
+          float sum = 0.f;
+          for (uint32_t k = 0; k < KS; k++) sum += part[tid * KS + k];
+          a.y[row] = a.accumulate ? a.y[row] + sum : sum;
         }
       }
       __syncthreads();
