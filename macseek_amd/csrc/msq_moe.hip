@@ -130,7 +130,10 @@ int moe_decode_impl(hipStream_t st, const MsqMoeDecodeArgs* p, const MsqBuffer* 
     // persistent workgroups, dealt to the routed experts and the shared expert in proportion to their bytes
     const long rows_r = (long)n_gu_r * inter, rows_s = gu_s ? inter : 0;
     const long total = std::max<long>(2, (long)cus * std::max(1, env_gu_wgs));
-    const double br = (double)n_gu_r * a.rb_gu_r, bs = gu_s ? (double)a.rb_gu_s : 0.0;
+    // ... weighted by the decode work per byte (IQ2_XXS takes two table lookups and sign flips per 8 weights: measured
+    // about 1.2x IQ1_S per byte)
+    auto cost = [](int t) { return t == MSQ_IQ2_XXS ? 1.2 : 1.0; };
+    const double br = (double)n_gu_r * a.rb_gu_r * cost(p->t_gate_up), bs = gu_s ? (double)a.rb_gu_s * cost(ts) : 0.0;
     long g_s = gu_s ? std::max<long>(1, (long)(total * bs / (br + bs) + 0.5)) : 0;
     long g_r = n_gu_r ? std::max<long>(1, total - g_s) : 0;
     if (g_r) { a.rows_per_wg_r = (uint32_t)((rows_r + g_r - 1) / g_r); g_r = (rows_r + a.rows_per_wg_r - 1) / a.rows_per_wg_r; }
