@@ -198,21 +198,23 @@ struct PfBlkArgs {
   uint32_t row_chunks;      // chunks of pf_blk_rows() weight rows
 };
 
-constexpr int kPfBlkTokens = 48, kPfBlkPitch = 256 * 2 + 16;
+constexpr int kPfBlkTokens = 48, kPfBigTokens = 80, kPfBlkPitch = 256 * 2 + 16;
 // waves per workgroup by token tiles per item: four per SIMD for the one-tile variant, three for the others
-constexpr int pf_blk_waves(int) { return 16; }
+constexpr int pf_blk_waves(int T) { return T > 3 ? 12 : 16; }
 // weight-row tiles per wave: two fragments per K step (gate + up of one tile, or two tiles of the down matrix) keep
 // the register count low enough for three or four waves per SIMD, which is what overlaps decode, matrix and LDS work
 constexpr int pf_blk_rt(bool gu, int) { return gu ? 1 : 2; }
 constexpr int pf_blk_rows(bool gu, int T) { return pf_blk_waves(T) * pf_blk_rt(gu, T) * 16; }  // weight rows per work item
+// activation staging: double-buffered for up to three token tiles, a single buffer (two barriers per block) for six
 template <class B>
-constexpr size_t pf_blk_lds() { return (size_t)B::LDS_WORDS * 4 + 2 * (size_t)kPfBlkTokens * kPfBlkPitch; }
+constexpr size_t pf_blk_lds(int T) { return (size_t)B::LDS_WORDS * 4 + (T > 3 ? 1 : 2) * (size_t)(T > 3 ? kPfBigTokens : kPfBlkTokens) * kPfBlkPitch; }
 
 template <class B, bool GU, int T>
 __device__ __forceinline__ void pf_block_body(const PfBlkArgs& a) {
   constexpr int WAVES = pf_blk_waves(T), NT = 64 * WAVES;
   constexpr int NM = GU ? 2 : 1, RT = pf_blk_rt(GU, T), R = RT * NM, PITCH = kPfBlkPitch;
-  constexpr int ABUF = kPfBlkTokens * PITCH;
+  constexpr bool DB = T <= 3;  // two activation buffers
+  constexpr int ABUF = (DB ? kPfBlkTokens : kPfBigTokens) * PITCH;
   constexpr int PPS = R / 2, NP = 8 * PPS;  // fragment pairs per K step, per block
   static_assert(R == 2 || R == 4, "fragments are processed in pairs");
   extern __shared__ __attribute__((aligned(16))) uint32_t smem[];
@@ -279,7 +281,7 @@ __device__ __forceinline__ void pf_block_body(const PfBlkArgs& a) {
 
   for (uint32_t kc = 0; kc < a.nblocks; kc++) {
     const uint32_t kn = kc + 1 < a.nblocks ? kc + 1 : kc;  // the last block fetches itself again: no branch around the loads
-    const uint8_t* arow = abuf + (kc & 1u) * ABUF + n16 * PITCH;
+    const uint8_t* arow = abuf + (DB ? (kc & 1u) * ABUF : 0u) + n16 * PITCH;
     f4_t blk[T][R];
     // table reads run one fragment pair ahead where registers allow (pair p = 2 j + half uses lk[p & 1]: fragments
     // 2 half, 2 half + 1 of step j): the one-tile variant has four waves per SIMD to hide them behind instead, the
@@ -290,7 +292,7 @@ __device__ __forceinline__ void pf_block_body(const PfBlkArgs& a) {
       lk[0][0] = B::lookup(cur[0], 0, tbl, n16);
       lk[0][1] = B::lookup(cur[1], 0, tbl, n16);
     }
-    uint32_t af[T][4];
+    uint32_t af[T > 3 ? 3 : T][4];
 #pragma unroll
     for (int p = 0; p < NP; p++) {
       const int j = p / PPS, r0 = 2 * (p % PPS);
@@ -306,7 +308,7 @@ __device__ __forceinline__ void pf_block_body(const PfBlkArgs& a) {
         nxt[p / 2 - 1] = B::load(wrow[p / 2 - 1] + (size_t)kn * B::BLOCK_BYTES, q);
         __builtin_amdgcn_sched_barrier(0);
       }
-      if (p % PPS == 0) {  // activations of step j, read with the fragments' column mapping
+      if (p % PPS == 0 && T <= 3) {  // activations of step j, read with the fragments' column mapping
 #pragma unroll
         for (int t = 0; t < T; t++) {
           const uint4 av = *(const uint4*)(arow + t * 16 * PITCH + 2u * blk_col_of(q, j));
@@ -326,8 +328,23 @@ __device__ __forceinline__ void pf_block_body(const PfBlkArgs& a) {
       B::finish(cur[r0 + 1], j, lk[p & 1][1], h[1]);
 #pragma unroll
       for (int t = 0; t < T; t++) {
-        blk[t][r0] = mfma_f16(af[t], h[0], j == 0 ? zero : blk[t][r0]);
-        blk[t][r0 + 1] = mfma_f16(af[t], h[1], j == 0 ? zero : blk[t][r0 + 1]);
+        if (T > 3) {  // six tiles: short of registers, each tile's activations are read two tiles ahead of their use
+          if (t == 0) {
+#pragma unroll
+            for (int u = 0; u < 2; u++) {
+              const uint4 av = *(const uint4*)(arow + u * 16 * PITCH + 2u * blk_col_of(q, j));
+              af[u][0] = av.x; af[u][1] = av.y; af[u][2] = av.z; af[u][3] = av.w;
+            }
+          }
+        }
+        const uint32_t(&x)[4] = af[T > 3 ? t % 3 : t];
+        if (T > 3 && t + 2 < T) {
+          const uint4 av = *(const uint4*)(arow + (t + 2) * 16 * PITCH + 2u * blk_col_of(q, j));
+          uint32_t(&y)[4] = af[(t + 2) % 3];
+          y[0] = av.x; y[1] = av.y; y[2] = av.z; y[3] = av.w;
+        }
+        blk[t][r0] = mfma_f16(x, h[0], j == 0 ? zero : blk[t][r0]);
+        blk[t][r0 + 1] = mfma_f16(x, h[1], j == 0 ? zero : blk[t][r0 + 1]);
       }
     }
 #pragma unroll
@@ -336,8 +353,10 @@ __device__ __forceinline__ void pf_block_body(const PfBlkArgs& a) {
 #pragma unroll
       for (int t = 0; t < T; t++) acc[t][r] += sc * blk[t][r];
     }
-    // the other activation buffer was last read one block ago, before the previous barrier: free to refill
-    a_store((kc & 1u) ^ 1u);
+    // the other activation buffer was last read one block ago, before the previous barrier: free to refill (with a
+    // single buffer every wave has to be done with the block first)
+    if (!DB) __syncthreads();
+    a_store(DB ? (kc & 1u) ^ 1u : 0u);
 #pragma unroll
     for (int r = 0; r < R; r++) cur[r] = nxt[r];
     __syncthreads();
@@ -374,12 +393,13 @@ __device__ __forceinline__ void pf_block_body(const PfBlkArgs& a) {
   }
 }
 
-// Kernel variants: T = 1 takes the items of one token tile (16 waves); T = 3 takes the larger ones, two or three
-// tiles each (8 waves), so that they share one launch and its tail.
+// Kernel variants: T = 1 takes the items of one token tile; T = 3 those of two or three tiles, so that they share one
+// launch and its tail; T = 6 the blocks of 49 to 96 entries that the popular experts are cut into (their weights are
+// then decoded half as often; 12 waves, one activation buffer).
 template <class B, bool GU, int T>
 __global__ __launch_bounds__(64 * pf_blk_waves(T)) void moe_pf_block_kernel(const PfBlkArgs a) {
-  if constexpr (T == 1) {
-    pf_block_body<B, GU, 1>(a);
+  if constexpr (T == 1 || T > 3) {
+    pf_block_body<B, GU, T>(a);
   } else {
     const uint32_t item = ((blockIdx.x >> 3) / a.row_chunks) * 8u + (blockIdx.x & 7u);
     if (item >= a.nitems) return;

@@ -13,7 +13,7 @@ namespace {
 size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
 size_t header_bytes(int total, int n, int n_exp) {
   const size_t tiles = (size_t)n_exp + total / 16 + n / 16 + 4;  // token tiles of up to 16 entries
-  const size_t items = (size_t)n_exp + total / kPfBlkTokens + n / kPfBlkTokens + 4;  // blocks of up to 64 entries
+  const size_t items = 2 * (size_t)n_exp + total / kPfBlkTokens + n / kPfBlkTokens + 4;  // blocks of up to 96 entries + remainders
   return align256(24 * (size_t)(n_exp + 1) + 4 * (size_t)(n_exp + 2) + 8 * tiles + 12 * items);
 }
 bool routed_ok(int t) { return t == MSQ_IQ1_S || t == MSQ_IQ2_XXS; }
@@ -55,25 +55,28 @@ int launch_block_tt(hipStream_t st, PfBlkArgs a) {
     attr_set = true;
   }
   const uint32_t grid = ((a.nitems + 7) / 8) * 8 * a.row_chunks;
-  hipLaunchKernelGGL((moe_pf_block_kernel<B, GU, T>), dim3(grid), dim3(64 * pf_blk_waves(T)), pf_blk_lds<B>(), st, a);
+  hipLaunchKernelGGL((moe_pf_block_kernel<B, GU, T>), dim3(grid), dim3(64 * pf_blk_waves(T)), pf_blk_lds<B>(T), st, a);
   MSQ_HIP(hipGetLastError());
   return MSQ_OK;
 }
-// items are sorted by size, largest first: n3 items of three token tiles, then n2 of two, then the one-tile items
+// items are sorted by size, largest first: n6 blocks of more than 48 entries, n3 items of three token tiles, n2 of two,
+// then the one-tile items
 template <class B, bool GU>
-int launch_block_t(hipStream_t st, PfBlkArgs a, uint32_t n3, uint32_t n2) {
+int launch_block_t(hipStream_t st, PfBlkArgs a, uint32_t n6, uint32_t n3, uint32_t n2) {
   const uint32_t* items = a.items;
   const uint32_t n = a.nitems;
   int rc;
-  a.items = items; a.nitems = n3 + n2;
+  a.items = items; a.nitems = n6;
+  if ((rc = launch_block_tt<B, GU, 5>(st, a))) return rc;
+  a.items = items + 3 * (size_t)n6; a.nitems = n3 + n2;
   if ((rc = launch_block_tt<B, GU, 3>(st, a))) return rc;
-  a.items = items + 3 * (size_t)(n3 + n2); a.nitems = n - n3 - n2;
+  a.items = items + 3 * (size_t)(n6 + n3 + n2); a.nitems = n - n6 - n3 - n2;
   return launch_block_tt<B, GU, 1>(st, a);
 }
 bool block_path(int t) { return t == MSQ_IQ1_S || t == MSQ_IQ2_XXS; }
 template <bool GU>
-int launch_block(int t, hipStream_t st, const PfBlkArgs& a, uint32_t n3, uint32_t n2) {
-  return t == MSQ_IQ1_S ? launch_block_t<BlkIQ1S, GU>(st, a, n3, n2) : launch_block_t<BlkIQ2XXS, GU>(st, a, n3, n2);
+int launch_block(int t, hipStream_t st, const PfBlkArgs& a, uint32_t n6, uint32_t n3, uint32_t n2) {
+  return t == MSQ_IQ1_S ? launch_block_t<BlkIQ1S, GU>(st, a, n6, n3, n2) : launch_block_t<BlkIQ2XXS, GU>(st, a, n6, n3, n2);
 }
 
 template <bool GU>
@@ -170,25 +173,29 @@ int msq_moe_prefill(void* stream, const MsqMoePrefillArgs* p) {
   // work items of the block GEMM: blocks of up to 64 entries, largest first (they take longest)
   uint32_t* items = tiles + 2 * (size_t)(nt_routed + nt_shared);
   uint32_t ni_routed = 0, ni_shared = 0;
-  uint32_t n3_routed = 0, n2_routed = 0, n3_shared = 0, n2_shared = 0;  // items of three / two token tiles
+  uint32_t nc_routed[3] = {0, 0, 0}, nc_shared[3] = {0, 0, 0};  // items of more than 48 entries / three tiles / two tiles
   {
-    std::vector<std::array<uint32_t, 3>> v;
-    for (int j = 0; j < ne; j++)
-      for (int t0 = 0; t0 < p->offs[j + 1] - p->offs[j]; t0 += kPfBlkTokens)
-        v.push_back({(uint32_t)j, (uint32_t)t0, (uint32_t)std::min(kPfBlkTokens, p->offs[j + 1] - p->offs[j] - t0)});
-    std::stable_sort(v.begin(), v.end(), [](const auto& x, const auto& y) { return x[2] > y[2]; });
-    for (const auto& it : v) {
-      std::copy(it.begin(), it.end(), items + 3 * (size_t)ni_routed);
-      ni_routed++;
-      n3_routed += it[2] > 32; n2_routed += it[2] > 16 && it[2] <= 32;
-    }
-    if (p->has_shared)
-      for (int t0 = 0; t0 < n; t0 += kPfBlkTokens) {
-        uint32_t* it = items + 3 * (size_t)(ni_routed + ni_shared);
-        it[0] = (uint32_t)ne; it[1] = (uint32_t)t0; it[2] = (uint32_t)std::min(kPfBlkTokens, n - t0);
-        ni_shared++;
-        n3_shared += it[2] > 32; n2_shared += it[2] > 16 && it[2] <= 32;
+    // an expert's entries are cut into blocks of 96 while more than 48 remain, then one block of at most 48
+    auto cut = [](std::vector<std::array<uint32_t, 3>>& v, uint32_t e, int m) {
+      int t0 = 0;
+      while (m - t0 > kPfBlkTokens) { const int c = std::min(kPfBigTokens, m - t0); v.push_back({e, (uint32_t)t0, (uint32_t)c}); t0 += c; }
+      if (m - t0 > 0) v.push_back({e, (uint32_t)t0, (uint32_t)(m - t0)});
+    };
+    auto emit = [&](std::vector<std::array<uint32_t, 3>>& v, uint32_t* dst, uint32_t* nc) {
+      std::stable_sort(v.begin(), v.end(), [](const auto& x, const auto& y) { return x[2] > y[2]; });
+      uint32_t k = 0;
+      for (const auto& it : v) {
+        std::copy(it.begin(), it.end(), dst + 3 * (size_t)k++);
+        nc[0] += it[2] > 48; nc[1] += it[2] > 32 && it[2] <= 48; nc[2] += it[2] > 16 && it[2] <= 32;
       }
+      return k;
+    };
+    std::vector<std::array<uint32_t, 3>> v;
+    for (int j = 0; j < ne; j++) cut(v, (uint32_t)j, p->offs[j + 1] - p->offs[j]);
+    ni_routed = emit(v, items, nc_routed);
+    v.clear();
+    if (p->has_shared) cut(v, (uint32_t)ne, n);
+    ni_shared = emit(v, items + 3 * (size_t)ni_routed, nc_shared);
   }
   uint8_t* sc = bptr_mut(&p->scratch);
   // pageable source: the copy is staged by the runtime before this call returns, and ordered on the stream
@@ -229,7 +236,8 @@ int msq_moe_prefill(void* stream, const MsqMoePrefillArgs* p) {
     if (block_path(type)) {
       b.A = A; b.K = K; b.N = N; b.nblocks = K / 256; b.row_bytes = (uint32_t)row_bytes;
       b.items = d_items + (shared ? 3 * (size_t)ni_routed : 0); b.nitems = shared ? ni_shared : ni_routed;
-      return launch_block<GU>(type, st, b, shared ? n3_shared : n3_routed, shared ? n2_shared : n2_routed);
+      const uint32_t* nc = shared ? nc_shared : nc_routed;
+      return launch_block<GU>(type, st, b, nc[0], nc[1], nc[2]);
     }
     a.A = A; a.N = N; steps(K); a.row_bytes = (uint32_t)row_bytes;
     a.tiles = d_tiles + (shared ? 2 * (size_t)nt_routed : 0); a.ntiles = shared ? nt_shared : nt_routed;
