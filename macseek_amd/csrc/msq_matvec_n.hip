@@ -9,24 +9,17 @@ namespace {
 
 template <class F>
 int launch_mvn(hipStream_t st, MvnArgs a) {
-  const uint32_t total_steps = a.cols / 32u;
-  const uint32_t chunk_steps = 16u * kMvnMaxSteps;  // 16 waves x 16 steps = 8192 columns per launch
   const int cus = device_info().cus;
-  for (uint32_t first = 0; first < total_steps; first += chunk_steps) {
-    MvnArgs c = a;
-    c.nsteps = std::min(chunk_steps, total_steps - first);
-    c.col0 = 32u * first;
-    c.col0_bytes = (uint32_t)msq_type_row_bytes_of_cols(a, c.col0);
-    if (first > 0) c.accumulate = 1u;
-    const uint32_t ks = std::min<uint32_t>(16u, c.nsteps);
-    c.steps_per_wave = (c.nsteps + ks - 1) / ks;
-    const uint32_t waves = (c.nsteps + c.steps_per_wave - 1) / c.steps_per_wave;
-    const size_t lds = (size_t)F::LDS_WORDS * 4 + (size_t)waves * 16 * 17 * 4;
-    const int wg_per_cu = std::max(1, std::min<int>(2048 / (64 * (int)waves), 2));
-    const long grid = std::min<long>(c.ntiles, (long)cus * wg_per_cu);
-    hipLaunchKernelGGL((mvn_kernel<F>), dim3((unsigned)grid), dim3(64 * waves), lds, st, c);
-    MSQ_HIP(hipGetLastError());
-  }
+  a.nsteps = a.cols / 32u;
+  a.col0 = 0; a.col0_bytes = 0;
+  const uint32_t ks = std::min<uint32_t>(16u, a.nsteps);
+  a.steps_per_wave = (a.nsteps + ks - 1) / ks;
+  const uint32_t waves = (a.nsteps + a.steps_per_wave - 1) / a.steps_per_wave;
+  const size_t lds = (size_t)F::LDS_WORDS * 4 + (size_t)waves * 16 * 17 * 4;
+  const int wg_per_cu = std::max(1, std::min<int>(2048 / (64 * (int)waves), 2));
+  const long grid = std::min<long>(a.ntiles, (long)cus * wg_per_cu);
+  hipLaunchKernelGGL((mvn_kernel<F>), dim3((unsigned)grid), dim3(64 * waves), lds, st, a);
+  MSQ_HIP(hipGetLastError());
   return MSQ_OK;
 }
 
@@ -48,7 +41,12 @@ extern "C" int msq_matvec_n(void* stream, int t, const MsqBuffer* W, int rows, i
     return fail(MSQ_ERR_ARGUMENT, "macseek quant: matvec_n: buffer missing or too small (type %s rows %d cols %d n %d)",
                 msq_type_name_of(t), rows, cols, n);
   const int rpg = rows / groups;
-  if (t == MSQ_F32 || (groups > 1 && rpg % 16)) {  // served as n decode matvecs
+  // A few tokens over a small matrix are served faster as n decode matvecs (the matrix stays in the caches after the
+  // first): measured on MI355X, a matvec launch costs about 3 us + 1 us per 1.5 MB of weights, an MFMA launch about
+  // 20 us + 1 us per MB (one 16-row tile per workgroup pass, K split over its waves).
+  const double mb = (double)rb * rows / 1e6;
+  const bool few = n * (3.0 + mb / 1.5) < 20.0 + mb;
+  if (t == MSQ_F32 || (groups > 1 && rpg % 16) || few) {  // served as n decode matvecs
     for (int i = 0; i < n; i++) {
       const MsqBuffer xi{X->dev, X->off + (size_t)i * xs * 4, xs * 4}, yi{Y->dev, Y->off + (size_t)i * rows * 4, (size_t)rows * 4};
       const int rc = msq_matvec(stream, t, W, rows, cols, &xi, &yi, accumulate, groups, nullptr);

@@ -17,7 +17,8 @@ namespace msq {
 
 typedef __bf16 bf8_t __attribute__((ext_vector_type(8)));
 
-constexpr int kMvnMaxSteps = 16;  // K steps (of 32 columns) whose activations one wave keeps in registers
+constexpr int kMvnMaxSteps = 16;  // K steps (of 32 columns) whose activations one wave of the token-tile GEMM keeps in registers
+constexpr int kMvnSubSteps = 8;   // K steps a wave of the small-N matvec fetches and multiplies at a time
 
 __device__ __forceinline__ f4_t mfma_f16(const uint32_t a[4], const uint32_t b[4], f4_t c) {
   typedef uint32_t u4_t __attribute__((ext_vector_type(4)));
@@ -180,10 +181,12 @@ struct FragQ5K {
     const uint32_t q0 = ((ql.x >> (4 * run)) & 0x0F0F0F0Fu) | (((qh.x >> is) & 0x01010101u) << 4);
     const uint32_t q1 = ((ql.y >> (4 * run)) & 0x0F0F0F0Fu) | (((qh.y >> is) & 0x01010101u) << 4);
     const uint32_t bias = 0xE400E400u;  // -1024 in both halves
-    const P s = b + 4;
+    // the 12 scale bytes, fetched unconditionally (a load inside a branch makes the waits that follow conservative)
+    const uint32_t s0 = ld32(b + 4), s1 = ld32(b + 8), s2 = ld32(b + 12);
+    auto byte = [&](uint32_t i) { const uint32_t w = i < 4 ? s0 : i < 8 ? s1 : s2; return (w >> (8 * (i & 3u))) & 0xFFu; };
     uint32_t sc, mn;
-    if (is < 4) { sc = ld8(s + is) & 63u; mn = ld8(s + is + 4) & 63u; }
-    else { sc = (ld8(s + is + 4) & 0xFu) | ((ld8(s + is - 4) >> 6) << 4); mn = (ld8(s + is + 4) >> 4) | ((ld8(s + is) >> 6) << 4); }
+    if (is < 4) { sc = byte(is) & 63u; mn = byte(is + 4) & 63u; }
+    else { sc = (byte(is + 4) & 0xFu) | ((byte(is - 4) >> 6) << 4); mn = (byte(is + 4) >> 4) | ((byte(is) >> 6) << 4); }
     const uint32_t dd = ld32(b);
     FragOut o;
     o.h[0] = pk_add_f16(bytes01_to_h2_1024(q0), bias); o.h[1] = pk_add_f16(bytes23_to_h2_1024(q0), bias);

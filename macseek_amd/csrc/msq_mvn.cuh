@@ -3,9 +3,9 @@
 // and for n >= 8 the tile matmul q_mm, src/kernels/quant_mm.metal:81-115).
 //
 // One weight read serves all n tokens through the matrix cores: a 16-row tile of W is the B operand, the (up to 16)
-// tokens are the A operand. A workgroup is KS waves that split K; each wave keeps the activations of its K steps in
-// registers as MFMA A fragments for the whole launch and walks the row tiles (persistent grid), so weights are the
-// only HBM stream. Per tile the KS partial 16 x 16 results meet in LDS and are added in a fixed order.
+// tokens are the A operand. A workgroup is KS waves that split K; a wave takes its K steps eight at a time: the weight
+// fragments of all eight are requested before the first MFMA, the activations are MFMA A fragments in registers (kept
+// for the whole launch when a wave has at most eight steps); the workgroups walk the row tiles (persistent grid). Per tile the KS partial 16 x 16 results meet in LDS and are added in a fixed order.
 #pragma once
 #include "msq_mfma.cuh"
 
@@ -31,6 +31,8 @@ inline size_t msq_type_row_bytes_of_cols(const MvnArgs& a, uint32_t col) { retur
 
 template <class F>
 __global__ __launch_bounds__(1024) void mvn_kernel(const MvnArgs a) {
+  constexpr int MS = kMvnSubSteps;
+  constexpr bool HALF_SCALES = requires(const uint8_t* r, float& s) { F::get_scales(r, 0u, s, s); };
   extern __shared__ __attribute__((aligned(16))) uint32_t smem[];
   uint32_t* tbl = smem;
   float* red = (float*)(smem + F::LDS_WORDS);  // [wave][token][17]
@@ -42,32 +44,45 @@ __global__ __launch_bounds__(1024) void mvn_kernel(const MvnArgs a) {
 
   F::fill_lds(tbl, (int)tid, (int)blockDim.x);
 
-  // activations of this wave's K steps, as A fragments (token m16, chunk q); bf16 math splits x into hi + lo
-  uint32_t xa[kMvnMaxSteps][4];
-  uint32_t xb[F::BF16_MATH ? kMvnMaxSteps : 1][4];
-  auto load_x = [&](uint32_t group) {
+  // activations of MS of this wave's K steps at a time, as A fragments (token m16, chunk q); bf16 math splits x into
+  // hi + lo. A wave with at most MS steps keeps them for the whole launch.
+  uint32_t xa[MS][4];
+  uint32_t xb[F::BF16_MATH ? MS : 1][4];
+  auto load_x = [&](uint32_t group, uint32_t c0) {
+    // all requests first, then the conversions (scheduling barrier in between): left to itself the scheduler pairs
+    // each step's loads with their conversion and waits for every step separately. No branch around the loads either
+    // (a wait after a conditional load waits for everything in flight): lanes past the last token repeat it -- their
+    // output rows are never stored -- and steps past the end repeat the last one, which the MFMA loop skips.
+    float4 raw[MS][2];
 #pragma unroll
-    for (int i = 0; i < kMvnMaxSteps; i++) {
-      const uint32_t step = s0 + i;
-      if ((uint32_t)i < S && step < a.nsteps && m16 < a.n) {
-        const float* xs = a.X + (size_t)m16 * a.x_stride + (size_t)group * a.x_group_stride + a.col0 + 32u * step;
-        float v[8];
+    for (int i = 0; i < MS; i++) {
+      const uint32_t step = min(s0 + c0 + i, a.nsteps - 1);
+      const float* xs = a.X + (size_t)min(m16, a.n - 1) * a.x_stride + (size_t)group * a.x_group_stride + a.col0 + 32u * step;
+      // the chunk's 8 columns as two 128-bit loads (col_of is 8 q + p, or for IQ4_NL 4 q + p / 2 + 16 (p % 2))
+      const bool natural = F::col_of(1, 1) == 9u;
+      raw[i][0] = *(const float4*)(xs + (natural ? 8u * q : 4u * q));
+      raw[i][1] = *(const float4*)(xs + (natural ? 8u * q + 4u : 4u * q + 16u));
+    }
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int p = 0; p < 8; p++) v[p] = xs[F::col_of(q, p)];
-#pragma unroll
-        for (int p = 0; p < 4; p++) {
-          if constexpr (F::BF16_MATH) {
-            const uint32_t h0 = bf16_rne(v[2 * p]), h1 = bf16_rne(v[2 * p + 1]);
-            const float r0 = v[2 * p] - __builtin_bit_cast(float, h0 << 16), r1 = v[2 * p + 1] - __builtin_bit_cast(float, h1 << 16);
-            xa[i][p] = h0 | (h1 << 16);
-            xb[i][p] = bf16_rne(r0) | (bf16_rne(r1) << 16);
-          } else {
-            xa[i][p] = pack_h2(v[2 * p], v[2 * p + 1]);
-          }
-        }
+    for (int i = 0; i < MS; i++) {
+      const float4 lo = raw[i][0], hi = raw[i][1];
+      float v[8];
+      if (F::col_of(1, 1) == 9u) {
+        v[0] = lo.x; v[1] = lo.y; v[2] = lo.z; v[3] = lo.w; v[4] = hi.x; v[5] = hi.y; v[6] = hi.z; v[7] = hi.w;
       } else {
+        v[0] = lo.x; v[1] = hi.x; v[2] = lo.y; v[3] = hi.y; v[4] = lo.z; v[5] = hi.z; v[6] = lo.w; v[7] = hi.w;
+      }
 #pragma unroll
-        for (int p = 0; p < 4; p++) { xa[i][p] = 0u; if constexpr (F::BF16_MATH) xb[i][p] = 0u; }
+      for (int p = 0; p < 4; p++) {
+        if constexpr (F::BF16_MATH) {
+          const uint32_t h0 = bf16_rne(v[2 * p]), h1 = bf16_rne(v[2 * p + 1]);
+          const float r0 = v[2 * p] - __builtin_bit_cast(float, h0 << 16), r1 = v[2 * p + 1] - __builtin_bit_cast(float, h1 << 16);
+          xa[i][p] = h0 | (h1 << 16);
+          xb[i][p] = bf16_rne(r0) | (bf16_rne(r1) << 16);
+        } else {
+          xa[i][p] = pack_h2(v[2 * p], v[2 * p + 1]);
+        }
       }
     }
   };
@@ -77,33 +92,49 @@ __global__ __launch_bounds__(1024) void mvn_kernel(const MvnArgs a) {
   const uint32_t ones[4] = {0x3C003C00u, 0x3C003C00u, 0x3C003C00u, 0x3C003C00u};
   for (uint32_t tile = blockIdx.x; tile < a.ntiles; tile += gridDim.x) {
     const uint32_t group = (tile * 16u) / a.rows_per_group;  // a tile never straddles two groups (host guarantees)
-    if (group != cur_group) { load_x(group); cur_group = group; }
     const uint32_t row = min(tile * 16u + m16, a.rows - 1);
-    const uint8_t* wr = a.W + (size_t)row * a.row_bytes + a.col0_bytes;
+    const gptr_t wr = as_global(a.W) + (size_t)row * a.row_bytes + a.col0_bytes;
     f4_t acc = {0.f, 0.f, 0.f, 0.f};
+    for (uint32_t c0 = 0; c0 < S; c0 += MS) {
+      // all of the sub-chunk's weight fragments are requested (and decoded as they arrive) before the first MFMA:
+      // a wave's steps are independent, and fetched one at a time each would cost a full memory latency
+      // activations first: their raw fp32 form takes twice the registers of the packed fragments, and requested
+      // after the weights they would be fetched and waited for one step at a time
+      if (S > MS || group != cur_group) {
+        load_x(group, c0);
+        cur_group = group;
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      FragOut fr[MS];
+      float sa[HALF_SCALES ? MS : 1], sb[HALF_SCALES ? MS : 1];
 #pragma unroll
-    for (int i = 0; i < kMvnMaxSteps; i++) {
-      const uint32_t step = s0 + i;
-      if ((uint32_t)i < S && step < a.nsteps) {  // wave-uniform
-        const f4_t zero = {0.f, 0.f, 0.f, 0.f};
-        const FragOut f = F::get(wr, step, q, tbl);
-        if constexpr (requires(float& s) { F::get_scales(wr, step, s, s); }) {
-          // half-step scale groups: chunks 0-1 and chunks 2-3 go through separate MFMAs
-          float sa, sb;
-          F::get_scales(wr, step, sa, sb);
-          uint32_t ha[4], hb[4];
+      for (int i = 0; i < MS; i++) {
+        const uint32_t step = min(s0 + c0 + i, a.nsteps - 1);  // past the end: the last step again, never multiplied
+        fr[i] = F::get(wr, step, q, tbl);
+        if constexpr (HALF_SCALES) F::get_scales(wr, step, sa[i], sb[i]);
+      }
 #pragma unroll
-          for (int p = 0; p < 4; p++) { ha[p] = q < 2 ? f.h[p] : 0u; hb[p] = q < 2 ? 0u : f.h[p]; }
-          const f4_t pa = mfma_f16(xa[i], ha, zero), pb = mfma_f16(xa[i], hb, zero);
-          acc += sa * pa + sb * pb;
-        } else if constexpr (F::BF16_MATH) {
-          f4_t p = mfma_bf16(xa[i], f.h, zero);
-          p = mfma_bf16(xb[i], f.h, p);
-          acc += f.scale * p;
-        } else {
-          const f4_t p = mfma_f16(xa[i], f.h, zero);
-          acc += f.scale * p;
-          if constexpr (F::HAS_ADD) acc += f.add * mfma_f16(xa[i], ones, zero);  // per-token sum of the step's x
+      for (int i = 0; i < MS; i++) {
+        const uint32_t step = s0 + c0 + i;
+        if (c0 + i < S && step < a.nsteps) {  // wave-uniform
+          const f4_t zero = {0.f, 0.f, 0.f, 0.f};
+          const FragOut& f = fr[i];
+          if constexpr (HALF_SCALES) {
+            // half-step scale groups: chunks 0-1 and chunks 2-3 go through separate MFMAs
+            uint32_t ha[4], hb[4];
+#pragma unroll
+            for (int p = 0; p < 4; p++) { ha[p] = q < 2 ? f.h[p] : 0u; hb[p] = q < 2 ? 0u : f.h[p]; }
+            const f4_t pa = mfma_f16(xa[i], ha, zero), pb = mfma_f16(xa[i], hb, zero);
+            acc += sa[i] * pa + sb[i] * pb;
+          } else if constexpr (F::BF16_MATH) {
+            f4_t p = mfma_bf16(xa[i], f.h, zero);
+            p = mfma_bf16(xb[i], f.h, p);
+            acc += f.scale * p;
+          } else {
+            const f4_t p = mfma_f16(xa[i], f.h, zero);
+            acc += f.scale * p;
+            if constexpr (F::HAS_ADD) acc += f.add * mfma_f16(xa[i], ones, zero);  // per-token sum of the step's x
+          }
         }
       }
     }
