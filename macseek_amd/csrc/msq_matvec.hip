@@ -106,6 +106,66 @@ int launch_mv(hipStream_t st, const MvShape& s, MvArgs& a) {
   return MSQ_OK;
 }
 
+// Launch shape of the small-N matvec: workgroups of at most 8 waves (the kernel keeps T activation slices per lane
+// and is built for 512 threads), one or two units per lane.
+bool mv_tok_shape(int t, int rows, int cols, int groups, int token_groups, MvShape* s) {
+  const int unit = mv_unit(t);
+  const int units = cols / unit;
+  int iters = 1;
+  while (iters < 2 && units > 64 * 8 * iters) iters *= 2;
+  const int ks = (units + 64 * iters - 1) / (64 * iters);
+  if (ks > 8) return false;
+  int rw = std::max(1, 8 / ks);
+  // rows per wave per tile: one workgroup per CU, one tile each, is what measures fastest (a wave prefetches along its
+  // run of rows; every tile ends in a workgroup-wide reduction)
+  const long wgs = std::max(1, device_info().cus / token_groups);
+  int rpw = (int)std::min<long>(32, std::max<long>(1, (rows + wgs * rw - 1) / (wgs * rw)));
+  const int rpg = rows / groups;
+  if (groups > 1) {  // every tile must stay inside one block-diagonal group
+    while (rpw > 1 && rpg % (rw * rpw)) rpw--;
+    while (rw > 1 && rpg % (rw * rpw)) rw /= 2;
+    if (rpg % (rw * rpw)) return false;
+  }
+  *s = {iters, ks, rw, rpw, unit};
+  return true;
+}
+
+template <class D, int T>
+int launch_mv_tok(hipStream_t st, const MvShape& s, MvTokArgs& ta) {
+  MvArgs& a = ta.m;
+  const int threads = 64 * s.rw * s.ks;
+  const int tile_rows = s.rw * s.rpw;
+  a.units = a.cols / D::UNIT;
+  a.ks = s.ks;
+  a.rpw = s.rpw;
+  a.ntiles = (a.rows + tile_rows - 1) / tile_rows;
+  const size_t lds = (size_t)D::LDS_WORDS * 4 + (size_t)tile_rows * s.ks * 4 * T * 4;
+  const int gy = ((int)ta.n + T - 1) / T;
+  // persistent workgroups, one per CU over all token groups
+  const int gx = (int)std::min<long>(a.ntiles, std::max(1, device_info().cus / gy));
+  const dim3 grid((unsigned)gx, (unsigned)gy);
+  if (s.iters == 1) hipLaunchKernelGGL((mv_tok_kernel<D, 1, T>), grid, dim3(threads), lds, st, ta);
+  else if constexpr (D::UNIT == 8) hipLaunchKernelGGL((mv_tok_kernel<D, 2, T>), grid, dim3(threads), lds, st, ta);
+  else return MSQ_ERR_UNSUPPORTED;  // two block-format units per lane and T activation slices do not fit the registers
+  MSQ_HIP(hipGetLastError());
+  return MSQ_OK;
+}
+
+template <int T>
+int launch_mv_tok_t(hipStream_t st, int t, const MvShape& s, MvTokArgs& ta) {
+  switch (t) {
+    case MSQ_IQ1_S: return launch_mv_tok<DecIQ1S, T>(st, s, ta);
+    case MSQ_IQ2_XXS: return launch_mv_tok<DecIQ2XXS, T>(st, s, ta);
+    case MSQ_IQ4_NL: return launch_mv_tok<DecIQ4NL, T>(st, s, ta);
+    case MSQ_Q6_K: return launch_mv_tok<DecQ6K, T>(st, s, ta);
+    case MSQ_Q5_K: return launch_mv_tok<DecQ5K, T>(st, s, ta);
+    case MSQ_F32: return launch_mv_tok<DecDense<MSQ_F32>, T>(st, s, ta);
+    case MSQ_F16: return launch_mv_tok<DecDense<MSQ_F16>, T>(st, s, ta);
+    case MSQ_BF16: return launch_mv_tok<DecDense<MSQ_BF16>, T>(st, s, ta);
+  }
+  return MSQ_ERR_UNSUPPORTED;
+}
+
 bool mv_type_ok(int t) {
   switch (t) {
     case MSQ_F32: case MSQ_F16: case MSQ_BF16: case MSQ_Q8_0: case MSQ_Q5_K: case MSQ_Q6_K: case MSQ_IQ1_S:
@@ -117,6 +177,28 @@ bool mv_type_ok(int t) {
 int mv_col_multiple(int t) { return msq_type_block_elems(t) == 1 ? 256 : msq_type_block_elems(t); }
 
 }  // namespace
+}  // namespace msq
+
+namespace msq {
+
+// Small-N matvec through the dot-product kernels. Returns MSQ_ERR_UNSUPPORTED without an error message when the shape
+// does not fit them (the caller then takes another path). Arguments are already validated.
+int matvec_tok(hipStream_t st, int t, const uint8_t* W, int rows, int cols, const float* X, float* Y, int n, int accumulate,
+               int groups) {
+  // Q8_0 keeps fp32 activations (32 registers per token): four tokens per pass, the other formats eight
+  const int T = (t == MSQ_Q8_0 || n <= 4) ? 4 : 8;
+  MvShape s;
+  if (!mv_tok_shape(t, rows, cols, groups, (n + T - 1) / T, &s)) return MSQ_ERR_UNSUPPORTED;
+  MvTokArgs ta{};
+  MvArgs& a = ta.m;
+  a.W = W; a.x = X; a.y = Y;
+  a.rows = (uint32_t)rows; a.cols = (uint32_t)cols; a.row_bytes = (uint32_t)msq_type_row_bytes(t, cols);
+  a.rows_per_group = (uint32_t)(rows / groups); a.x_group_stride = (uint32_t)cols; a.accumulate = accumulate ? 1u : 0u;
+  ta.n = (uint32_t)n; ta.x_stride = (uint32_t)((size_t)cols * groups); ta.y_stride = (uint32_t)rows;
+  if (t == MSQ_Q8_0) return launch_mv_tok<DecQ8_0, 4>(st, s, ta);
+  return T == 4 ? launch_mv_tok_t<4>(st, t, s, ta) : launch_mv_tok_t<8>(st, t, s, ta);
+}
+
 }  // namespace msq
 
 using namespace msq;

@@ -190,4 +190,99 @@ __global__ __launch_bounds__(1024) void mv_ring_kernel(const MvArgs a) {
   }
 }
 
+// Small-N form of mv_kernel: T tokens per pass over the weights (reference operator: ms::q::encode_matvec_n,
+// src/kernels/quant.mm:129-156; reference kernel q_mvn, src/kernels/quant_mv.metal:148-202). A lane keeps the
+// activation slices of T tokens; a weight unit is fetched once and its decode is shared by the T dot products (the T
+// calls of dec_dot are inlined over the same raw bytes, so only the dot2 chains differ). blockIdx.y picks the token
+// group: groups beyond the first find the weights in the caches. Lanes are laid out over a row exactly as in
+// mv_kernel, so every load is a contiguous run over the wave.
+struct MvTokArgs {
+  MvArgs m;
+  uint32_t n;                    // tokens
+  uint32_t x_stride, y_stride;   // elements between the activation / output rows of consecutive tokens
+};
+
+template <class D, int ITERS, int T>
+__global__ __launch_bounds__(512) void mv_tok_kernel(const MvTokArgs ta) {
+  const MvArgs& a = ta.m;
+  extern __shared__ __attribute__((aligned(16))) uint32_t smem[];
+  uint32_t* tbl = smem;
+  float* part = (float*)(smem + D::LDS_WORDS);  // [row of tile][ks][16-lane row of the wave][T]
+
+  const uint32_t tid = threadIdx.x, lane = tid & 63u, nwaves = blockDim.x >> 6;
+  const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
+  const uint32_t KS = a.ks, ks = wave % KS, rw = wave / KS, RW = nwaves / KS;
+  const uint32_t tile_rows = RW * a.rpw;
+  const uint32_t t0 = blockIdx.y * T;
+
+  D::fill_lds(tbl, (int)tid, (int)blockDim.x);
+
+  uint32_t unit[ITERS];
+  bool valid[ITERS];
+#pragma unroll
+  for (int i = 0; i < ITERS; i++) {
+    const uint32_t u = (ks * ITERS + i) * 64u + lane;
+    valid[i] = u < a.units;
+    unit[i] = valid[i] ? u : a.units - 1;  // idle lanes shadow the last unit; their result is dropped
+  }
+  typename D::X xr[T][ITERS];
+  uint32_t cur_group = 0xFFFFFFFFu;
+  if (D::LDS_WORDS) __syncthreads();
+
+  for (uint32_t tile = blockIdx.x; tile < a.ntiles; tile += gridDim.x) {
+    const uint32_t tile_row0 = tile * tile_rows;
+    const uint32_t group = tile_row0 / a.rows_per_group;  // a tile never straddles two groups (host guarantees)
+    if (group != cur_group) {
+#pragma unroll
+      for (int t = 0; t < T; t++) {  // tokens past the last repeat it; their results are never stored
+        const float* xg = a.x + (size_t)min(t0 + t, ta.n - 1) * ta.x_stride + (size_t)group * a.x_group_stride;
+#pragma unroll
+        for (int i = 0; i < ITERS; i++) xr[t][i] = D::load_x(xg, unit[i]);
+      }
+      cur_group = group;
+    }
+    const uint32_t row0 = tile_row0 + rw * a.rpw;
+    typename D::Raw raw[ITERS];
+    {
+      const gptr_t wr = as_global(a.W) + (size_t)min(row0, a.rows - 1) * a.row_bytes;
+#pragma unroll
+      for (int i = 0; i < ITERS; i++) raw[i] = D::load(wr, unit[i]);
+    }
+    for (uint32_t j = 0; j < a.rpw; j++) {
+      typename D::Raw nxt[ITERS];  // the next row's bytes are requested before this row's arithmetic
+      {
+        const gptr_t wr = as_global(a.W) + (size_t)min(row0 + j + 1, a.rows - 1) * a.row_bytes;
+#pragma unroll
+        for (int i = 0; i < ITERS; i++) nxt[i] = D::load(wr, unit[i]);
+      }
+      float acc[T];
+#pragma unroll
+      for (int t = 0; t < T; t++) {
+        acc[t] = 0.f;
+#pragma unroll
+        for (int i = 0; i < ITERS; i++) {
+          const float v = dec_dot<D>(raw[i], xr[t][i], tbl, unit[i]);
+          acc[t] += valid[i] ? v : 0.f;
+        }
+      }
+      // transposed fold: afterwards acc[0] of lane l is token group8_sel<T>(l) summed over l's 16-lane row
+      row16_fold<T>(acc, lane);
+      if (!(lane & 8u)) part[(((rw * a.rpw + j) * KS + ks) * 4 + (lane >> 4)) * T + group8_sel<T>(lane)] = acc[0];
+#pragma unroll
+      for (int i = 0; i < ITERS; i++) raw[i] = nxt[i];
+    }
+    __syncthreads();
+    for (uint32_t idx = tid; idx < tile_rows * T; idx += blockDim.x) {
+      const uint32_t r = idx % tile_rows, t = idx / tile_rows, row = tile_row0 + r;  // consecutive lanes: consecutive rows
+      if (row < a.rows && t0 + t < ta.n) {
+        float s = 0.f;
+        for (uint32_t k = 0; k < 4 * KS; k++) s += part[(r * 4 * KS + k) * T + t];
+        float* y = a.y + (size_t)(t0 + t) * ta.y_stride + row;
+        *y = a.accumulate ? *y + s : s;
+      }
+    }
+    __syncthreads();
+  }
+}
+
 }  // namespace msq

@@ -20,7 +20,9 @@ CASES = [  # (type, rows, cols, groups, n, accumulate): tests/test_quant_matvec_
     (O.F16, 300, 1280, 1, 16, False), (O.Q6_K, 32768, 1280, 1, 9, False),
     (O.IQ4_NL, 1024, 4096, 1, 7, True), (O.Q5_K, 37, 256, 1, 2, False), (O.Q8_0, 16, 32, 1, 16, False),
     (O.Q6_K, 24, 512, 3, 3, False),           # group size 8 rows: served as n decode matvecs
-    (O.Q8_0, 64, 16384, 1, 4, False),         # wider than one launch covers: K chunks accumulate
+    (O.Q8_0, 64, 16384, 1, 4, False),         # the widest rows the dot-product kernel takes
+    (O.Q6_K, 32, 18432, 1, 8, True), (O.F16, 48, 9216, 1, 9, False),  # wider: MFMA kernel, several K sub-chunks per wave
+    (O.IQ2_XXS, 64, 20480, 1, 2, False),      # wider, few tokens: n decode matvecs
 ]
 BASELINE5 = [(O.Q6_K, 1536, 7168), (O.Q5_K, 512, 7168), (O.IQ4_NL, 7168, 4096), (O.BF16, 384, 7168)]
 CASES += [(t, r, c, 1, n, False) for (t, r, c) in BASELINE5 for n in (1, 2, 4, 8, 16)]
@@ -50,10 +52,15 @@ def test_matvec_n_vs_oracle(dev, t, rows, cols, groups, n, acc):
     e.wait()
     got = Yd.cpu().numpy().astype(np.float64).reshape(n, rows)
     assert np.all(np.isfinite(got))
-    # few tokens over a small matrix are served as n decode matvecs (the library's launch-cost model)
+    # the library's dispatch: rows of up to 16384 columns (dense types: 8192) go through the dot-product kernel, which
+    # stages activations like the decode matvec, unless more than eight tokens meet a large matrix of a format with
+    # cheap MFMA fragments; wider rows through the MFMA kernel, or as n decode matvecs when that is cheaper
+    dots = cols <= (8192 if t in (O.F32, O.F16, O.BF16) else 16384)
     mb = q.row_bytes(q.QType(t), cols) * rows / 1e6
-    few = n * (3.0 + mb / 1.5) < 20.0 + mb
-    uses_mfma = n > 1 and t != O.F32 and not (groups > 1 and (rows // groups) % 16) and not few
+    mfma_ok = n > 1 and t != O.F32 and not (groups > 1 and (rows // groups) % 16)
+    mfma_first = mfma_ok and n > 8 and mb > 12.0 and t in (O.IQ4_NL, O.Q8_0, O.F16, O.BF16)
+    few = not mfma_first and n * (3.0 + mb / 1.5) < 20.0 + mb
+    uses_mfma = mfma_first or (mfma_ok and not dots and not few)
     Xh = half_round(X, t) if uses_mfma else X
     if not uses_mfma and t not in (O.F32, O.F16, O.BF16, O.Q8_0):
         Xh = X.astype(np.float16).astype(np.float32)  # the decode (n = 1) path stages fp16 pairs for the block formats
