@@ -108,18 +108,25 @@ int launch_mv(hipStream_t st, const MvShape& s, MvArgs& a) {
 
 // Launch shape of the small-N matvec: workgroups of at most 8 waves (the kernel keeps T activation slices per lane
 // and is built for 512 threads), one or two units per lane.
-bool mv_tok_shape(int t, int rows, int cols, int groups, int token_groups, MvShape* s) {
+bool mv_tok_shape(int t, int rows, int cols, int groups, int token_groups, const MsqMvCfg* cfg, MvShape* s) {
   const int unit = mv_unit(t);
   const int units = cols / unit;
   int iters = 1;
   while (iters < 2 && units > 64 * 8 * iters) iters *= 2;
-  const int ks = (units + 64 * iters - 1) / (64 * iters);
-  if (ks > 8) return false;
+  int ks = (units + 64 * iters - 1) / (64 * iters);
+  if (cfg && cfg->ks > 0) {
+    ks = cfg->ks;
+    iters = units > 64 * ks ? 2 : 1;
+  }
+  if (ks > 8 || units > 64 * ks * iters) return false;
   int rw = std::max(1, 8 / ks);
+  if (cfg && cfg->rsg > 0) rw = cfg->rsg;
+  if (rw * ks > 8) return false;
   // rows per wave per tile: one workgroup per CU, one tile each, is what measures fastest (a wave prefetches along its
   // run of rows; every tile ends in a workgroup-wide reduction)
   const long wgs = std::max(1, device_info().cus / token_groups);
   int rpw = (int)std::min<long>(32, std::max<long>(1, (rows + wgs * rw - 1) / (wgs * rw)));
+  if (cfg && cfg->nr > 0) rpw = std::min(cfg->nr, 64);
   const int rpg = rows / groups;
   if (groups > 1) {  // every tile must stay inside one block-diagonal group
     while (rpw > 1 && rpg % (rw * rpw)) rpw--;
@@ -128,6 +135,13 @@ bool mv_tok_shape(int t, int rows, int cols, int groups, int token_groups, MvSha
   }
   *s = {iters, ks, rw, rpw, unit};
   return true;
+}
+
+// n = 1: the prefetching kernel pays from two full rows per wave and CU on (below that mv_kernel does the same with
+// less ceremony); an imposed shape with nr >= 2 names it outright
+bool tok_serves_single(int rows, const MvShape& s, const MsqMvCfg* cfg) {
+  if (cfg && cfg->nr > 0) return s.rpw >= 2;
+  return s.rpw >= 2 && (long)rows >= 2L * device_info().cus * s.rw;
 }
 
 template <class D, int T>
@@ -184,17 +198,19 @@ namespace msq {
 // Small-N matvec through the dot-product kernels. Returns MSQ_ERR_UNSUPPORTED without an error message when the shape
 // does not fit them (the caller then takes another path). Arguments are already validated.
 int matvec_tok(hipStream_t st, int t, const uint8_t* W, int rows, int cols, const float* X, float* Y, int n, int accumulate,
-               int groups) {
+               int groups, const MsqMvCfg* cfg) {
   // Q8_0 keeps fp32 activations (32 registers per token): four tokens per pass, the other formats eight
-  const int T = (t == MSQ_Q8_0 || n <= 4) ? 4 : 8;
+  const int T = n == 1 ? 1 : (t == MSQ_Q8_0 || n <= 4) ? 4 : 8;
   MvShape s;
-  if (!mv_tok_shape(t, rows, cols, groups, (n + T - 1) / T, &s)) return MSQ_ERR_UNSUPPORTED;
+  if (!mv_tok_shape(t, rows, cols, groups, (n + T - 1) / T, cfg, &s)) return MSQ_ERR_UNSUPPORTED;
+  if (n == 1 && !tok_serves_single(rows, s, cfg)) return MSQ_ERR_UNSUPPORTED;
   MvTokArgs ta{};
   MvArgs& a = ta.m;
   a.W = W; a.x = X; a.y = Y;
   a.rows = (uint32_t)rows; a.cols = (uint32_t)cols; a.row_bytes = (uint32_t)msq_type_row_bytes(t, cols);
   a.rows_per_group = (uint32_t)(rows / groups); a.x_group_stride = (uint32_t)cols; a.accumulate = accumulate ? 1u : 0u;
   ta.n = (uint32_t)n; ta.x_stride = (uint32_t)((size_t)cols * groups); ta.y_stride = (uint32_t)rows;
+  if (n == 1) return t == MSQ_Q8_0 ? launch_mv_tok<DecQ8_0, 1>(st, s, ta) : launch_mv_tok_t<1>(st, t, s, ta);
   if (t == MSQ_Q8_0) return launch_mv_tok<DecQ8_0, 4>(st, s, ta);
   return T == 4 ? launch_mv_tok_t<4>(st, t, s, ta) : launch_mv_tok_t<8>(st, t, s, ta);
 }
@@ -224,8 +240,9 @@ int msq_matvec_supported(int t) { return mv_type_ok(t) ? 1 : 0; }
 int msq_matvec_cfg(int t, int rows, int cols, MsqMvCfg* out) {
   MvShape s;
   if (!out) return fail(MSQ_ERR_ARGUMENT, "macseek quant: matvec_cfg: null output");
-  if (!mv_type_ok(t) || rows < 1 || cols < 1 || cols % mv_col_multiple(t) || !mv_shape(t, rows, cols, 1, nullptr, &s))
-    return unsupported("matvec_cfg", t, rows, cols);
+  if (!mv_type_ok(t) || rows < 1 || cols < 1 || cols % mv_col_multiple(t)) return unsupported("matvec_cfg", t, rows, cols);
+  const bool tok = mv_tok_shape(t, rows, cols, 1, 1, nullptr, &s) && tok_serves_single(rows, s, nullptr);  // as msq_matvec decides
+  if (!tok && !mv_shape(t, rows, cols, 1, nullptr, &s)) return unsupported("matvec_cfg", t, rows, cols);
   out->nr = s.rpw; out->rsg = s.rw; out->ks = s.ks;
   return MSQ_OK;
 }
@@ -238,13 +255,19 @@ int msq_matvec(void* stream, int t, const MsqBuffer* W, int rows, int cols, cons
   if (!buf_ok(W, rb * (size_t)rows) || !buf_ok(x, (size_t)cols * groups * 4) || !buf_ok(y, (size_t)rows * 4))
     return fail(MSQ_ERR_ARGUMENT, "macseek quant: matvec: buffer missing or too small (type %s rows %d cols %d)",
                 msq_type_name_of(t), rows, cols);
+  hipStream_t st = (hipStream_t)stream;
+  {  // shapes with several rows per wave (chosen for matrices of more than a row per wave and CU, or imposed by cfg) go
+     // through the prefetching kernel; a shape names its kernel, so row chunks launched with the shape of the whole
+     // matrix repeat its bits
+    const int rc = matvec_tok(st, t, bptr(W), rows, cols, (const float*)bptr(x), (float*)bptr_mut(y), 1, accumulate, groups, cfg);
+    if (rc != MSQ_ERR_UNSUPPORTED) return rc;
+  }
   MvShape s;
   if (!mv_shape(t, rows, cols, groups, cfg, &s)) return unsupported("matvec launch shape", t, rows, cols);
   MvArgs a{};
   a.W = bptr(W); a.x = (const float*)bptr(x); a.y = (float*)bptr_mut(y);
   a.rows = (uint32_t)rows; a.cols = (uint32_t)cols; a.row_bytes = (uint32_t)rb;
   a.rows_per_group = (uint32_t)(rows / groups); a.x_group_stride = (uint32_t)cols; a.accumulate = accumulate ? 1u : 0u;
-  hipStream_t st = (hipStream_t)stream;
   switch (t) {
     case MSQ_IQ1_S: return launch_mv<DecIQ1S>(st, s, a);
     case MSQ_IQ2_XXS: return launch_mv<DecIQ2XXS>(st, s, a);

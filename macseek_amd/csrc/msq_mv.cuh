@@ -242,16 +242,17 @@ __global__ __launch_bounds__(512) void mv_tok_kernel(const MvTokArgs ta) {
       cur_group = group;
     }
     const uint32_t row0 = tile_row0 + rw * a.rpw;
+    const uint32_t last = min(min(row0 + a.rpw, a.rows) - 1u, a.rows - 1u);  // last row of this wave's run
     typename D::Raw raw[ITERS];
     {
-      const gptr_t wr = as_global(a.W) + (size_t)min(row0, a.rows - 1) * a.row_bytes;
+      const gptr_t wr = as_global(a.W) + (size_t)min(row0, last) * a.row_bytes;
 #pragma unroll
       for (int i = 0; i < ITERS; i++) raw[i] = D::load(wr, unit[i]);
     }
     for (uint32_t j = 0; j < a.rpw; j++) {
-      typename D::Raw nxt[ITERS];  // the next row's bytes are requested before this row's arithmetic
-      {
-        const gptr_t wr = as_global(a.W) + (size_t)min(row0 + j + 1, a.rows - 1) * a.row_bytes;
+      typename D::Raw nxt[ITERS];  // the next row's bytes are requested before this row's arithmetic (after the
+      {                            // run's last row: that row again, which the caches hold)
+        const gptr_t wr = as_global(a.W) + (size_t)min(row0 + j + 1, last) * a.row_bytes;
 #pragma unroll
         for (int i = 0; i < ITERS; i++) nxt[i] = D::load(wr, unit[i]);
       }
