@@ -78,10 +78,13 @@ int msq_matvec(void* stream, int qtype, const MsqBuffer* W, int rows, int cols, 
 
 /* reference: ms::q::encode_matvec_n (quant.hpp:32-35, quant.mm:129-156).
  * Y[n x rows] (+)= X[n x cols] . W^T for n in 1..16 (one weight read serves all n tokens). X row stride is
- * cols * groups, Y row stride is rows. n == 1 is exactly msq_matvec. For n >= 2 the block formats, F16 and BF16 run
- * on the matrix cores with activations rounded to fp16 (BF16 weights: split into two bf16 terms) and exact weights;
- * the reference rounds activations to fp16 the same way and, from n >= 8, weights too (quant.mm:133-137). F32 weights,
- * and block-diagonal calls whose group size is not a multiple of 16 rows, are served as n decode matvecs. */
+ * cols * groups, Y row stride is rows. n == 1 is exactly msq_matvec. For n >= 2, rows of up to 16384 columns (dense
+ * types: 8192) run in a dot-product kernel that stages activations like msq_matvec does (fp16 pairs for the K / IQ
+ * formats, fp32 for Q8_0 and the dense types) and decodes each weight once for up to eight tokens. Wider rows, and
+ * more than eight tokens over a large IQ4_NL / Q8_0 / F16 / BF16 matrix, run on the matrix cores with activations
+ * rounded to fp16 (BF16 weights: split into two bf16 terms) and exact weights; the reference rounds activations to
+ * fp16 the same way and, from n >= 8, weights too (quant.mm:133-137). Wide F32 matrices, and wide block-diagonal
+ * calls whose group size is not a multiple of 16 rows, are served as n decode matvecs. */
 int msq_matvec_n(void* stream, int qtype, const MsqBuffer* W, int rows, int cols, const MsqBuffer* X,
                  const MsqBuffer* Y, int n, int accumulate, int groups);
 
