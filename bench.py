@@ -442,13 +442,70 @@ def bench_copy_calibration(torch, args):
             "cpu_baseline": None, "pct_of_hbm_peak": 100 * gbps / HBM_PEAK_GBPS}
 
 
+def bench_router(torch, args):
+    """The MoE router ahead of the two MoE paths: the fused decode router (BF16 384 x 7168 logits matvec + top-6 in one
+    launch, BASELINE configs[4]'s router shape) and, for a 2048-token prefill, top-6 from logits + the expert-sorted
+    routing lists. value = the fused router's algorithmic bytes (W + x + bias + ids + weights) per second."""
+    import oracle as O
+    from macseek_amd import arch, quant as q
+    dev = torch.device("cuda:0")
+    n_exp, dim, n = 384, 7168, 2048
+    copies = 64  # 64 x 5.5 MB of router weights: successive launches do not find theirs in the caches
+    W = (torch.randn(copies, n_exp, dim, device=dev) * 0.02).to(torch.bfloat16)
+    bias = torch.randn(n_exp, device=dev) * 0.1
+    x = torch.randn(dim, device=dev)
+    s = arch.Scratch.create(n_exp)
+    ids1 = torch.zeros(6, dtype=torch.int32, device=dev)
+    w1 = torch.zeros(6, dtype=torch.float32, device=dev)
+    e = q.Enc()
+    Wb = [q.Buffer.of(W).sub(i * n_exp * dim * 2, n_exp * dim * 2) for i in range(copies)]
+
+    def fused(i):
+        arch.encode_router_fused(q.Enc(torch.cuda.current_stream()), q.Buffer.of(x), Wb[i % copies], q.Buffer.of(bias), q.Buffer.of(ids1),
+                                 q.Buffer.of(w1), s, dim, q.QType.BF16)
+    fused_ms = graph_ms_per_launch(torch, fused, 256)
+    fused_bytes = n_exp * dim * 2 + dim * 4 + n_exp * 4 + 48
+    logits_h = O.randn(n * n_exp, 1, 3.0).reshape(n, n_exp)
+    logits = torch.from_numpy(logits_h).to(dev)
+    ids = torch.zeros((n, 6), dtype=torch.int32, device=dev)
+    w = torch.zeros((n, 6), dtype=torch.float32, device=dev)
+    L = arch.RouteLists.create(n, n_exp)
+
+    def topk(i):
+        arch.encode_router_topk(q.Enc(torch.cuda.current_stream()), q.Buffer.of(logits), q.Buffer.of(bias), q.Buffer.of(ids), q.Buffer.of(w), n)
+
+    def lists(i):
+        arch.encode_route_lists(q.Enc(torch.cuda.current_stream()), q.Buffer.of(ids), q.Buffer.of(w), n, L)
+    topk(0)
+    torch.cuda.synchronize()
+    topk_ms = graph_ms_per_launch(torch, topk, 100)
+    lists_ms = graph_ms_per_launch(torch, lists, 100)
+    cpu = None
+    if not args.gpu_only:
+        bias_h = bias.cpu().numpy()
+        t0 = time.perf_counter()
+        rid, rw = O.router(logits_h, bias_h)
+        O.route_lists(rid, rw)
+        el = time.perf_counter() - t0
+        cpu = {"value": n / el, "unit": "tokens/s", "cores": 1, "kind": "port",
+               "sample": "oracle.c router + route_lists over the same 2048 x 384 logits, %.3f s; the GPU pair takes %.1f us" % (el, (topk_ms + lists_ms) * 1e3)}
+    gbps = fused_bytes / (fused_ms * 1e-3) / 1e9
+    return {"value": gbps, "ms_per_step": fused_ms, "dtype": "bf16 weights x f32 activations, f32 accumulate; f64 scores",
+            "config": {"workload": "MoE router: fused decode router BF16 384x7168 (one launch per token); prefill: top-6 of 2048x384 logits + routing lists",
+                       "fused_bytes_per_launch": fused_bytes, "fused_us": fused_ms * 1e3, "topk_2048_tokens_us": topk_ms * 1e3,
+                       "route_lists_2048_tokens_us": lists_ms * 1e3},
+            "roofline": {"bound": "hbm", "achieved": gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": gbps / HBM_PEAK_GBPS, "traffic": None,
+                         "kernel": "router_fused_kernel<BF16>", "bytes_per_launch": fused_bytes, "avg_launch_us": fused_ms * 1e3},
+            "cpu_baseline": cpu, "pct_of_hbm_peak": 100 * gbps / HBM_PEAK_GBPS}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=500)
     ap.add_argument("--warmup", type=int, default=100)
     ap.add_argument("--workload", default="moe_decode",
-                    choices=["moe_decode", "moe_prefill", "matvec_iq1s", "matvec_iq2xxs", "q8_0", "stream", "copy_calibration"])
+                    choices=["moe_decode", "moe_prefill", "matvec_iq1s", "matvec_iq2xxs", "q8_0", "router", "stream", "copy_calibration"])
     ap.add_argument("--gpu-only", action="store_true",
                     help="profiling runs: skip the CPU baseline leg and the prefill appendix of the default workload")
     args = ap.parse_args()
@@ -479,6 +536,8 @@ def main():
         r = bench_stream(torch, args)
     elif args.workload == "copy_calibration":
         r = bench_copy_calibration(torch, args)
+    elif args.workload == "router":
+        r = bench_router(torch, args)
     elif args.workload == "matvec_iq1s":
         r = bench_matvec(torch, args, q.QType.IQ1_S, 4096, 7168, 0.01, "BASELINE configs[1]: single-expert decode matvec IQ1_S 4096x7168, batch 1")
     elif args.workload == "matvec_iq2xxs":

@@ -200,6 +200,45 @@ size_t msq_moe_prefill_scratch_bytes(int total_entries, int n_tokens, int n_exp,
  * does nothing (quant.mm:435). */
 int msq_moe_prefill(void* stream, const MsqMoePrefillArgs* a);
 
+/* ---- router and routing lists: what produces the ids / weights of msq_moe_decode and the expert-sorted
+ * tok / wt / slot_of / offs of msq_moe_prefill (reference module: src/kernels/arch.hpp:79-97) ---- */
+
+/* reference: ms::arch::encode_router_topk (arch.hpp:84-85; kernel arch_router_topk, src/kernels/arch_router.metal:26-83;
+ * CPU twin ref_arch::router, tests/ref/arch_ref.cpp:97-113). logits F32 [n_tokens][n_exp], bias F32 [n_exp] ->
+ * ids int32 [n_tokens][6], w F32 [n_tokens][6], descending by key = sqrt(softplus(logit)) + bias, ties to the lower
+ * expert id; w = score / (sum of the six scores + 1e-20) * route_scale (the reference fixes n_exp = 384 and
+ * route_scale = 1.5; here n_exp is a multiple of 64 up to 512). n_tokens == 0 does nothing. */
+int msq_router_topk(void* stream, const MsqBuffer* logits, const MsqBuffer* bias, const MsqBuffer* ids, const MsqBuffer* w,
+                    int n_tokens, int n_exp, float route_scale);
+
+/* reference: ms::arch::encode_router_fused (arch.hpp:79-83; kernel arch_router_fused, arch_router.metal:86-121):
+ * logits = W[n_exp][dim] . x[dim] and the selection in one launch; W is F32 (the reference's ffn_gate_inp) or BF16.
+ * scratch (>= msq_router_scratch_bytes(n_exp), the reference's Scratch::router_logits + counter) receives the logits in
+ * its first n_exp floats; the caller zeroes it once before the first call and the call leaves its counter re-armed.
+ * Calls sharing a scratch must not overlap. */
+size_t msq_router_scratch_bytes(int n_exp);
+int msq_router_fused(void* stream, int wtype, const MsqBuffer* x, const MsqBuffer* W, const MsqBuffer* bias,
+                     const MsqBuffer* scratch, const MsqBuffer* ids, const MsqBuffer* w, int dim, int n_exp,
+                     float route_scale);
+
+/* reference: ms::arch::RouteLists (arch.hpp:87-96): device buffers for up to max_tokens tokens. */
+typedef struct {
+  MsqBuffer counts;  /* u32 [n_exp] */
+  MsqBuffer offsets; /* u32 [n_exp + 1] exclusive scan, offsets[n_exp] = number of entries with a valid id */
+  MsqBuffer entry;   /* u32 [6 n] entry index t * 6 + k */
+  MsqBuffer tok;     /* u32 [6 n] token t */
+  MsqBuffer w;       /* f32 [6 n] routing weight */
+  MsqBuffer slot_of; /* u32 [6 n] position of entry t * 6 + k in the sorted lists */
+  int max_tokens;
+} MsqRouteLists;
+
+/* reference: ms::arch::encode_route_lists (arch.hpp:97; kernels arch_route_count / arch_route_scatter,
+ * arch_router.metal:124-183; CPU twin ref_arch::route_lists, tests/ref/arch_ref.cpp:114-130). Entries (t, k) = t * 6 + k
+ * sorted by expert, then entry index; no atomics, so the lists are identical on every run. tok / w / slot_of / offsets
+ * are the tok / wt / slot_of / offs inputs of msq_moe_prefill. Entries whose id is outside 0..n_exp-1 are left out
+ * (their slot_of is not written). */
+int msq_route_lists(void* stream, const MsqBuffer* ids, const MsqBuffer* w, int n_tokens, int n_exp, const MsqRouteLists* L);
+
 #ifdef __cplusplus
 }
 #endif

@@ -38,6 +38,11 @@ class MsqMoePrefillArgs(C.Structure):
                 ("x_is_bf16", C.c_int)]
 
 
+class MsqRouteLists(C.Structure):
+    _fields_ = [("counts", MsqBuffer), ("offsets", MsqBuffer), ("entry", MsqBuffer), ("tok", MsqBuffer),
+                ("w", MsqBuffer), ("slot_of", MsqBuffer), ("max_tokens", C.c_int)]
+
+
 _lib = None
 
 # name -> (restype, argtypes); every symbol include/msq.h declares
@@ -62,6 +67,10 @@ SIGNATURES = {
     "msq_moe_decode_table_part": (C.c_int, [C.c_void_p, C.POINTER(MsqMoeDecodeArgs), _BP, C.c_int]),
     "msq_moe_prefill_scratch_bytes": (C.c_size_t, [C.c_int, C.c_int, C.c_int, C.c_int, C.c_int]),
     "msq_moe_prefill": (C.c_int, [C.c_void_p, C.POINTER(MsqMoePrefillArgs)]),
+    "msq_router_topk": (C.c_int, [C.c_void_p, _BP, _BP, _BP, _BP, C.c_int, C.c_int, C.c_float]),
+    "msq_router_scratch_bytes": (C.c_size_t, [C.c_int]),
+    "msq_router_fused": (C.c_int, [C.c_void_p, C.c_int, _BP, _BP, _BP, _BP, _BP, _BP, C.c_int, C.c_int, C.c_float]),
+    "msq_route_lists": (C.c_int, [C.c_void_p, _BP, _BP, C.c_int, C.c_int, C.POINTER(MsqRouteLists)]),
 }
 
 

@@ -419,3 +419,47 @@ int orc_random_blocks(int t, int64_t n, uint64_t seed, float scale, uint8_t* out
   }
   return 0;
 }
+
+/* ---------------------------------------------------------------------------------------------- router, route lists */
+void orc_router(const float* logits, const float* bias, int n_exp, int top_k, float route_scale, int* ids, float* w) {
+  double* sc = (double*)malloc(sizeof(double) * (size_t)n_exp);
+  double* key = (double*)malloc(sizeof(double) * (size_t)n_exp);
+  for (int e = 0; e < n_exp; e++) {
+    const double x = logits[e];
+    const double sp = x > 20 ? x : log1p(exp(x));
+    sc[e] = sqrt(sp);
+    key[e] = (double)(float)((float)sc[e] + bias[e]);
+  }
+  double sum = 0;
+  for (int k = 0; k < top_k; k++) { /* the first top_k of a stable descending sort: repeated first-maximum */
+    int best = -1;
+    for (int e = 0; e < n_exp; e++) {
+      int taken = 0;
+      for (int j = 0; j < k; j++) taken |= ids[j] == e;
+      if (!taken && (best < 0 || key[e] > key[best])) best = e;
+    }
+    ids[k] = best;
+    sum += sc[best];
+  }
+  for (int k = 0; k < top_k; k++) w[k] = (float)(sc[ids[k]] / (sum + 1e-20) * route_scale);
+  free(sc);
+  free(key);
+}
+
+void orc_route_lists(const int* ids, const float* w, int n_entries, int n_exp, int top_k, uint32_t* counts,
+                     uint32_t* offsets, uint32_t* entry, uint32_t* tok, float* lw, uint32_t* slot_of) {
+  memset(counts, 0, sizeof(uint32_t) * (size_t)n_exp);
+  for (int i = 0; i < n_entries; i++) counts[ids[i]]++;
+  offsets[0] = 0;
+  for (int e = 0; e < n_exp; e++) offsets[e + 1] = offsets[e] + counts[e];
+  uint32_t* fill = (uint32_t*)malloc(sizeof(uint32_t) * (size_t)n_exp);
+  memcpy(fill, offsets, sizeof(uint32_t) * (size_t)n_exp);
+  for (int i = 0; i < n_entries; i++) {
+    const uint32_t p = fill[ids[i]]++;
+    entry[p] = (uint32_t)i;
+    tok[p] = (uint32_t)(i / top_k);
+    lw[p] = w[i];
+    slot_of[i] = p;
+  }
+  free(fill);
+}

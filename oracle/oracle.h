@@ -11,10 +11,12 @@
  *   MoE decode reference  tests/test_quant_moe.mm:64-93
  *   MoE prefill reference tests/test_quant_moe_prefill.mm:25-47,186-212; reduce order
  *                         src/kernels/quant_moe_prefill.metal:330-344
+ *   router, route lists   tests/ref/arch_ref.cpp:97-130 (kernels: src/kernels/arch_router.metal:26-160)
  *
  * Pinned by: bit-equality with the reference's own dequant.cpp compiled from /root/reference (oracle/_ref, and the
  * golden fixtures written from it under tests/golden/), closed-form known answers per format, codebook invariants,
- * and numpy float64 dots on tiny cases (tests/test_oracle.py).
+ * and numpy float64 dots on tiny cases (tests/test_oracle.py). Router and route lists: equality with the reference's
+ * arch_ref.cpp compiled the same way, softplus / tie / normalisation known answers, and a stable numpy argsort.
  */
 #ifndef MSQ_ORACLE_H
 #define MSQ_ORACLE_H
@@ -79,6 +81,18 @@ int orc_moe_prefill(int t_gu, int t_down, int t_shared, int n_tokens, int n_exp,
  * fp16 scale(s) overwritten with sc = scale*(0.5+0.5|N(0,1)|) (Q8_0 sc/16, Q5_K d=sc/8 dmin=sc/4, Q6_K sc/32). */
 void orc_randn(float* out, int64_t n, uint64_t seed, float scale);
 int orc_random_blocks(int t, int64_t n_elems, uint64_t seed, float scale, uint8_t* out);
+
+/* MoE router for one token (tests/ref/arch_ref.cpp:97-113): score = sqrt(softplus(logit)) in double (softplus(x) = x
+ * for x > 20, else log1p(exp(x))); key = (float)score + bias, rounded to float; the top_k experts by key, descending,
+ * ties to the lower expert id; w[k] = (float)(score_k / (sum of the top_k scores + 1e-20) * route_scale). The reference
+ * fixes n_exp = 384, top_k = 6, route_scale = 1.5. */
+void orc_router(const float* logits, const float* bias, int n_exp, int top_k, float route_scale, int* ids, float* w);
+
+/* Expert-sorted routing lists of n_entries = n_tokens * top_k entries (arch_ref.cpp:114-130): counts[n_exp],
+ * offsets[n_exp + 1] (exclusive scan), and per sorted position p (expert-major, entry index ascending inside an expert)
+ * entry[p] = i, tok[p] = i / top_k, lw[p] = w[i]; slot_of[i] = p. */
+void orc_route_lists(const int* ids, const float* w, int n_entries, int n_exp, int top_k, uint32_t* counts,
+                     uint32_t* offsets, uint32_t* entry, uint32_t* tok, float* lw, uint32_t* slot_of);
 
 #ifdef __cplusplus
 }

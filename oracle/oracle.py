@@ -49,6 +49,8 @@ def load():
     L.orc_moe_prefill.argtypes = [i32] * 8 + [vp] * 8 + [i32, i32, vp, vp, i32]; L.orc_moe_prefill.restype = i32
     L.orc_randn.argtypes = [vp, i64, u64, f32]
     L.orc_random_blocks.argtypes = [i32, i64, u64, f32, vp]; L.orc_random_blocks.restype = i32
+    L.orc_router.argtypes = [vp, vp, i32, i32, f32, vp, vp]; L.orc_router.restype = None
+    L.orc_route_lists.argtypes = [vp, vp, i32, i32, i32] + [vp] * 6; L.orc_route_lists.restype = None
     _lib = L
     return L
 
@@ -67,6 +69,24 @@ def load_ref():
         R.refshim_fp16_to_f32.argtypes = [C.c_ushort]; R.refshim_fp16_to_f32.restype = C.c_float
         _ref = R
     return _ref
+
+
+_ref_arch = None
+
+
+def load_ref_arch():
+    """The reference's tests/ref/arch_ref.cpp (router, route lists) as a shared object, or None when not built here."""
+    global _ref_arch
+    if _ref_arch is None:
+        so = os.path.join(HERE, "_ref", "libref_arch.so")
+        if not os.path.exists(so):
+            return None
+        R = C.CDLL(so)
+        R.refshim_router.argtypes = [C.c_void_p] * 4 + [C.c_float]; R.refshim_router.restype = None
+        R.refshim_route_lists.argtypes = [C.c_void_p, C.c_void_p, C.c_int] + [C.c_void_p] * 6
+        R.refshim_route_lists.restype = None
+        _ref_arch = R
+    return _ref_arch
 
 
 def _p(a):
@@ -174,3 +194,53 @@ def moe_prefill(t_gu, t_down, t_shared, n_tokens, n_exp, has_shared, dim, inter,
     if rc != 0:
         raise ValueError("moe_prefill: unsupported arguments")
     return Y, Ymag
+
+
+N_EXPERTS, TOP_K, ROUTE_SCALE = 384, 6, 1.5  # the reference's router constants (src/kernels/arch_router.metal:5-6,53)
+
+
+def router(logits, bias, top_k=TOP_K, route_scale=ROUTE_SCALE):
+    """logits float32 [n, n_exp], bias float32 [n_exp] -> ids int32 [n, top_k], w float32 [n, top_k]."""
+    logits = np.ascontiguousarray(logits, dtype=np.float32)
+    bias = np.ascontiguousarray(bias, dtype=np.float32)
+    n, n_exp = logits.shape
+    ids = np.empty((n, top_k), dtype=np.int32)
+    w = np.empty((n, top_k), dtype=np.float32)
+    L = load()
+    for t in range(n):
+        L.orc_router(_p(logits[t]), _p(bias), n_exp, top_k, route_scale, _p(ids[t]), _p(w[t]))
+    return ids, w
+
+
+def ref_router(logits, bias, route_scale=ROUTE_SCALE):
+    R = load_ref_arch()
+    logits = np.ascontiguousarray(logits, dtype=np.float32)
+    bias = np.ascontiguousarray(bias, dtype=np.float32)
+    n = logits.shape[0]
+    ids = np.empty((n, 6), dtype=np.int32)
+    w = np.empty((n, 6), dtype=np.float32)
+    for t in range(n):
+        R.refshim_router(_p(logits[t]), _p(bias), _p(ids[t]), _p(w[t]), route_scale)
+    return ids, w
+
+
+def _route_outputs(n_entries, n_exp):
+    return (np.empty(n_exp, np.uint32), np.empty(n_exp + 1, np.uint32), np.empty(n_entries, np.uint32),
+            np.empty(n_entries, np.uint32), np.empty(n_entries, np.float32), np.empty(n_entries, np.uint32))
+
+
+def route_lists(ids, w, n_exp=N_EXPERTS, top_k=TOP_K):
+    """ids int32 / w float32 [n_tokens * top_k] -> (counts, offsets, entry, tok, lw, slot_of)."""
+    ids = np.ascontiguousarray(ids, dtype=np.int32).reshape(-1)
+    w = np.ascontiguousarray(w, dtype=np.float32).reshape(-1)
+    out = _route_outputs(ids.size, n_exp)
+    load().orc_route_lists(_p(ids), _p(w), ids.size, n_exp, top_k, *[_p(o) for o in out])
+    return out
+
+
+def ref_route_lists(ids, w):
+    ids = np.ascontiguousarray(ids, dtype=np.int32).reshape(-1)
+    w = np.ascontiguousarray(w, dtype=np.float32).reshape(-1)
+    out = _route_outputs(ids.size, 384)
+    load_ref_arch().refshim_route_lists(_p(ids), _p(w), ids.size // 6, *[_p(o) for o in out])
+    return out

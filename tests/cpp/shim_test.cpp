@@ -10,6 +10,7 @@
 #include <cstring>
 #include <vector>
 
+#include "macseek_amd/arch.hpp"
 #include "macseek_amd/quant.hpp"
 
 #define HIP_OK(e) do { hipError_t r_ = (e); if (r_ != hipSuccess) { fprintf(stderr, "HIP: %s\n", hipGetErrorString(r_)); return 2; } } while (0)
@@ -53,6 +54,37 @@ int main() {
   printf("  encode_matvec_n Q8_0 [%d -> %d] n=%d %s\n", cols, rows, n, f2 ? "FAIL" : "ok");
   fails += f2;
   if (mq::matvec_cfg(mq::QType::Q8_0, rows, cols).ks < 1) fails++;
+  {  // ms::arch router shim: known answers (ties go to the lower expert id; equal logits share the scale equally)
+    namespace ma = ms::arch;
+    const int nt = 2, E = ma::kExperts;
+    std::vector<float> logits((size_t)nt * E, -30.f), bias(E, 0.f);
+    const int pick[6] = {300, 200, 50, 100, 20, 10};
+    const float val[6] = {30.f, 25.f, 0.f, 0.f, -1.f, -2.f};
+    for (int k = 0; k < 6; k++) logits[pick[k]] = val[k];
+    for (int i = 0; i < E; i++) logits[E + i] = 0.f;
+    ms::Buffer bl = upload(logits.data(), logits.size() * 4), bb = upload(bias.data(), bias.size() * 4);
+    std::vector<uint32_t> z(512, 0);
+    ms::Buffer ids = upload(z.data(), nt * 24), wts = upload(z.data(), nt * 24);
+    ma::RouteLists L;
+    L.counts = upload(z.data(), E * 4); L.offsets = upload(z.data(), (E + 1) * 4);
+    L.entry = upload(z.data(), nt * 24); L.tok = upload(z.data(), nt * 24); L.w = upload(z.data(), nt * 24);
+    L.slot_of = upload(z.data(), nt * 24); L.max_tokens = nt;
+    ma::encode_router_topk(e, bl, bb, ids, wts, nt);
+    ma::encode_route_lists(e, ids, wts, nt, L);
+    HIP_OK(hipStreamSynchronize((hipStream_t)e.stream));
+    int gid[12]; float gw[12]; uint32_t off[385], slot[12], ent[12];
+    HIP_OK(hipMemcpy(gid, ids.buf, 48, hipMemcpyDeviceToHost)); HIP_OK(hipMemcpy(gw, wts.buf, 48, hipMemcpyDeviceToHost));
+    HIP_OK(hipMemcpy(off, L.offsets.buf, 385 * 4, hipMemcpyDeviceToHost)); HIP_OK(hipMemcpy(slot, L.slot_of.buf, 48, hipMemcpyDeviceToHost));
+    HIP_OK(hipMemcpy(ent, L.entry.buf, 48, hipMemcpyDeviceToHost));
+    int f3 = 0;
+    float sum0 = 0.f;
+    for (int k = 0; k < 6; k++) { f3 += gid[k] != pick[k]; f3 += gid[6 + k] != k; f3 += std::fabs(gw[6 + k] - 0.25f) > 1e-6f; sum0 += gw[k]; }
+    f3 += std::fabs(sum0 - 1.5f) > 1e-5f;
+    f3 += off[E] != 12;
+    for (int i = 0; i < 12; i++) f3 += ent[slot[i]] != (uint32_t)i;
+    printf("  ms::arch router_topk + route_lists %s\n", f3 ? "FAIL" : "ok");
+    fails += f3;
+  }
   // misuse aborts like the reference (src/kernels/quant.mm:34-37): cols not a multiple of the block size
   fflush(stdout);
   const pid_t pid = fork();

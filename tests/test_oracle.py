@@ -322,3 +322,66 @@ def test_generators():
         assert np.array_equal(b, O.random_blocks(t, 256 * 40, 3))
         w = O.dequant(t, b, 256 * 40)
         assert np.all(np.isfinite(w)) and np.max(np.abs(w)) < 100
+
+
+# ------------------------------------------------------------------------------------------------ router, route lists
+def _router_golden():
+    return np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "router_golden.npz"))
+
+
+def test_router_matches_reference_golden():
+    g = _router_golden()
+    ids, w = O.router(g["logits"], g["bias"])
+    assert np.array_equal(ids, g["ids"]) and np.array_equal(w.view(np.uint32), g["w_bits"])
+    lists = O.route_lists(ids, w)
+    for got, name in zip(lists, ("counts", "offsets", "entry", "tok", "lw_bits", "slot_of")):
+        assert np.array_equal(got.view(np.uint32), g[name]), name
+
+
+@pytest.mark.skipif(O.load_ref_arch() is None, reason="reference checkout not compiled here (oracle/_ref)")
+def test_router_differential_vs_compiled_reference():
+    logits = O.randn(200 * 384, 5, 3.0).reshape(200, 384)
+    logits[:, ::7] += 25.0
+    bias = O.randn(384, 6, 0.3)
+    ids, w = O.router(logits, bias)
+    rid, rw = O.ref_router(logits, bias)
+    assert np.array_equal(ids, rid) and np.array_equal(w.view(np.uint32), rw.view(np.uint32))
+    for a, b in zip(O.route_lists(ids, w), O.ref_route_lists(ids, w)):
+        assert np.array_equal(a.view(np.uint32), b.view(np.uint32))
+
+
+def test_router_known_answers():
+    # equal logits, zero bias: every key ties, the six lowest ids win and share the scale equally
+    ids, w = O.router(np.zeros((1, 384), np.float32), np.zeros(384, np.float32))
+    assert ids.tolist() == [[0, 1, 2, 3, 4, 5]] and np.allclose(w, 0.25, rtol=1e-7)
+    # score = sqrt(softplus(x)): ln 2 at 0, x itself above the threshold 20; weights are score ratios times 1.5
+    lg = np.full((1, 384), -30.0, np.float32)
+    lg[0, [300, 200, 100, 50, 20, 10]] = [30.0, 25.0, 0.0, 0.0, -1.0, -2.0]
+    ids, w = O.router(lg, np.zeros(384, np.float32))
+    sc = np.sqrt([30.0, 25.0, np.log(2.0), np.log(2.0), np.log1p(np.exp(-1.0)), np.log1p(np.exp(-2.0))])
+    assert ids.tolist() == [[300, 200, 50, 100, 20, 10]]  # the tie between 50 and 100 goes to the lower id
+    assert np.allclose(w[0], sc / sc.sum() * 1.5, rtol=1e-6) and abs(float(w.sum()) - 1.5) < 1e-6
+    # the bias picks, the score weighs: a large bias brings in an expert with a tiny score, first in the order
+    b = np.zeros(384, np.float32)
+    b[7] = 100.0
+    ids2, w2 = O.router(lg, b)
+    assert ids2[0, 0] == 7 and ids2[0, 1:].tolist() == [300, 200, 50, 100, 20]
+    s7 = np.sqrt(np.log1p(np.exp(-30.0)))
+    assert np.isclose(w2[0, 0], s7 / (s7 + sc[:5].sum()) * 1.5, rtol=1e-5)
+    # other sizes and scales
+    ids3, w3 = O.router(O.randn(4 * 128, 3).reshape(4, 128), np.zeros(128, np.float32), top_k=6, route_scale=2.5)
+    assert np.allclose(w3.sum(1), 2.5, rtol=1e-6) and all(len(set(r)) == 6 for r in ids3.tolist())
+
+
+def test_route_lists_are_a_stable_sort():
+    rng = np.random.default_rng(3)
+    for n, n_exp in ((1, 384), (17, 384), (300, 64), (0, 384)):
+        ids = rng.integers(0, n_exp, n * 6).astype(np.int32)
+        if n > 1:
+            ids[: 6 * (n // 2)] = ids[0]  # one crowded expert
+        w = rng.random(n * 6).astype(np.float32)
+        counts, offsets, entry, tok, lw, slot_of = O.route_lists(ids, w, n_exp=n_exp)
+        order = np.argsort(ids, kind="stable")
+        assert np.array_equal(entry, order) and np.array_equal(tok, order // 6) and np.array_equal(lw, w[order])
+        assert np.array_equal(slot_of[order], np.arange(n * 6)) and np.array_equal(counts, np.bincount(ids, minlength=n_exp))
+        assert np.array_equal(offsets, np.concatenate([[0], np.cumsum(counts)]))
