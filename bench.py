@@ -499,13 +499,66 @@ def bench_router(torch, args):
             "cpu_baseline": cpu, "pct_of_hbm_peak": 100 * gbps / HBM_PEAK_GBPS}
 
 
+def bench_matmul(torch, args):
+    """Prefill matmul Y[n x rows] = X[n x cols] . W^T (msq_matmul) at n = 2048 on the attention-projection shapes of
+    BASELINE configs[4]; value = algorithmic FLOPs (2 n rows cols) per second of the Q6_K 1536x7168 case, the whole call
+    (activation conversion, weight dequantization to fp16, GEMM) timed with a HIP event pair over back-to-back calls."""
+    import oracle as O
+    from macseek_amd import quant as q
+    dev = torch.device("cuda:0")
+    n = 2048
+    rows_out = []
+    for t, name, rows, cols in ((q.QType.Q6_K, "Q6_K", 1536, 7168), (q.QType.Q5_K, "Q5_K", 512, 7168),
+                                (q.QType.IQ4_NL, "IQ4_NL", 7168, 4096), (q.QType.BF16, "BF16", 384, 7168)):
+        if int(t) == 30:
+            W = (torch.randn(rows * cols, device=dev) * 0.02).to(torch.bfloat16).view(torch.uint8)
+        else:
+            W = gen_blocks(torch, t, rows * cols // q.block_elems(t), 0.01, 1, dev)
+        X = torch.randn(n * cols, device=dev)
+        Y = torch.zeros(n * rows, device=dev)
+        e = q.Enc()
+        Wb, Xb, Yb = q.Buffer.of(W), q.Buffer.of(X), q.Buffer.of(Y)
+        for _ in range(3):
+            q.encode_matmul(e, t, Wb, rows, cols, Xb, Yb, n)
+        torch.cuda.synchronize()
+        reps = 20
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for _ in range(reps):
+            q.encode_matmul(e, t, Wb, rows, cols, Xb, Yb, n)
+        b.record()
+        torch.cuda.synchronize()
+        ms = a.elapsed_time(b) / reps
+        flops = 2.0 * n * rows * cols
+        rows_out.append({"type": name, "rows": rows, "cols": cols, "n": n, "us_per_call": ms * 1e3, "TFLOPs": flops / (ms * 1e-3) / 1e12})
+    head = rows_out[0]
+    cpu = None
+    if not args.gpu_only:
+        rows, cols, nt = 1536, 7168, 64
+        Wh = O.random_blocks(O.Q6_K, rows * cols, 1)
+        xh = O.randn(nt * cols, 2)
+        nth = min(16, os.cpu_count() or 1)
+        t0 = time.perf_counter()
+        for i in range(nt):
+            O.matvec(O.Q6_K, Wh, rows, cols, xh[i * cols:(i + 1) * cols], 1, nth)
+        el = time.perf_counter() - t0
+        cpu = {"value": 2.0 * nt * rows * cols / el / 1e12, "unit": "TFLOP/s", "cores": nth, "kind": "port",
+               "sample": "%d tokens of the Q6_K 1536x7168 case through oracle.c (dequant each row, double dot), %.2f s; whole job = x%d" % (nt, el, n // nt)}
+    return {"value": head["TFLOPs"], "ms_per_step": head["us_per_call"] * 1e-3, "dtype": "f16 x f16 MFMA (weights and activations rounded to fp16), f32 accumulate",
+            "config": {"workload": "prefill matmul, 2048 tokens, BASELINE configs[4] shapes; one step = one msq_matmul call of the Q6_K 1536x7168 case", "cases": rows_out},
+            "roofline": {"bound": "mfma", "achieved": head["TFLOPs"], "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": head["TFLOPs"] / MFMA_PEAK_TFLOPS,
+                         "traffic": None, "kernel": "dequant_kernel<Q6_K, fp16> + rocBLAS fp16 GEMM (whole call)", "flops_per_launch": 2.0 * n * 1536 * 7168,
+                         "avg_launch_us": head["us_per_call"]},
+            "cpu_baseline": cpu}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=500)
     ap.add_argument("--warmup", type=int, default=100)
     ap.add_argument("--workload", default="moe_decode",
-                    choices=["moe_decode", "moe_prefill", "matvec_iq1s", "matvec_iq2xxs", "q8_0", "router", "stream", "copy_calibration"])
+                    choices=["moe_decode", "moe_prefill", "matvec_iq1s", "matvec_iq2xxs", "q8_0", "router", "matmul", "stream", "copy_calibration"])
     ap.add_argument("--gpu-only", action="store_true",
                     help="profiling runs: skip the CPU baseline leg and the prefill appendix of the default workload")
     args = ap.parse_args()
@@ -529,6 +582,13 @@ def main():
                "vs_baseline": None, "dtype": r["dtype"], "data": "synthetic", "config": r["config"], "roofline": r["roofline"],
                "cpu_baseline": r["cpu_baseline"], "pct_of_mfma_peak": r["pct_of_mfma_peak"]}
         print(json.dumps(out))
+        return
+    if args.workload == "matmul":
+        r = bench_matmul(torch, args)
+        print(json.dumps({"metric": METRIC, "value": r["value"], "unit": "TFLOP/s", "n_gpus": 1, "steps": 20, "warmup": 3,
+                          "ms_per_step": r["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+                          "dtype": r["dtype"], "data": "synthetic", "config": r["config"], "roofline": r["roofline"],
+                          "cpu_baseline": r["cpu_baseline"], "pct_of_mfma_peak": 100 * r["value"] / MFMA_PEAK_TFLOPS}))
         return
     if args.workload == "moe_decode":
         r = bench_moe_decode(torch, args)

@@ -68,6 +68,22 @@ inline void encode_matvec_n(Enc& e, QType t, const Buffer& W, int rows, int cols
   detail::check(msq_matvec_n(e.stream, (int)t, &w, rows, cols, &xb, &yb, n, accumulate, groups));
 }
 
+// reference: quant.hpp:40-45
+inline void encode_matmul(Enc& e, QType t, const Buffer& W, int rows, int cols, const Buffer& X, const Buffer& Y, int n,
+                          bool accumulate = false) {
+  const MsqBuffer w = W.c(), xb = X.c(), yb = Y.c();
+  detail::check(msq_matmul(e.stream, (int)t, &w, rows, cols, &xb, &yb, n, accumulate));
+}
+inline void encode_f32_to_f16(Enc& e, const Buffer& X, const Buffer& X16, size_t count) {
+  const MsqBuffer xb = X.c(), hb = X16.c();
+  detail::check(msq_f32_to_f16(e.stream, &xb, &hb, count));
+}
+inline void encode_matmul_h(Enc& e, QType t, const Buffer& W, int rows, int cols, const Buffer& X16, const Buffer& Y, int n,
+                            bool accumulate = false, int x_stride = 0) {
+  const MsqBuffer w = W.c(), xb = X16.c(), yb = Y.c();
+  detail::check(msq_matmul_h(e.stream, (int)t, &w, rows, cols, &xb, &yb, n, accumulate, x_stride));
+}
+
 // ---- MoE ----
 constexpr int kExpertDim = MSQ_EXPERT_DIM, kExpertInter = MSQ_EXPERT_INTER, kMaxRouted = MSQ_MAX_ROUTED;
 

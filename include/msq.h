@@ -88,6 +88,22 @@ int msq_matvec(void* stream, int qtype, const MsqBuffer* W, int rows, int cols, 
 int msq_matvec_n(void* stream, int qtype, const MsqBuffer* W, int rows, int cols, const MsqBuffer* X,
                  const MsqBuffer* Y, int n, int accumulate, int groups);
 
+/* reference: ms::q::encode_f32_to_f16 (quant.hpp:42, quant.mm:186-191). count % 4 == 0; X 16-byte aligned. */
+int msq_f32_to_f16(void* stream, const MsqBuffer* X, const MsqBuffer* X16, size_t count);
+
+/* reference: ms::q::encode_matmul_h (quant.hpp:43-45, quant.mm:193-238). Prefill matmul
+ * Y[n x rows] (+)= X16[n x x_stride] . W^T, X16 fp16 (x_stride = cols if 0), Y F32, any n >= 1, cols % 128 == 0.
+ * Weights are rounded to fp16 and products accumulate in fp32, the reference's numerics (quant.hpp:36-39). The fp16
+ * copy of W lives in scratch the library owns and grows on demand (reference: quant.mm:176-184): calls sharing it
+ * must be enqueued on one stream at a time, and a call that grows it synchronises that stream and allocates. */
+int msq_matmul_h(void* stream, int qtype, const MsqBuffer* W, int rows, int cols, const MsqBuffer* X16, const MsqBuffer* Y,
+                 int n, int accumulate, int x_stride);
+
+/* reference: ms::q::encode_matmul (quant.hpp:40-41, quant.mm:240-248): converts X (F32 [n x cols], 16-byte aligned)
+ * into library-owned fp16 scratch, then msq_matmul_h. */
+int msq_matmul(void* stream, int qtype, const MsqBuffer* W, int rows, int cols, const MsqBuffer* X, const MsqBuffer* Y, int n,
+               int accumulate);
+
 /* Whole-buffer dequantization to fp32, bit-exact with the reference's CPU dequantizer
  * (reference: ref::dequant_row, tests/ref/dequant.cpp:34-120; GPU relative: q_deq_f16, quant_mm.metal:143-154).
  * n_elems must be a multiple of the block size; out holds n_elems floats. */

@@ -59,6 +59,9 @@ SIGNATURES = {
     "msq_matvec_cfg": (C.c_int, [C.c_int, C.c_int, C.c_int, C.POINTER(MsqMvCfg)]),
     "msq_matvec": (C.c_int, [C.c_void_p, C.c_int, _BP, C.c_int, C.c_int, _BP, _BP, C.c_int, C.c_int, C.POINTER(MsqMvCfg)]),
     "msq_matvec_n": (C.c_int, [C.c_void_p, C.c_int, _BP, C.c_int, C.c_int, _BP, _BP, C.c_int, C.c_int, C.c_int]),
+    "msq_f32_to_f16": (C.c_int, [C.c_void_p, _BP, _BP, C.c_size_t]),
+    "msq_matmul_h": (C.c_int, [C.c_void_p, C.c_int, _BP, C.c_int, C.c_int, _BP, _BP, C.c_int, C.c_int, C.c_int]),
+    "msq_matmul": (C.c_int, [C.c_void_p, C.c_int, _BP, C.c_int, C.c_int, _BP, _BP, C.c_int, C.c_int]),
     "msq_dequant": (C.c_int, [C.c_void_p, C.c_int, _BP, C.c_int64, _BP]),
     "msq_bw_probe": (C.c_int, [C.c_void_p, _BP, C.c_size_t, _BP]),
     "msq_moe_decode_scratch_bytes": (C.c_size_t, [C.c_int]),

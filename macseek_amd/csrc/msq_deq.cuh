@@ -11,8 +11,10 @@ __device__ __forceinline__ float tbl_half(const uint32_t* w, int j) {  // elemen
   return half_bits_to_float((j & 1) ? (v >> 16) : (v & 0xFFFFu));
 }
 
-template <int QT>
-__global__ __launch_bounds__(256) void dequant_kernel(const uint8_t* __restrict__ src, float* __restrict__ dst, int64_t nchunks) {
+// OUT = float: the bit-exact fp32 result. OUT = uint16_t: the same values rounded to fp16 (nearest even), the weight
+// operand of the prefill matmul (reference: q_deq_f16, src/kernels/quant_mm.metal:143-154).
+template <int QT, class OUT = float>
+__global__ __launch_bounds__(256) void dequant_kernel(const uint8_t* __restrict__ src, OUT* __restrict__ dst, int64_t nchunks) {
 #pragma clang fp contract(off)
   const int64_t c = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (c >= nchunks) return;
@@ -86,9 +88,13 @@ __global__ __launch_bounds__(256) void dequant_kernel(const uint8_t* __restrict_
       y[j] = d1 * (float)q - m1;
     }
   }
-  float4* o = (float4*)(dst + 8 * c);
-  o[0] = make_float4(y[0], y[1], y[2], y[3]);
-  o[1] = make_float4(y[4], y[5], y[6], y[7]);
+  if constexpr (sizeof(OUT) == 4) {
+    float4* o = (float4*)(dst + 8 * c);
+    o[0] = make_float4(y[0], y[1], y[2], y[3]);
+    o[1] = make_float4(y[4], y[5], y[6], y[7]);
+  } else {
+    *(uint4*)(dst + 8 * c) = uint4{pack_h2(y[0], y[1]), pack_h2(y[2], y[3]), pack_h2(y[4], y[5]), pack_h2(y[6], y[7])};
+  }
 }
 
 }  // namespace msq

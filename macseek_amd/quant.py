@@ -122,6 +122,18 @@ def encode_matvec_n(e, t, W, rows, cols, X, Y, n, accumulate=False, groups=1):  
     _check(_lib.load().msq_matvec_n(e.handle, int(t), _bp(W), rows, cols, _bp(X), _bp(Y), n, int(bool(accumulate)), groups))
 
 
+def encode_matmul(e, t, W, rows, cols, X, Y, n, accumulate=False):  # reference: quant.hpp:40-41
+    _check(_lib.load().msq_matmul(e.handle, int(t), _bp(W), rows, cols, _bp(X), _bp(Y), n, int(bool(accumulate))))
+
+
+def encode_f32_to_f16(e, X, X16, count):  # reference: quant.hpp:42
+    _check(_lib.load().msq_f32_to_f16(e.handle, _bp(X), _bp(X16), count))
+
+
+def encode_matmul_h(e, t, W, rows, cols, X16, Y, n, accumulate=False, x_stride=0):  # reference: quant.hpp:43-45
+    _check(_lib.load().msq_matmul_h(e.handle, int(t), _bp(W), rows, cols, _bp(X16), _bp(Y), n, int(bool(accumulate)), x_stride))
+
+
 def encode_dequant(e, t, W, n_elems, out):
     """Whole-buffer dequantization to fp32 (bit-exact with ref::dequant_row, tests/ref/dequant.cpp:34-120)."""
     _check(_lib.load().msq_dequant(e.handle, int(t), _bp(W), n_elems, _bp(out)))
