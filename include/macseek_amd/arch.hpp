@@ -50,4 +50,11 @@ inline void encode_route_lists(Enc& e, Buffer ids, Buffer w, int n, const RouteL
   q::detail::check(msq_route_lists(e.stream, &ib, &wb, n, L.n_exp, &l));
 }
 
+// reference: arch.hpp:127-130 (w.buf == nullptr: no weight)
+inline void encode_rmsnorm(Enc& e, Buffer x, Buffer w, Buffer y, int rows, int dim, float eps, int in_stride = 0,
+                           int out_stride = 0) {
+  const MsqBuffer xb = x.c(), wb = w.c(), yb = y.c();
+  q::detail::check(msq_rmsnorm(e.stream, &xb, w.buf ? &wb : nullptr, &yb, rows, dim, eps, in_stride, out_stride));
+}
+
 }  // namespace ms::arch

@@ -62,6 +62,12 @@ inline void encode_matvec(Enc& e, QType t, const Buffer& W, int rows, int cols, 
   const MsqMvCfg c{cfg.nr, cfg.rsg, cfg.ks};
   detail::check(msq_matvec(e.stream, (int)t, &w, rows, cols, &xb, &yb, accumulate, groups, &c));
 }
+// reference: quant.hpp:20-26
+inline void encode_matvec_rmsnorm(Enc& e, QType t, const Buffer& W, int rows, int cols, const Buffer& x, const Buffer& norm_w,
+                                  float eps, const Buffer& y, int tiles_per_tg = 0) {
+  const MsqBuffer w = W.c(), xb = x.c(), nb = norm_w.c(), yb = y.c();
+  detail::check(msq_matvec_rmsnorm(e.stream, (int)t, &w, rows, cols, &xb, &nb, eps, &yb, tiles_per_tg));
+}
 inline void encode_matvec_n(Enc& e, QType t, const Buffer& W, int rows, int cols, const Buffer& X, const Buffer& Y, int n,
                             bool accumulate = false, int groups = 1) {
   const MsqBuffer w = W.c(), xb = X.c(), yb = Y.c();

@@ -76,6 +76,22 @@ int msq_matvec_cfg(int qtype, int rows, int cols, MsqMvCfg* out);
 int msq_matvec(void* stream, int qtype, const MsqBuffer* W, int rows, int cols, const MsqBuffer* x,
                const MsqBuffer* y, int accumulate, int groups, const MsqMvCfg* cfg);
 
+/* reference: ms::q::encode_matvec_rmsnorm (quant.hpp:20-26, quant.mm:107-127; kernel q_mv_rn, quant_mv.metal:58-141).
+ * y = W . (x * rsqrt(mean(x^2) + eps) * norm_w): the decode matvec with the input RMSNorm fused into the activation
+ * loads. Bit-identical to msq_rmsnorm(x, norm_w, tmp, 1, cols, eps) followed by msq_matvec(tmp) with no imposed launch
+ * shape, for every cols (the reference: for cols > 1024): each workgroup replays msq_rmsnorm's reduction exactly.
+ * Types F32 F16 BF16 Q8_0 Q5_K Q6_K (as the reference) and IQ4_NL; no block-diagonal groups, no accumulate; rows of
+ * up to about 15000 columns (the normalized row is staged in LDS). tiles_per_tg is accepted and ignored (workgroups
+ * are persistent: every one computes the scale once). */
+int msq_matvec_rmsnorm(void* stream, int qtype, const MsqBuffer* W, int rows, int cols, const MsqBuffer* x,
+                       const MsqBuffer* norm_w, float eps, const MsqBuffer* y, int tiles_per_tg);
+
+/* reference: ms::arch::encode_rmsnorm (src/kernels/arch.hpp:127-130; kernel arch_rmsnorm, src/kernels/arch_sample.metal:
+ * 216-233). y[r] = x[r] * rsqrt(mean(x[r]^2) + eps) * w for `rows` rows of `dim` floats; w may be NULL (no weight);
+ * strides in floats (0 = dim); y may alias x. */
+int msq_rmsnorm(void* stream, const MsqBuffer* x, const MsqBuffer* w, const MsqBuffer* y, int rows, int dim, float eps,
+                int in_stride, int out_stride);
+
 /* reference: ms::q::encode_matvec_n (quant.hpp:32-35, quant.mm:129-156).
  * Y[n x rows] (+)= X[n x cols] . W^T for n in 1..16 (one weight read serves all n tokens). X row stride is
  * cols * groups, Y row stride is rows. n == 1 is exactly msq_matvec. For n >= 2, rows of up to 16384 columns (dense

@@ -58,6 +58,8 @@ SIGNATURES = {
     "msq_matvec_supported": (C.c_int, [C.c_int]),
     "msq_matvec_cfg": (C.c_int, [C.c_int, C.c_int, C.c_int, C.POINTER(MsqMvCfg)]),
     "msq_matvec": (C.c_int, [C.c_void_p, C.c_int, _BP, C.c_int, C.c_int, _BP, _BP, C.c_int, C.c_int, C.POINTER(MsqMvCfg)]),
+    "msq_matvec_rmsnorm": (C.c_int, [C.c_void_p, C.c_int, _BP, C.c_int, C.c_int, _BP, _BP, C.c_float, _BP, C.c_int]),
+    "msq_rmsnorm": (C.c_int, [C.c_void_p, _BP, _BP, _BP, C.c_int, C.c_int, C.c_float, C.c_int, C.c_int]),
     "msq_matvec_n": (C.c_int, [C.c_void_p, C.c_int, _BP, C.c_int, C.c_int, _BP, _BP, C.c_int, C.c_int, C.c_int]),
     "msq_f32_to_f16": (C.c_int, [C.c_void_p, _BP, _BP, C.c_size_t]),
     "msq_matmul_h": (C.c_int, [C.c_void_p, C.c_int, _BP, C.c_int, C.c_int, _BP, _BP, C.c_int, C.c_int, C.c_int]),

@@ -63,3 +63,7 @@ class RouteLists:
 
 def encode_route_lists(e, ids, w, n, L):  # reference: arch.hpp:97
     _check(_lib.load().msq_route_lists(e.handle, _bp(ids), _bp(w), n, L.n_exp, C.byref(L.c())))
+
+
+def encode_rmsnorm(e, x, w, y, rows, dim, eps, in_stride=0, out_stride=0):  # reference: arch.hpp:127-130
+    _check(_lib.load().msq_rmsnorm(e.handle, _bp(x), _bp(w), _bp(y), rows, dim, eps, in_stride, out_stride))

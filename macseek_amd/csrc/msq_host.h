@@ -42,6 +42,6 @@ const DeviceInfo& device_info();  // cached facts of the current device (CU coun
 // small-N matvec through the dot-product kernels (msq_matvec.hip); MSQ_ERR_UNSUPPORTED, without a message, when the
 // shape does not fit them
 int matvec_tok(hipStream_t st, int t, const uint8_t* W, int rows, int cols, const float* X, float* Y, int n, int accumulate,
-               int groups, const MsqMvCfg* cfg = nullptr);
+               int groups, const MsqMvCfg* cfg = nullptr, const float* norm_w = nullptr, float eps = 0.f);
 
 }  // namespace msq

@@ -86,10 +86,28 @@ int launch_mv(hipStream_t st, const MvShape& s, MvArgs& a) {
   a.ks = s.ks;
   a.rpw = s.rpw;
   a.ntiles = (a.rows + tile_rows - 1) / tile_rows;
-  const size_t lds = (size_t)D::LDS_WORDS * 4 + (size_t)tile_rows * s.ks * 4;
+  size_t lds = (size_t)D::LDS_WORDS * 4 + (size_t)tile_rows * s.ks * 4;
+  if (a.norm_w) {  // fused input norm: partial sums and the normalized activations follow in LDS
+    lds = (lds + 15) / 16 * 16;
+    a.norm_off = (uint32_t)(lds / 4);
+    lds += 16 + (size_t)a.cols * 4;
+    if (lds > 64 * 1024) return MSQ_ERR_UNSUPPORTED;
+  }
   // persistent workgroups: as many as can be resident, never more than there are tiles
   const int wg_per_cu = std::max(1, std::min(2048 / threads, (int)((160 * 1024) / std::max<size_t>(lds, 1))));
   const int grid = (int)std::min<long>(a.ntiles, (long)device_info().cus * wg_per_cu);
+  if (a.norm_w) {
+    if constexpr (requires { D::STAGES; }) return MSQ_ERR_UNSUPPORTED;  // codebook formats: as in the reference (quant.mm:110)
+    else {
+      switch (s.iters) {
+        case 1: hipLaunchKernelGGL((mv_kernel<D, 1, true>), dim3(grid), dim3(threads), lds, st, a); break;
+        case 2: hipLaunchKernelGGL((mv_kernel<D, 2, true>), dim3(grid), dim3(threads), lds, st, a); break;
+        default: hipLaunchKernelGGL((mv_kernel<D, 4, true>), dim3(grid), dim3(threads), lds, st, a); break;
+      }
+      MSQ_HIP(hipGetLastError());
+      return MSQ_OK;
+    }
+  }
   if constexpr (requires { D::STAGES; }) {  // codebook formats: ring kernel (one unit per lane, matrix below 4 GiB)
     if (s.iters == 1 && (uint64_t)a.rows * a.row_bytes < (1ull << 32)) {
       hipLaunchKernelGGL((mv_ring_kernel<D>), dim3(grid), dim3(threads), lds, st, a);
@@ -157,8 +175,23 @@ int launch_mv_tok(hipStream_t st, const MvShape& s, MvTokArgs& ta) {
   a.ks = s.ks;
   a.rpw = s.rpw;
   a.ntiles = (a.rows + tile_rows - 1) / tile_rows;
-  const size_t lds = (size_t)D::LDS_WORDS * 4 + (size_t)tile_rows * s.ks * 4 * T * 4;
+  size_t lds = (size_t)D::LDS_WORDS * 4 + (size_t)tile_rows * s.ks * 4 * T * 4;
   const int gy = ((int)ta.n + T - 1) / T;
+  if (a.norm_w) {  // fused input norm (single token): partial sums and the normalized activations follow in LDS
+    lds = (lds + 15) / 16 * 16;
+    a.norm_off = (uint32_t)(lds / 4);
+    lds += 16 + (size_t)a.cols * 4;
+    if (lds > 64 * 1024) return MSQ_ERR_UNSUPPORTED;
+    if constexpr (T != 1 || requires { D::STAGES; }) return MSQ_ERR_UNSUPPORTED;
+    else {
+      const int gxn = (int)std::min<long>(a.ntiles, std::max(1, device_info().cus));
+      if (s.iters == 1) hipLaunchKernelGGL((mv_tok_kernel<D, 1, 1, true>), dim3(gxn), dim3(threads), lds, st, ta);
+      else if constexpr (D::UNIT == 8) hipLaunchKernelGGL((mv_tok_kernel<D, 2, 1, true>), dim3(gxn), dim3(threads), lds, st, ta);
+      else return MSQ_ERR_UNSUPPORTED;
+      MSQ_HIP(hipGetLastError());
+      return MSQ_OK;
+    }
+  }
   // persistent workgroups, one per CU over all token groups
   const int gx = (int)std::min<long>(a.ntiles, std::max(1, device_info().cus / gy));
   const dim3 grid((unsigned)gx, (unsigned)gy);
@@ -202,7 +235,7 @@ namespace msq {
 // Small-N matvec through the dot-product kernels. Returns MSQ_ERR_UNSUPPORTED without an error message when the shape
 // does not fit them (the caller then takes another path). Arguments are already validated.
 int matvec_tok(hipStream_t st, int t, const uint8_t* W, int rows, int cols, const float* X, float* Y, int n, int accumulate,
-               int groups, const MsqMvCfg* cfg) {
+               int groups, const MsqMvCfg* cfg, const float* norm_w, float eps) {
   // Q8_0 keeps fp32 activations (32 registers per token): four tokens per pass, the other formats eight
   const int T = n == 1 ? 1 : (t == MSQ_Q8_0 || n <= 4) ? 4 : 8;
   MvShape s;
@@ -214,6 +247,7 @@ int matvec_tok(hipStream_t st, int t, const uint8_t* W, int rows, int cols, cons
   a.rows = (uint32_t)rows; a.cols = (uint32_t)cols; a.row_bytes = (uint32_t)msq_type_row_bytes(t, cols);
   a.rows_per_group = (uint32_t)(rows / groups); a.x_group_stride = (uint32_t)cols; a.accumulate = accumulate ? 1u : 0u;
   ta.n = (uint32_t)n; ta.x_stride = (uint32_t)((size_t)cols * groups); ta.y_stride = (uint32_t)rows;
+  a.norm_w = norm_w; a.eps = eps;
   if (n == 1) return t == MSQ_Q8_0 ? launch_mv_tok<DecQ8_0, 1>(st, s, ta) : launch_mv_tok_t<1>(st, t, s, ta);
   if (t == MSQ_Q8_0) return launch_mv_tok<DecQ8_0, 4>(st, s, ta);
   return T == 4 ? launch_mv_tok_t<4>(st, t, s, ta) : launch_mv_tok_t<8>(st, t, s, ta);
@@ -251,19 +285,20 @@ int msq_matvec_cfg(int t, int rows, int cols, MsqMvCfg* out) {
   return MSQ_OK;
 }
 
-int msq_matvec(void* stream, int t, const MsqBuffer* W, int rows, int cols, const MsqBuffer* x, const MsqBuffer* y,
-               int accumulate, int groups, const MsqMvCfg* cfg) {
-  if (!mv_type_ok(t) || rows < 1 || cols < 1 || cols % mv_col_multiple(t) || groups < 1 || rows % groups)
-    return unsupported("matvec", t, rows, cols);
+// msq_matvec and msq_matvec_rmsnorm (norm_w != nullptr: the activations are normalized on the way in; the kernel is the
+// one msq_matvec picks for the matrix, so the two agree bit for bit on a pre-normalized input)
+static int matvec_impl(void* stream, const char* what, int t, const MsqBuffer* W, int rows, int cols, const MsqBuffer* x,
+                       const MsqBuffer* y, int accumulate, int groups, const MsqMvCfg* cfg, const float* norm_w, float eps) {
   const size_t rb = msq_type_row_bytes(t, cols);
   if (!buf_ok(W, rb * (size_t)rows) || !buf_ok(x, (size_t)cols * groups * 4) || !buf_ok(y, (size_t)rows * 4))
-    return fail(MSQ_ERR_ARGUMENT, "macseek quant: matvec: buffer missing or too small (type %s rows %d cols %d)",
+    return fail(MSQ_ERR_ARGUMENT, "macseek quant: %s: buffer missing or too small (type %s rows %d cols %d)", what,
                 msq_type_name_of(t), rows, cols);
   hipStream_t st = (hipStream_t)stream;
   {  // shapes with several rows per wave (chosen for matrices of more than a row per wave and CU, or imposed by cfg) go
      // through the prefetching kernel; a shape names its kernel, so row chunks launched with the shape of the whole
      // matrix repeat its bits
-    const int rc = matvec_tok(st, t, bptr(W), rows, cols, (const float*)bptr(x), (float*)bptr_mut(y), 1, accumulate, groups, cfg);
+    const int rc = matvec_tok(st, t, bptr(W), rows, cols, (const float*)bptr(x), (float*)bptr_mut(y), 1, accumulate, groups, cfg,
+                              norm_w, eps);
     if (rc != MSQ_ERR_UNSUPPORTED) return rc;
   }
   MvShape s;
@@ -272,18 +307,53 @@ int msq_matvec(void* stream, int t, const MsqBuffer* W, int rows, int cols, cons
   a.W = bptr(W); a.x = (const float*)bptr(x); a.y = (float*)bptr_mut(y);
   a.rows = (uint32_t)rows; a.cols = (uint32_t)cols; a.row_bytes = (uint32_t)rb;
   a.rows_per_group = (uint32_t)(rows / groups); a.x_group_stride = (uint32_t)cols; a.accumulate = accumulate ? 1u : 0u;
+  a.norm_w = norm_w; a.eps = eps;
+  int rc = MSQ_ERR_UNSUPPORTED;
   switch (t) {
-    case MSQ_IQ1_S: return launch_mv<DecIQ1S>(st, s, a);
-    case MSQ_IQ2_XXS: return launch_mv<DecIQ2XXS>(st, s, a);
-    case MSQ_Q8_0: return launch_mv<DecQ8_0>(st, s, a);
-    case MSQ_IQ4_NL: return launch_mv<DecIQ4NL>(st, s, a);
-    case MSQ_Q6_K: return launch_mv<DecQ6K>(st, s, a);
-    case MSQ_Q5_K: return launch_mv<DecQ5K>(st, s, a);
-    case MSQ_F32: return launch_mv<DecDense<MSQ_F32>>(st, s, a);
-    case MSQ_F16: return launch_mv<DecDense<MSQ_F16>>(st, s, a);
-    case MSQ_BF16: return launch_mv<DecDense<MSQ_BF16>>(st, s, a);
+    case MSQ_IQ1_S: rc = launch_mv<DecIQ1S>(st, s, a); break;
+    case MSQ_IQ2_XXS: rc = launch_mv<DecIQ2XXS>(st, s, a); break;
+    case MSQ_Q8_0: rc = launch_mv<DecQ8_0>(st, s, a); break;
+    case MSQ_IQ4_NL: rc = launch_mv<DecIQ4NL>(st, s, a); break;
+    case MSQ_Q6_K: rc = launch_mv<DecQ6K>(st, s, a); break;
+    case MSQ_Q5_K: rc = launch_mv<DecQ5K>(st, s, a); break;
+    case MSQ_F32: rc = launch_mv<DecDense<MSQ_F32>>(st, s, a); break;
+    case MSQ_F16: rc = launch_mv<DecDense<MSQ_F16>>(st, s, a); break;
+    case MSQ_BF16: rc = launch_mv<DecDense<MSQ_BF16>>(st, s, a); break;
   }
-  return unsupported("matvec", t, rows, cols);
+  return rc == MSQ_ERR_UNSUPPORTED ? unsupported(what, t, rows, cols) : rc;
+}
+
+int msq_matvec(void* stream, int t, const MsqBuffer* W, int rows, int cols, const MsqBuffer* x, const MsqBuffer* y,
+               int accumulate, int groups, const MsqMvCfg* cfg) {
+  if (!mv_type_ok(t) || rows < 1 || cols < 1 || cols % mv_col_multiple(t) || groups < 1 || rows % groups)
+    return unsupported("matvec", t, rows, cols);
+  return matvec_impl(stream, "matvec", t, W, rows, cols, x, y, accumulate, groups, cfg, nullptr, 0.f);
+}
+
+int msq_matvec_rmsnorm(void* stream, int t, const MsqBuffer* W, int rows, int cols, const MsqBuffer* x, const MsqBuffer* norm_w,
+                       float eps, const MsqBuffer* y, int tiles_per_tg) {
+  (void)tiles_per_tg;  // the reference's amortisation knob for the norm prologue; workgroups here are persistent
+  if (!mv_type_ok(t) || t == MSQ_IQ1_S || t == MSQ_IQ2_XXS || rows < 1 || cols < 1 || cols % mv_col_multiple(t))
+    return unsupported("matvec_rmsnorm", t, rows, cols);
+  if (!buf_ok(norm_w, (size_t)cols * 4))
+    return fail(MSQ_ERR_ARGUMENT, "macseek quant: matvec_rmsnorm: norm weights missing or too small (cols %d)", cols);
+  return matvec_impl(stream, "matvec_rmsnorm", t, W, rows, cols, x, y, 0, 1, nullptr, (const float*)bptr(norm_w), eps);
+}
+
+int msq_rmsnorm(void* stream, const MsqBuffer* x, const MsqBuffer* w, const MsqBuffer* y, int rows, int dim, float eps,
+                int in_stride, int out_stride) {
+  if (rows < 0 || dim < 1 || (in_stride && in_stride < dim) || (out_stride && out_stride < dim))
+    return unsupported("rmsnorm", MSQ_F32, rows, dim);
+  if (rows == 0) return MSQ_OK;
+  const int is = in_stride ? in_stride : dim, os = out_stride ? out_stride : dim;
+  const bool has_w = w && w->dev;
+  if (!buf_ok(x, ((size_t)(rows - 1) * is + dim) * 4) || !buf_ok(y, ((size_t)(rows - 1) * os + dim) * 4) ||
+      (has_w && !buf_ok(w, (size_t)dim * 4)))
+    return fail(MSQ_ERR_ARGUMENT, "macseek quant: rmsnorm: buffer missing or too small (rows %d dim %d)", rows, dim);
+  hipLaunchKernelGGL(rmsnorm_kernel, dim3((unsigned)rows), dim3(256), 0, (hipStream_t)stream, (const float*)bptr(x),
+                     has_w ? (const float*)bptr(w) : nullptr, (float*)bptr_mut(y), (uint32_t)dim, eps, (uint32_t)is, (uint32_t)os);
+  MSQ_HIP(hipGetLastError());
+  return MSQ_OK;
 }
 
 int msq_bw_probe(void* stream, const MsqBuffer* src, size_t bytes, const MsqBuffer* sink) {

@@ -24,9 +24,63 @@ struct MvArgs {
   uint32_t ks;      // waves splitting K
   uint32_t rpw;     // rows per wave per tile
   uint32_t ntiles;  // ceil(rows / (RW * rpw))
+  // fused input RMSNorm (NORM kernels only): x is replaced by x * rsqrt(mean(x^2) + eps) * norm_w
+  const float* norm_w;
+  float eps;
+  uint32_t norm_off;  // word offset in dynamic LDS of {partial sums [4], normalized activations [cols]}
 };
 
-template <class D, int ITERS>
+// ---------------------------------------------------------------------------------------------------- RMSNorm
+// scale = 1 / sqrt(mean(x^2) + eps) of one row, computed by a workgroup with a reduction whose order does not depend
+// on the workgroup's size: four virtual waves, virtual lane v (0..255) adds x[v], x[v + 256], ... with fused
+// multiply-adds, a DPP wave sum per virtual wave, then (s0 + s1) + (s2 + s3). The standalone norm kernel and the
+// matvec kernels with a fused norm both call this, so "norm, then matvec" and the fused call produce the same bits
+// (reference contract: src/kernels/quant.hpp:20-23; reduction being replayed there: src/kernels/quant_mv.metal:72-86).
+// `red` is four floats of LDS; all threads of the workgroup must call (it synchronises).
+__device__ __forceinline__ float rms_scale(const float* __restrict__ x, uint32_t dim, float eps, float* red, uint32_t lane,
+                                           uint32_t wave, uint32_t nwaves) {
+  for (uint32_t v = wave; v < 4u; v += nwaves) {
+    float ss = 0.f;
+    for (uint32_t i = v * 64u + lane; i < dim; i += 256u) ss = __builtin_fmaf(x[i], x[i], ss);
+    ss = wave_sum(ss);
+    if (lane == 0) red[v] = ss;
+  }
+  __syncthreads();
+  const float total = (red[0] + red[1]) + (red[2] + red[3]);
+  return 1.0f / __builtin_sqrtf(total / (float)dim + eps);
+}
+
+// y[row] = (x[row] * scale) * w (w may be null): reference ms::arch::encode_rmsnorm (src/kernels/arch.hpp:127-130,
+// kernel arch_rmsnorm, src/kernels/arch_sample.metal:216-233). One workgroup of 256 threads per row; y may alias x.
+__global__ __launch_bounds__(256) void rmsnorm_kernel(const float* x, const float* __restrict__ w, float* y, uint32_t dim,
+                                                      float eps, uint32_t in_stride, uint32_t out_stride) {
+  __shared__ float red[4];
+  const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+  const float* xr = x + (size_t)blockIdx.x * in_stride;
+  float* yr = y + (size_t)blockIdx.x * out_stride;
+  const float r = rms_scale(xr, dim, eps, red, lane, wave, 4u);
+  for (uint32_t i = tid; i < dim; i += 256u) {
+    const float v = xr[i] * r;
+    yr[i] = w ? v * w[i] : v;
+  }
+}
+
+// Prologue of the NORM matvec kernels: the normalized activations of the (single) input row go to LDS as fp32, from
+// where load_x() converts them exactly as it would from device memory. Returns the LDS row.
+__device__ __forceinline__ const float* stage_normed_x(const MvArgs& a, uint32_t* smem, uint32_t tid, uint32_t lane, uint32_t wave,
+                                                       uint32_t nwaves) {
+  float* red = (float*)(smem + a.norm_off);
+  float* xs = red + 4;
+  const float r = rms_scale(a.x, a.cols, a.eps, red, lane, wave, nwaves);
+  for (uint32_t i = tid; i < a.cols; i += nwaves * 64u) {
+    const float v = a.x[i] * r;
+    xs[i] = v * a.norm_w[i];
+  }
+  __syncthreads();
+  return xs;
+}
+
+template <class D, int ITERS, bool NORM = false>
 __global__ __launch_bounds__(1024) void mv_kernel(const MvArgs a) {
   extern __shared__ __attribute__((aligned(16))) uint32_t smem[];
   uint32_t* tbl = smem;
@@ -48,13 +102,15 @@ __global__ __launch_bounds__(1024) void mv_kernel(const MvArgs a) {
   }
   typename D::X xr[ITERS];
   uint32_t cur_group = 0xFFFFFFFFu;
-  if (D::LDS_WORDS) __syncthreads();
+  const float* xbase = a.x;
+  if constexpr (NORM) xbase = stage_normed_x(a, smem, tid, lane, wave, nwaves);  // synchronises (one group only)
+  else if (D::LDS_WORDS) __syncthreads();
 
   for (uint32_t tile = blockIdx.x; tile < a.ntiles; tile += gridDim.x) {
     const uint32_t tile_row0 = tile * tile_rows;
     const uint32_t group = tile_row0 / a.rows_per_group;  // a tile never straddles two groups (host guarantees)
     if (group != cur_group) {
-      const float* xg = a.x + (size_t)group * a.x_group_stride;
+      const float* xg = xbase + (size_t)group * a.x_group_stride;
 #pragma unroll
       for (int i = 0; i < ITERS; i++) xr[i] = D::load_x(xg, unit[i]);
       cur_group = group;
@@ -202,7 +258,7 @@ struct MvTokArgs {
   uint32_t x_stride, y_stride;   // elements between the activation / output rows of consecutive tokens
 };
 
-template <class D, int ITERS, int T>
+template <class D, int ITERS, int T, bool NORM = false>
 __global__ __launch_bounds__(512) void mv_tok_kernel(const MvTokArgs ta) {
   const MvArgs& a = ta.m;
   extern __shared__ __attribute__((aligned(16))) uint32_t smem[];
@@ -227,7 +283,9 @@ __global__ __launch_bounds__(512) void mv_tok_kernel(const MvTokArgs ta) {
   }
   typename D::X xr[T][ITERS];
   uint32_t cur_group = 0xFFFFFFFFu;
-  if (D::LDS_WORDS) __syncthreads();
+  const float* xbase = a.x;
+  if constexpr (NORM) xbase = stage_normed_x(a, smem, tid, lane, wave, nwaves);  // synchronises (one token, one group)
+  else if (D::LDS_WORDS) __syncthreads();
 
   for (uint32_t tile = blockIdx.x; tile < a.ntiles; tile += gridDim.x) {
     const uint32_t tile_row0 = tile * tile_rows;
@@ -235,7 +293,7 @@ __global__ __launch_bounds__(512) void mv_tok_kernel(const MvTokArgs ta) {
     if (group != cur_group) {
 #pragma unroll
       for (int t = 0; t < T; t++) {  // tokens past the last repeat it; their results are never stored
-        const float* xg = a.x + (size_t)min(t0 + t, ta.n - 1) * ta.x_stride + (size_t)group * a.x_group_stride;
+        const float* xg = xbase + (size_t)min(t0 + t, ta.n - 1) * ta.x_stride + (size_t)group * a.x_group_stride;
 #pragma unroll
         for (int i = 0; i < ITERS; i++) xr[t][i] = D::load_x(xg, unit[i]);
       }

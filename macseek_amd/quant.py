@@ -118,6 +118,10 @@ def encode_matvec(e, t, W, rows, cols, x, y, accumulate=False, groups=1, cfg=Non
                                   C.byref(c) if c is not None else None))
 
 
+def encode_matvec_rmsnorm(e, t, W, rows, cols, x, norm_w, eps, y, tiles_per_tg=0):  # reference: quant.hpp:20-26
+    _check(_lib.load().msq_matvec_rmsnorm(e.handle, int(t), _bp(W), rows, cols, _bp(x), _bp(norm_w), eps, _bp(y), tiles_per_tg))
+
+
 def encode_matvec_n(e, t, W, rows, cols, X, Y, n, accumulate=False, groups=1):  # reference: quant.hpp:32-35
     _check(_lib.load().msq_matvec_n(e.handle, int(t), _bp(W), rows, cols, _bp(X), _bp(Y), n, int(bool(accumulate)), groups))
 

@@ -463,3 +463,10 @@ void orc_route_lists(const int* ids, const float* w, int n_entries, int n_exp, i
   }
   free(fill);
 }
+
+void orc_rmsnorm(const float* x, const float* w, float* y, int dim, double eps) {
+  double ss = 0;
+  for (int i = 0; i < dim; i++) ss += (double)x[i] * x[i];
+  const double r = 1.0 / sqrt(ss / dim + eps);
+  for (int i = 0; i < dim; i++) y[i] = (float)(x[i] * r * (w ? w[i] : 1.0f));
+}

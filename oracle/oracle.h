@@ -12,6 +12,7 @@
  *   MoE prefill reference tests/test_quant_moe_prefill.mm:25-47,186-212; reduce order
  *                         src/kernels/quant_moe_prefill.metal:330-344
  *   router, route lists   tests/ref/arch_ref.cpp:97-130 (kernels: src/kernels/arch_router.metal:26-160)
+ *   rmsnorm               tests/ref/arch_ref.cpp:66-71
  *
  * Pinned by: bit-equality with the reference's own dequant.cpp compiled from /root/reference (oracle/_ref, and the
  * golden fixtures written from it under tests/golden/), closed-form known answers per format, codebook invariants,
@@ -87,6 +88,9 @@ int orc_random_blocks(int t, int64_t n_elems, uint64_t seed, float scale, uint8_
  * ties to the lower expert id; w[k] = (float)(score_k / (sum of the top_k scores + 1e-20) * route_scale). The reference
  * fixes n_exp = 384, top_k = 6, route_scale = 1.5. */
 void orc_router(const float* logits, const float* bias, int n_exp, int top_k, float route_scale, int* ids, float* w);
+
+/* y[i] = (float)(x[i] * r * w[i]) with r = 1 / sqrt(mean(x^2) + eps) in double; w may be NULL (tests/ref/arch_ref.cpp:66-71) */
+void orc_rmsnorm(const float* x, const float* w, float* y, int dim, double eps);
 
 /* Expert-sorted routing lists of n_entries = n_tokens * top_k entries (arch_ref.cpp:114-130): counts[n_exp],
  * offsets[n_exp + 1] (exclusive scan), and per sorted position p (expert-major, entry index ascending inside an expert)

@@ -50,6 +50,7 @@ def load():
     L.orc_randn.argtypes = [vp, i64, u64, f32]
     L.orc_random_blocks.argtypes = [i32, i64, u64, f32, vp]; L.orc_random_blocks.restype = i32
     L.orc_router.argtypes = [vp, vp, i32, i32, f32, vp, vp]; L.orc_router.restype = None
+    L.orc_rmsnorm.argtypes = [vp, vp, vp, i32, C.c_double]; L.orc_rmsnorm.restype = None
     L.orc_route_lists.argtypes = [vp, vp, i32, i32, i32] + [vp] * 6; L.orc_route_lists.restype = None
     _lib = L
     return L
@@ -85,6 +86,7 @@ def load_ref_arch():
         R.refshim_router.argtypes = [C.c_void_p] * 4 + [C.c_float]; R.refshim_router.restype = None
         R.refshim_route_lists.argtypes = [C.c_void_p, C.c_void_p, C.c_int] + [C.c_void_p] * 6
         R.refshim_route_lists.restype = None
+        R.refshim_rmsnorm.argtypes = [C.c_void_p] * 3 + [C.c_int, C.c_double]; R.refshim_rmsnorm.restype = None
         _ref_arch = R
     return _ref_arch
 
@@ -244,3 +246,20 @@ def ref_route_lists(ids, w):
     out = _route_outputs(ids.size, 384)
     load_ref_arch().refshim_route_lists(_p(ids), _p(w), ids.size // 6, *[_p(o) for o in out])
     return out
+
+
+def rmsnorm(x, w, eps):
+    """float32[dim]: x * rsqrt(mean(x^2) + eps) * w in double, rounded once (w may be None)."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    w = None if w is None else np.ascontiguousarray(w, dtype=np.float32)
+    y = np.empty_like(x)
+    load().orc_rmsnorm(_p(x), _p(w) if w is not None else None, _p(y), x.size, float(eps))
+    return y
+
+
+def ref_rmsnorm(x, w, eps):
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    w = None if w is None else np.ascontiguousarray(w, dtype=np.float32)
+    y = np.empty_like(x)
+    load_ref_arch().refshim_rmsnorm(_p(x), _p(w) if w is not None else None, _p(y), x.size, float(eps))
+    return y

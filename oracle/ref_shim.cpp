@@ -22,6 +22,7 @@ extern "C" {
 void refshim_router(const float* logits, const float* bias, int* ids, float* w, float route_scale) {
   ref_arch::router(logits, bias, ids, w, route_scale);
 }
+void refshim_rmsnorm(const float* x, const float* w, float* y, int dim, double eps) { ref_arch::rmsnorm(x, w, y, dim, eps); }
 void refshim_route_lists(const int* ids, const float* w, int n, unsigned* counts, unsigned* offsets, unsigned* entry,
                          unsigned* tok, float* lw, unsigned* slot_of) {
   std::vector<uint32_t> c, o, e, t, s;

@@ -385,3 +385,18 @@ def test_route_lists_are_a_stable_sort():
         assert np.array_equal(entry, order) and np.array_equal(tok, order // 6) and np.array_equal(lw, w[order])
         assert np.array_equal(slot_of[order], np.arange(n * 6)) and np.array_equal(counts, np.bincount(ids, minlength=n_exp))
         assert np.array_equal(offsets, np.concatenate([[0], np.cumsum(counts)]))
+
+
+def test_rmsnorm_known_answers_and_reference():
+    x = np.full(512, 2.0, np.float32)
+    assert np.allclose(O.rmsnorm(x, None, 0.0), 1.0, rtol=1e-7)                 # x / sqrt(mean(x^2)) = 1
+    w = np.arange(512, dtype=np.float32)
+    assert np.allclose(O.rmsnorm(x, w, 0.0), w, rtol=1e-7)                      # ... times the weight
+    assert np.allclose(O.rmsnorm(x, None, 12.0), 2.0 / 4.0, rtol=1e-7)          # sqrt(4 + 12) = 4
+    xr, wr = O.randn(1280, 3, 3.0), 1.0 + 0.2 * O.randn(1280, 4)
+    y = O.rmsnorm(xr, wr, 1e-20)
+    want = xr.astype(np.float64) / np.sqrt(np.mean(xr.astype(np.float64) ** 2) + 1e-20) * wr
+    assert np.allclose(y, want, rtol=2e-7, atol=0)
+    if O.load_ref_arch() is not None:
+        assert np.array_equal(y.view(np.uint32), O.ref_rmsnorm(xr, wr, 1e-20).view(np.uint32))
+        assert np.array_equal(O.rmsnorm(xr, None, 1e-6).view(np.uint32), O.ref_rmsnorm(xr, None, 1e-6).view(np.uint32))
