@@ -251,7 +251,8 @@ def bench_matvec(torch, args, t, rows, cols, d_sigma, label):
     ms_step = timed_graph(torch, lambda n: [launch(i) for i in range(n)], args.steps, args.warmup)
     step_bytes = mat_b + 4 * cols + 4 * rows
     value = step_bytes / (ms_step * 1e-3) / 1e9
-    k_mean, k_med, k_min = event_ms_per_launch(torch, launch, min(max(args.steps, 50), 400))
+    e_mean, e_med, e_min = event_ms_per_launch(torch, launch, min(max(args.steps, 50), 400))
+    k_mean = graph_ms_per_launch(torch, launch, 400)  # an eager event pair brackets the host's launch latency as well
     achieved = step_bytes / (k_mean * 1e-3) / 1e9
     nth = cores()
     Wh, xh = arena[:mat_b].cpu().numpy(), x.cpu().numpy()
@@ -261,14 +262,16 @@ def bench_matvec(torch, args, t, rows, cols, d_sigma, label):
         O.matvec(int(t), Wh, rows, cols, xh, 1, nthreads=nth)
         n_cpu += 1
         el = time.perf_counter() - t0
-        if el > 10.0 or n_cpu >= 2000:
+        if el > (0.2 if args.gpu_only else 10.0) or n_cpu >= 2000:  # profiling runs: a token CPU leg
             break
     return {
         "value": value, "ms_per_step": ms_step, "dtype": "f32" if t == q.QType.Q8_0 else "f16 activations, f32 accumulate",
         "config": {"workload": label, "bytes_per_step": step_bytes, "rows": rows, "cols": cols, "weight_copies": copies},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBPS,
-                     "traffic": None, "kernel": "mv_kernel<%s>" % q.type_name(t), "bytes_per_launch": step_bytes,
-                     "avg_launch_us": k_mean * 1e3, "median_launch_us": k_med * 1e3, "min_launch_us": k_min * 1e3},
+                     "traffic": None, "kernel": "decode matvec <%s> (mv_tok_kernel, mv_kernel or mv_ring_kernel by shape)" % q.type_name(t),
+                     "bytes_per_launch": step_bytes, "avg_launch_us": k_mean * 1e3,
+                     "timing": "HIP event pair around one graph replay of 400 back-to-back launches",
+                     "eager_event_pair_us": {"mean": e_mean * 1e3, "median": e_med * 1e3, "min": e_min * 1e3}},
         "cpu_baseline": {"value": step_bytes * n_cpu / el / 1e9, "unit": "GB/s", "cores": nth, "kind": "port",
                          "sample": "%d matvecs of the same matrix through oracle.c (dequant row + double dot), %.1f s" % (n_cpu, el)},
         "pct_of_hbm_peak": 100 * value / HBM_PEAK_GBPS,
@@ -358,11 +361,11 @@ def bench_moe_prefill(torch, steps, warmup, with_cpu=True):
                    "tokens_per_expert_median": float(np.median(counts[used])), "flops_per_step": flops,
                    "weight_bytes_touched": int(len(used)) * per_exp},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": achieved / MFMA_PEAK_TFLOPS,
-                     "traffic": None, "kernel": "moe_pf_block_kernel<BlkIQ2XXS, gate/up> (two launches: multi-tile items, one-tile items)",
+                     "traffic": None, "kernel": "moe_pf_block_kernel<BlkIQ2XXS, gate/up> (three launches: 49..80-entry blocks, two- and three-tile items, one-tile items)",
                      "flops_per_launch": gu_flops,
                      "avg_launch_us": gu_mean * 1e3, "min_launch_us": gu_min * 1e3,
                      "weight_GBps": int(len(used)) * 2 * gu_b / (gu_mean * 1e-3) / 1e9,
-                     "second_kernel": {"kernel": "moe_pf_block_kernel<BlkIQ2XXS, down> (two launches)", "avg_launch_us": dn_mean * 1e3,
+                     "second_kernel": {"kernel": "moe_pf_block_kernel<BlkIQ2XXS, down> (three launches)", "avg_launch_us": dn_mean * 1e3,
                                        "achieved": 2.0 * DIM * INTER * total / (dn_mean * 1e-3) / 1e12}},
         "pct_of_mfma_peak": 100 * value / MFMA_PEAK_TFLOPS,
     }
@@ -440,6 +443,64 @@ def bench_copy_calibration(torch, args):
             "roofline": {"bound": "hbm", "achieved": gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": gbps / HBM_PEAK_GBPS, "traffic": 2 * n,
                          "kernel": "torch elementwise copy"},
             "cpu_baseline": None, "pct_of_hbm_peak": 100 * gbps / HBM_PEAK_GBPS}
+
+
+def bench_matvec_n(torch, args):
+    """BASELINE configs[4]: small-N matvec on the attention-projection shapes, N in {1, 2, 4, 8, 16}. value = algorithmic
+    bytes (W + 4 N (cols + rows)) per second of the Q6_K 1536 x 7168 case at N = 8; every case is listed in config."""
+    import oracle as O
+    from macseek_amd import _lib, quant as q
+    L = _lib.load()
+    dev = torch.device("cuda:0")
+    cases = []
+    head = None
+    for t, name, rows, cols in ((q.QType.Q6_K, "Q6_K", 1536, 7168), (q.QType.Q5_K, "Q5_K", 512, 7168),
+                                (q.QType.IQ4_NL, "IQ4_NL", 7168, 4096), (q.QType.BF16, "BF16", 384, 7168)):
+        nb = q.row_bytes(t, cols) * rows
+        copies = 32  # successive launches read different copies of the matrix
+        if int(t) == 30:
+            arena = (torch.randn(copies * rows * cols, device=dev) * 0.02).to(torch.bfloat16).view(torch.uint8)
+        else:
+            arena = gen_blocks(torch, t, copies * nb // q.block_bytes(t), 0.01, 1, dev)
+        Ws = [q.Buffer.of(arena).sub(i * nb, nb).c() for i in range(copies)]
+        for n in (1, 2, 4, 8, 16):
+            x = torch.randn(n * cols, device=dev)
+            y = torch.zeros(n * rows, device=dev)
+            xb, yb = q.Buffer.of(x).c(), q.Buffer.of(y).c()
+
+            def launch(i):
+                rc = L.msq_matvec_n(C.c_void_p(torch.cuda.current_stream().cuda_stream), int(t), C.byref(Ws[i % copies]), rows, cols,
+                                    C.byref(xb), C.byref(yb), n, 0, 1)
+                if rc != 0:
+                    raise RuntimeError(L.msq_last_error().decode())
+            ms = graph_ms_per_launch(torch, launch, 200)
+            byt = nb + 4 * n * (cols + rows)
+            row = {"type": name, "rows": rows, "cols": cols, "n": n, "us_per_launch": ms * 1e3, "bytes": byt, "GBps": byt / (ms * 1e-3) / 1e9}
+            cases.append(row)
+            if name == "Q6_K" and n == 8:
+                head = row
+    cpu = None
+    if not args.gpu_only:
+        rows, cols, nt = 1536, 7168, 8
+        Wh = O.random_blocks(O.Q6_K, rows * cols, 1)
+        xh = O.randn(nt * cols, 2)
+        nth = cores()
+        t0 = time.perf_counter()
+        reps = 0
+        while time.perf_counter() - t0 < 5.0:
+            for i in range(nt):
+                O.matvec(O.Q6_K, Wh, rows, cols, xh[i * cols:(i + 1) * cols], 1, nth)
+            reps += 1
+        el = time.perf_counter() - t0
+        cpu = {"value": head["bytes"] * reps / el / 1e9, "unit": "GB/s", "cores": nth, "kind": "port",
+               "sample": "%d x 8 tokens of the Q6_K 1536x7168 case through oracle.c (dequant row + double dot per token), %.1f s" % (reps, el)}
+    return {"value": head["GBps"], "ms_per_step": head["us_per_launch"] * 1e-3, "dtype": "f16 activations (f32 for BF16 weights), f32 accumulate",
+            "config": {"workload": "BASELINE configs[4]: small-N matvec (speculative verify), attention projections, N in {1,2,4,8,16}; "
+                                   "one step = one msq_matvec_n launch of Q6_K 1536x7168 at N=8", "cases": cases},
+            "roofline": {"bound": "hbm", "achieved": head["GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": head["GBps"] / HBM_PEAK_GBPS,
+                         "traffic": None, "kernel": "mv_tok_kernel<DecQ6K, 1, 8>", "bytes_per_launch": head["bytes"],
+                         "avg_launch_us": head["us_per_launch"], "timing": "HIP event pair around one graph replay of 200 back-to-back launches"},
+            "cpu_baseline": cpu, "pct_of_hbm_peak": 100 * head["GBps"] / HBM_PEAK_GBPS}
 
 
 def bench_router(torch, args):
@@ -558,7 +619,7 @@ def main():
     ap.add_argument("--steps", type=int, default=500)
     ap.add_argument("--warmup", type=int, default=100)
     ap.add_argument("--workload", default="moe_decode",
-                    choices=["moe_decode", "moe_prefill", "matvec_iq1s", "matvec_iq2xxs", "q8_0", "router", "matmul", "stream", "copy_calibration"])
+                    choices=["moe_decode", "moe_prefill", "matvec_iq1s", "matvec_iq2xxs", "q8_0", "matvec_n", "router", "matmul", "stream", "copy_calibration"])
     ap.add_argument("--gpu-only", action="store_true",
                     help="profiling runs: skip the CPU baseline leg and the prefill appendix of the default workload")
     args = ap.parse_args()
@@ -598,6 +659,8 @@ def main():
         r = bench_copy_calibration(torch, args)
     elif args.workload == "router":
         r = bench_router(torch, args)
+    elif args.workload == "matvec_n":
+        r = bench_matvec_n(torch, args)
     elif args.workload == "matvec_iq1s":
         r = bench_matvec(torch, args, q.QType.IQ1_S, 4096, 7168, 0.01, "BASELINE configs[1]: single-expert decode matvec IQ1_S 4096x7168, batch 1")
     elif args.workload == "matvec_iq2xxs":
