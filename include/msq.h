@@ -271,6 +271,79 @@ typedef struct {
  * (their slot_of is not written). */
 int msq_route_lists(void* stream, const MsqBuffer* ids, const MsqBuffer* w, int n_tokens, int n_exp, const MsqRouteLists* L);
 
+/* ---- GGUF reader and resident expert placement: the on-disk format on the input side of the kernels ---- */
+
+/* reference: ms::Gguf (src/gguf/gguf.hpp:38-96, src/gguf/gguf.cpp). Opaque handle over one model: one file, or all M
+ * splits when the path matches "*-0000N-of-0000M.gguf". GGUF versions 2 and 3. Metadata is merged across splits (the
+ * first occurrence wins); tensors are listed in file order, split by split, with ABSOLUTE file offsets. Pure host
+ * code: nothing here touches the GPU except msq_gguf_load_tensor and msq_gguf_place_experts. */
+typedef struct MsqGguf MsqGguf;
+int msq_gguf_open(const char* path, MsqGguf** out);
+void msq_gguf_close(MsqGguf* g);
+int msq_gguf_n_splits(const MsqGguf* g);
+int msq_gguf_n_tensors(const MsqGguf* g);
+int msq_gguf_n_kv(const MsqGguf* g);
+uint32_t msq_gguf_alignment(const MsqGguf* g); /* general.alignment of the first split, 32 if absent */
+uint32_t msq_gguf_version(const MsqGguf* g);
+const char* msq_gguf_split_path(const MsqGguf* g, int split);
+uint64_t msq_gguf_data_offset(const MsqGguf* g, int split);
+int msq_gguf_split_count_of_path(const char* path); /* reference: Gguf::expand_splits(path).size() */
+
+/* reference: ms::type_bytes / ms::type_name (gguf.hpp:19-22): every ggml type id, also those the kernels do not take */
+uint64_t msq_gguf_type_bytes(int ggml_type, uint64_t n_elems);
+const char* msq_gguf_type_name(int ggml_type); /* "?" if unknown */
+
+/* reference: ms::TensorInfo (gguf.hpp:40-51); name stays valid until msq_gguf_close */
+typedef struct {
+  const char* name;
+  int type;      /* ggml type id */
+  int n_dims;
+  int64_t ne[4]; /* ggml order: ne[0] contiguous (= cols of a weight matrix), ne[1] = rows, ne[2] = experts */
+  uint64_t nbytes;
+  int split;
+  uint64_t offset; /* absolute byte offset of the data in that split file */
+} MsqGgufTensor;
+int msq_gguf_tensor(const MsqGguf* g, int index, MsqGgufTensor* out);
+int msq_gguf_find(const MsqGguf* g, const char* name); /* index, or -1 */
+
+/* metadata; value types as in the container: 0 u8, 1 i8, 2 u16, 3 i16, 4 u32, 5 i32, 6 f32, 7 bool, 8 string, 9 array,
+ * 10 u64, 11 i64, 12 f64. Getters return the default for a missing key or a mismatched kind (gguf.hpp:66-71). */
+const char* msq_gguf_key(const MsqGguf* g, int index); /* insertion order */
+int msq_gguf_kv_type(const MsqGguf* g, const char* key, int* arr_type); /* -1 if missing; *arr_type = element type or -1 */
+int64_t msq_gguf_get_i64(const MsqGguf* g, const char* key, int64_t dflt);
+double msq_gguf_get_f64(const MsqGguf* g, const char* key, double dflt);
+const char* msq_gguf_get_str(const MsqGguf* g, const char* key, const char* dflt);
+int64_t msq_gguf_arr_len(const MsqGguf* g, const char* key); /* -1 if missing or not an array */
+int64_t msq_gguf_arr_i64(const MsqGguf* g, const char* key, int64_t* out, int64_t cap); /* values written */
+int64_t msq_gguf_arr_f64(const MsqGguf* g, const char* key, double* out, int64_t cap);
+const char* msq_gguf_arr_str(const MsqGguf* g, const char* key, int64_t index);
+int64_t msq_gguf_arr_nested_i64(const MsqGguf* g, const char* key, int64_t index, int64_t* out, int64_t cap); /* inner length */
+
+/* reference: ms::pread_full on the tensor's split (gguf.hpp:99): bytes [byte_off, byte_off + len) of the tensor's data
+ * into host memory; returns the bytes read, -1 on a bad range. */
+int64_t msq_gguf_read(const MsqGguf* g, int tensor, uint64_t byte_off, void* dst, uint64_t len);
+/* The same range into device memory (pinned staging, copies enqueued on `stream`; returns after the last chunk has been
+ * read from the file and copied). */
+int msq_gguf_load_tensor(void* stream, const MsqGguf* g, int tensor, uint64_t byte_off, uint64_t len, const MsqBuffer* dst);
+
+/* reference: ms::ExpertLayout::from_gguf for one layer (src/store/experts.hpp:35-42, src/store/experts.mm:36-56):
+ * index k = 0 gate (blk.L.ffn_gate_exps.weight), 1 up, 2 down; stride = nbytes / n_experts, the per-expert slab. */
+typedef struct {
+  int n_experts;
+  int type[3];         /* ggml type of the gate / up / down matrices */
+  int64_t rows[3], cols[3];
+  uint64_t stride[3];  /* bytes of one expert's matrix */
+  int tensor[3];       /* tensor indices */
+  uint64_t arena_bytes; /* device bytes msq_gguf_place_experts needs: every slab padded to 256 bytes */
+} MsqExpertLayout;
+int msq_gguf_expert_layout(const MsqGguf* g, int layer, MsqExpertLayout* out);
+
+/* Resident placement of one layer's experts (no reference counterpart: the reference streams experts from SSD into a
+ * cache arena, src/store/experts.hpp:60-250; an MI355X keeps them all in HBM). Copies the three stacked tensors into
+ * `arena` (device memory, 256-byte aligned, >= arena_bytes), every expert matrix at a 256-byte aligned offset, and
+ * fills slots[e] (e < n_experts <= n_slots) with views of it for msq_moe_decode / msq_moe_prefill. */
+int msq_gguf_place_experts(void* stream, const MsqGguf* g, int layer, const MsqBuffer* arena, MsqExpertSlot* slots, int n_slots);
+
 #ifdef __cplusplus
 }
 #endif

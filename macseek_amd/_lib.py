@@ -43,6 +43,16 @@ class MsqRouteLists(C.Structure):
                 ("w", MsqBuffer), ("slot_of", MsqBuffer), ("max_tokens", C.c_int)]
 
 
+class MsqGgufTensor(C.Structure):
+    _fields_ = [("name", C.c_char_p), ("type", C.c_int), ("n_dims", C.c_int), ("ne", C.c_int64 * 4), ("nbytes", C.c_uint64),
+                ("split", C.c_int), ("offset", C.c_uint64)]
+
+
+class MsqExpertLayout(C.Structure):
+    _fields_ = [("n_experts", C.c_int), ("type", C.c_int * 3), ("rows", C.c_int64 * 3), ("cols", C.c_int64 * 3),
+                ("stride", C.c_uint64 * 3), ("tensor", C.c_int * 3), ("arena_bytes", C.c_uint64)]
+
+
 _lib = None
 
 # name -> (restype, argtypes); every symbol include/msq.h declares
@@ -75,6 +85,34 @@ SIGNATURES = {
     "msq_router_topk": (C.c_int, [C.c_void_p, _BP, _BP, _BP, _BP, C.c_int, C.c_int, C.c_float]),
     "msq_router_scratch_bytes": (C.c_size_t, [C.c_int]),
     "msq_router_fused": (C.c_int, [C.c_void_p, C.c_int, _BP, _BP, _BP, _BP, _BP, _BP, C.c_int, C.c_int, C.c_float]),
+    "msq_gguf_open": (C.c_int, [C.c_char_p, C.POINTER(C.c_void_p)]),
+    "msq_gguf_close": (None, [C.c_void_p]),
+    "msq_gguf_n_splits": (C.c_int, [C.c_void_p]),
+    "msq_gguf_n_tensors": (C.c_int, [C.c_void_p]),
+    "msq_gguf_n_kv": (C.c_int, [C.c_void_p]),
+    "msq_gguf_alignment": (C.c_uint32, [C.c_void_p]),
+    "msq_gguf_version": (C.c_uint32, [C.c_void_p]),
+    "msq_gguf_split_path": (C.c_char_p, [C.c_void_p, C.c_int]),
+    "msq_gguf_data_offset": (C.c_uint64, [C.c_void_p, C.c_int]),
+    "msq_gguf_split_count_of_path": (C.c_int, [C.c_char_p]),
+    "msq_gguf_type_bytes": (C.c_uint64, [C.c_int, C.c_uint64]),
+    "msq_gguf_type_name": (C.c_char_p, [C.c_int]),
+    "msq_gguf_tensor": (C.c_int, [C.c_void_p, C.c_int, C.POINTER(MsqGgufTensor)]),
+    "msq_gguf_find": (C.c_int, [C.c_void_p, C.c_char_p]),
+    "msq_gguf_key": (C.c_char_p, [C.c_void_p, C.c_int]),
+    "msq_gguf_kv_type": (C.c_int, [C.c_void_p, C.c_char_p, C.POINTER(C.c_int)]),
+    "msq_gguf_get_i64": (C.c_int64, [C.c_void_p, C.c_char_p, C.c_int64]),
+    "msq_gguf_get_f64": (C.c_double, [C.c_void_p, C.c_char_p, C.c_double]),
+    "msq_gguf_get_str": (C.c_char_p, [C.c_void_p, C.c_char_p, C.c_char_p]),
+    "msq_gguf_arr_len": (C.c_int64, [C.c_void_p, C.c_char_p]),
+    "msq_gguf_arr_i64": (C.c_int64, [C.c_void_p, C.c_char_p, C.c_void_p, C.c_int64]),
+    "msq_gguf_arr_f64": (C.c_int64, [C.c_void_p, C.c_char_p, C.c_void_p, C.c_int64]),
+    "msq_gguf_arr_str": (C.c_char_p, [C.c_void_p, C.c_char_p, C.c_int64]),
+    "msq_gguf_arr_nested_i64": (C.c_int64, [C.c_void_p, C.c_char_p, C.c_int64, C.c_void_p, C.c_int64]),
+    "msq_gguf_read": (C.c_int64, [C.c_void_p, C.c_int, C.c_uint64, C.c_void_p, C.c_uint64]),
+    "msq_gguf_load_tensor": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.c_uint64, C.c_uint64, _BP]),
+    "msq_gguf_expert_layout": (C.c_int, [C.c_void_p, C.c_int, C.POINTER(MsqExpertLayout)]),
+    "msq_gguf_place_experts": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, _BP, C.POINTER(MsqExpertSlot), C.c_int]),
     "msq_route_lists": (C.c_int, [C.c_void_p, _BP, _BP, C.c_int, C.c_int, C.POINTER(MsqRouteLists)]),
 }
 

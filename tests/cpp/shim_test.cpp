@@ -11,6 +11,7 @@
 #include <vector>
 
 #include "macseek_amd/arch.hpp"
+#include "macseek_amd/gguf.hpp"
 #include "macseek_amd/quant.hpp"
 
 #define HIP_OK(e) do { hipError_t r_ = (e); if (r_ != hipSuccess) { fprintf(stderr, "HIP: %s\n", hipGetErrorString(r_)); return 2; } } while (0)
@@ -84,6 +85,36 @@ int main() {
     for (int i = 0; i < 12; i++) f3 += ent[slot[i]] != (uint32_t)i;
     printf("  ms::arch router_topk + route_lists %s\n", f3 ? "FAIL" : "ok");
     fails += f3;
+  }
+  {  // ms::Gguf shim: a two-tensor file written here (GGUF v3, default alignment 32)
+    std::vector<uint8_t> f;
+    auto put = [&](const void* p, size_t n) { f.insert(f.end(), (const uint8_t*)p, (const uint8_t*)p + n); };
+    auto u32 = [&](uint32_t v) { put(&v, 4); };
+    auto u64 = [&](uint64_t v) { put(&v, 8); };
+    auto str = [&](const char* s) { u64(strlen(s)); put(s, strlen(s)); };
+    u32(0x46554747u); u32(3); u64(1); u64(2);
+    str("general.architecture"); u32(8); str("deepseek41");
+    str("deepseek41.expert_count"); u32(4); u32(384);
+    str("w"); u32(2); u64(32); u64(2); u32(8); u64(0);  // Q8_0 [32, 2]
+    while (f.size() % 32) f.push_back(0);
+    const size_t data_off = f.size();
+    for (int i = 0; i < 68; i++) f.push_back((uint8_t)(i * 3 + 1));
+    const char* path = "/tmp/msq_shim_test.gguf";
+    FILE* fp = fopen(path, "wb");
+    int f4 = fp == nullptr;
+    if (fp) { f4 += fwrite(f.data(), 1, f.size(), fp) != f.size(); fclose(fp); }
+    if (!f4) {
+      ms::Gguf g(path);
+      const ms::TensorInfo t = g.at("w");
+      uint8_t back[68];
+      f4 += g.get_str("general.architecture") != "deepseek41" || g.get_i64("deepseek41.expert_count") != 384;
+      f4 += t.type != 8 || t.ne[0] != 32 || t.ne[1] != 2 || t.nbytes != 68 || t.offset != data_off || t.row_bytes() != 34;
+      f4 += g.read(t, back, 68) != 68 || memcmp(back, f.data() + data_off, 68) != 0;
+      f4 += g.tensors().size() != 1 || g.alignment() != 32;
+    }
+    remove(path);
+    printf("  ms::Gguf parse + read %s\n", f4 ? "FAIL" : "ok");
+    fails += f4;
   }
   // misuse aborts like the reference (src/kernels/quant.mm:34-37): cols not a multiple of the block size
   fflush(stdout);
