@@ -226,22 +226,7 @@ __device__ __forceinline__ void copy_words16(uint32_t* dst, const uint32_t* src,
   for (int i = tid; i < nwords / 4; i += nthreads) d[i] = s[i];
 }
 
-// ------------------------------------------------------------------------------------------------ slice streaming
-// A wave streams the bytes of its K slice of a row (SLICE_BYTES, a whole number of blocks, only 2-byte aligned) with
-// one fully coalesced 128-bit load: lane l fetches the 16-byte granule l of the 16-byte-aligned window that contains
-// the slice. The window goes to a per-wave LDS staging area, from which every lane picks the few bytes of its own
-// unit; `shift` (slice start within its first granule) is wave-uniform.
-constexpr int kStageBytes = 576;  // per staged slice: up to 528 slice bytes + 15 shift, rounded to 64
 typedef uint32_t __attribute__((ext_vector_type(4))) u32x4;
-__device__ __forceinline__ uint4 slice_load(gptr_t start, uint32_t nbytes, uint32_t lane) {
-  const uint32_t shift = (uint32_t)((uintptr_t)start & 15u);
-  u32x4 v = {0u, 0u, 0u, 0u};
-  if (16u * lane < shift + nbytes) v = *(const MSQ_GLOBAL u32x4*)(start - shift + 16u * lane);
-  return {v.x, v.y, v.z, v.w};
-}
-__device__ __forceinline__ void slice_stage(uint8_t* stage, const uint4& v, uint32_t lane) {
-  if (lane < kStageBytes / 16) ((uint4*)stage)[lane] = v;
-}
 
 // ------------------------------------------------------------------------------------------------ x slices
 // 32 consecutive activations -> 16 fp16 pairs (round to nearest even) + the sum of the rounded values
@@ -280,7 +265,6 @@ __device__ __forceinline__ float sum_h2(const uint32_t* v, int n) {
 // ---- IQ1_S: {fp16 d; u8 qs[32]; u16 qh[8]}, 50 bytes / 256 weights; unit = one 32-weight sub-block
 struct DecIQ1S {
   static constexpr int UNIT = 32, LDS_WORDS = MSQ_IQ1S_GRID_N * 4;
-  static constexpr int SLICE_BYTES = 8 * 50;  // bytes of the 64 units (8 blocks) one wave covers per row
   typedef X32 X;
   struct Raw { uint32_t qs, qh, d; };
   __device__ static void fill_lds(uint32_t* lds, int tid, int nt) { copy_words16(lds, g_tbl_iq1s.w, LDS_WORDS, tid, nt); }
@@ -359,7 +343,6 @@ struct DecIQ1S {
 // ---- IQ2_XXS: {fp16 d; u16 qs[32]}, 66 bytes / 256 weights; unit = one 32-weight sub-block (8 bytes)
 struct DecIQ2XXS {
   static constexpr int UNIT = 32, LDS_WORDS = MSQ_IQ2XXS_GRID_N * 4 + 128 * 4;
-  static constexpr int SLICE_BYTES = 8 * 66;
   typedef X32 X;
   struct Raw { uint32_t a0, a1, d; };
   __device__ static void fill_lds(uint32_t* lds, int tid, int nt) {
@@ -439,7 +422,7 @@ struct DecIQ2XXS {
 
 // ---- Q8_0: {fp16 d; int8 qs[32]}, 34 bytes / 32 weights; unit = one block, activations kept in fp32
 struct DecQ8_0 {
-  static constexpr int UNIT = 32, LDS_WORDS = 0, SLICE_BYTES = 0;
+  static constexpr int UNIT = 32, LDS_WORDS = 0;
   struct X { float v[32]; };
   struct Raw { uint32_t q[8]; uint32_t d; };
   __device__ static void fill_lds(uint32_t*, int, int) {}
@@ -472,7 +455,7 @@ struct DecQ8_0 {
 
 // ---- IQ4_NL: {fp16 d; u8 qs[16]}, 18 bytes / 32 weights; byte j holds columns j (low nibble) and j + 16 (high)
 struct DecIQ4NL {
-  static constexpr int UNIT = 32, LDS_WORDS = 256, SLICE_BYTES = 0;
+  static constexpr int UNIT = 32, LDS_WORDS = 256;
   struct X { uint32_t v[16]; };  // pair j = (x[j], x[j + 16])
   struct Raw { uint32_t q[4]; uint32_t d; };
   __device__ static void fill_lds(uint32_t* lds, int tid, int nt) { copy_words16(lds, g_tbl_iq4nl.w, 256, tid, nt); }
@@ -508,7 +491,7 @@ struct DecIQ4NL {
 // Unit j of a block (8 per block): half h = j >> 2, l0 = 8 * (j & 3); it owns the four 8-column runs
 // 128 h + 32 k + l0 .. + 7 (k = 0..3), which share the bytes ql[64 h + l0 ..], ql[64 h + 32 + l0 ..], qh[32 h + l0 ..].
 struct DecQ6K {
-  static constexpr int UNIT = 32, LDS_WORDS = 0, SLICE_BYTES = 0;
+  static constexpr int UNIT = 32, LDS_WORDS = 0;
   struct X { uint32_t v[16]; float sx[4]; };
   struct Raw { uint32_t qa[2], qb[2], qh[2], sc[2], d; };
   __device__ static void fill_lds(uint32_t*, int, int) {}
@@ -559,7 +542,7 @@ struct DecQ6K {
 // Unit j of a block: 64-column group g = j >> 1, l0 = 16 * (j & 1); it owns columns 64 g + l0 .. + 15 (low nibbles,
 // scale index 2 g) and 64 g + 32 + l0 .. + 15 (high nibbles, scale index 2 g + 1).
 struct DecQ5K {
-  static constexpr int UNIT = 32, LDS_WORDS = 0, SLICE_BYTES = 0;
+  static constexpr int UNIT = 32, LDS_WORDS = 0;
   struct X { uint32_t v[16]; float sx[2]; };
   struct Raw { uint32_t ql[4], qh[4], pa, pb, pc, dd; };
   __device__ static void fill_lds(uint32_t*, int, int) {}
@@ -610,7 +593,7 @@ struct DecQ5K {
 // ---- dense rows (F32 / F16 / BF16): unit = 8 consecutive elements, fp32 activations
 template <int QT>
 struct DecDense {
-  static constexpr int UNIT = 8, LDS_WORDS = 0, SLICE_BYTES = 0;
+  static constexpr int UNIT = 8, LDS_WORDS = 0;
   struct X { float v[8]; };
   struct Raw { uint32_t w[QT == MSQ_F32 ? 8 : 4]; };
   __device__ static void fill_lds(uint32_t*, int, int) {}

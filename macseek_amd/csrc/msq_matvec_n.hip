@@ -11,7 +11,6 @@ template <class F>
 int launch_mvn(hipStream_t st, MvnArgs a) {
   const int cus = device_info().cus;
   a.nsteps = a.cols / 32u;
-  a.col0 = 0; a.col0_bytes = 0;
   const uint32_t ks = std::min<uint32_t>(16u, a.nsteps);
   a.steps_per_wave = (a.nsteps + ks - 1) / ks;
   const uint32_t waves = (a.nsteps + a.steps_per_wave - 1) / a.steps_per_wave;
@@ -73,7 +72,6 @@ extern "C" int msq_matvec_n(void* stream, int t, const MsqBuffer* W, int rows, i
   a.x_stride = (uint32_t)xs; a.y_stride = (uint32_t)rows;
   a.rows_per_group = (uint32_t)rpg; a.x_group_stride = (uint32_t)cols; a.accumulate = accumulate ? 1u : 0u;
   a.ntiles = (uint32_t)((rows + 15) / 16);
-  a.qtype = t;
   hipStream_t st = (hipStream_t)stream;
   switch (t) {
     case MSQ_IQ1_S: return launch_mvn<FragIQ1S>(st, a);

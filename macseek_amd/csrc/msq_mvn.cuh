@@ -5,7 +5,9 @@
 // One weight read serves all n tokens through the matrix cores: a 16-row tile of W is the B operand, the (up to 16)
 // tokens are the A operand. A workgroup is KS waves that split K; a wave takes its K steps eight at a time: the weight
 // fragments of all eight are requested before the first MFMA, the activations are MFMA A fragments in registers (kept
-// for the whole launch when a wave has at most eight steps); the workgroups walk the row tiles (persistent grid). Per tile the KS partial 16 x 16 results meet in LDS and are added in a fixed order.
+// for the whole launch when a wave has at most eight steps); the workgroups walk the row tiles (persistent grid). Per
+// tile the KS partial 16 x 16 results meet in LDS and are added in a fixed order. msq_matvec_n uses this kernel for
+// rows too wide for the dot-product kernel (mv_tok_kernel) and for many tokens over large matrices.
 #pragma once
 #include "msq_mfma.cuh"
 
@@ -19,15 +21,10 @@ struct MvnArgs {
   uint32_t x_stride, y_stride;   // elements between activation / output rows of consecutive tokens
   uint32_t rows_per_group, x_group_stride;
   uint32_t accumulate;
-  uint32_t col0, col0_bytes;     // first column this launch covers and its byte offset in a row (K chunking)
-  uint32_t nsteps;               // K steps this launch covers
+  uint32_t nsteps;               // K steps of 32 columns
   uint32_t steps_per_wave;
   uint32_t ntiles;               // ceil(rows / 16)
-  int qtype;
 };
-
-// byte offset of column `col` (a multiple of 256) inside a row
-inline size_t msq_type_row_bytes_of_cols(const MvnArgs& a, uint32_t col) { return msq_type_row_bytes(a.qtype, col); }
 
 template <class F>
 __global__ __launch_bounds__(1024) void mvn_kernel(const MvnArgs a) {
@@ -57,7 +54,7 @@ __global__ __launch_bounds__(1024) void mvn_kernel(const MvnArgs a) {
 #pragma unroll
     for (int i = 0; i < MS; i++) {
       const uint32_t step = min(s0 + c0 + i, a.nsteps - 1);
-      const float* xs = a.X + (size_t)min(m16, a.n - 1) * a.x_stride + (size_t)group * a.x_group_stride + a.col0 + 32u * step;
+      const float* xs = a.X + (size_t)min(m16, a.n - 1) * a.x_stride + (size_t)group * a.x_group_stride + 32u * step;
       // the chunk's 8 columns as two 128-bit loads (col_of is 8 q + p, or for IQ4_NL 4 q + p / 2 + 16 (p % 2))
       const bool natural = F::col_of(1, 1) == 9u;
       raw[i][0] = *(const float4*)(xs + (natural ? 8u * q : 4u * q));
@@ -93,7 +90,7 @@ __global__ __launch_bounds__(1024) void mvn_kernel(const MvnArgs a) {
   for (uint32_t tile = blockIdx.x; tile < a.ntiles; tile += gridDim.x) {
     const uint32_t group = (tile * 16u) / a.rows_per_group;  // a tile never straddles two groups (host guarantees)
     const uint32_t row = min(tile * 16u + m16, a.rows - 1);
-    const gptr_t wr = as_global(a.W) + (size_t)row * a.row_bytes + a.col0_bytes;
+    const gptr_t wr = as_global(a.W) + (size_t)row * a.row_bytes;
     f4_t acc = {0.f, 0.f, 0.f, 0.f};
     for (uint32_t c0 = 0; c0 < S; c0 += MS) {
       // all of the sub-chunk's weight fragments are requested (and decoded as they arrive) before the first MFMA:

@@ -81,9 +81,7 @@ int launch_block(int t, hipStream_t st, const PfBlkArgs& a, uint32_t n6, uint32_
 
 template <bool GU>
 int launch_gemm(int t, hipStream_t st, const PfArgs& a, int cus) {
-  switch (t) {
-    case MSQ_IQ1_S: return launch_gemm_t<FragIQ1S, GU>(st, a, cus);
-    case MSQ_IQ2_XXS: return launch_gemm_t<FragIQ2XXS, GU>(st, a, cus);
+  switch (t) {  // the codebook formats never come here (block_path)
     case MSQ_Q6_K: return launch_gemm_t<FragQ6K, GU>(st, a, cus);
     case MSQ_Q8_0: return launch_gemm_t<FragQ8_0, GU>(st, a, cus);
   }
