@@ -228,12 +228,96 @@ __device__ __forceinline__ void copy_words16(uint32_t* dst, const uint32_t* src,
 
 typedef uint32_t __attribute__((ext_vector_type(4))) u32x4;
 
+// One piece of a workgroup's prologue copy into LDS: n16 16-byte items from device memory to the LDS word offset dst;
+// padded: the items are activations and go to the padded rows of XLds (below).
+struct CopyJob {
+  const uint4* src;
+  uint32_t dst, n16;
+  bool padded;
+};
+// All pieces as one pass over their concatenation, K items per thread in flight: every load of a batch is requested
+// before the first LDS store waits for one (piece by piece, each copy would cost its own round trip to memory).
+// Indices past the end repeat the last item (no branch around a load); only the stores are conditional.
+template <int K, int NJ>
+__device__ __forceinline__ void copy_jobs(uint32_t* smem, const CopyJob (&jobs)[NJ], uint32_t tid, uint32_t nt) {
+  uint32_t total = 0;
+#pragma unroll
+  for (int j = 0; j < NJ; j++) total += jobs[j].n16;
+  if (total == 0) return;
+  for (uint32_t base = tid; base < total; base += K * nt) {
+    uint4 v[K];
+    uint32_t dw[K];
+#pragma unroll
+    for (int k = 0; k < K; k++) {
+      const uint32_t i = min(base + k * nt, total - 1u);
+      // the piece item i falls in: the last one that starts at or before i (pieces of no items are passed over)
+      const uint4* src = jobs[0].src;
+      uint32_t dst = jobs[0].dst, pad = jobs[0].padded ? 4u : 0u, loc = i, first = 0;
+#pragma unroll
+      for (int j = 1; j < NJ; j++) {
+        first += jobs[j - 1].n16;
+        if (i >= first) { src = jobs[j].src; dst = jobs[j].dst; pad = jobs[j].padded ? 4u : 0u; loc = i - first; }
+      }
+      v[k] = src[loc];
+      dw[k] = dst + 4u * loc + (loc >> 3) * pad;
+    }
+#pragma unroll
+    for (int k = 0; k < K; k++)
+      if (base + k * nt < total) *(uint4*)(smem + dw[k]) = v[k];
+  }
+}
+
+// table piece k of decoder D for copy_jobs (an empty piece when D stages no such table or is not in use)
+template <class D>
+__device__ __forceinline__ CopyJob tbl_job_of(int k, uint32_t at, bool live) {
+  if constexpr (requires { D::NTBL; }) {
+    if (live && k < D::NTBL) return D::tbl_job(k, at);
+  }
+  return {nullptr, 0u, 0u, false};
+}
+
 // ------------------------------------------------------------------------------------------------ x slices
 // 32 consecutive activations -> 16 fp16 pairs (round to nearest even) + the sum of the rounded values
 struct X32 {
   uint32_t v[16];
   float sx;
 };
+// Where load_x() finds the activations: plain memory (const float*), or a workgroup's LDS copy (XLds) in which every
+// 32-float slice is followed by four floats of padding. A lane's slice of a row is 32 (or 8, or 16) consecutive
+// floats, so read straight from device memory each 128-bit load of a wave touches 64 different cache lines; staged with
+// contiguous loads and read back from the padded LDS rows (36 words apart: 16 consecutive lanes hit 16 different bank
+// quads) the same data costs one pass over the row per workgroup. Runs handed to one vector load never cross a slice.
+struct XLds { const float* p; };
+__device__ __forceinline__ const float* xat(const float* x, uint32_t col) { return x + col; }
+__device__ __forceinline__ const float* xat(XLds x, uint32_t col) { return x.p + col + (col >> 5) * 4u; }
+__host__ __device__ constexpr uint32_t xlds_words(uint32_t cols) { return cols + (cols >> 5) * 4u; }
+// Cooperative copy of the first G (<= GMAX, workgroup-uniform) activation rows src[g] of n floats each (multiple of
+// 4) into consecutive padded LDS rows of roww words. Every thread has up to K 128-bit loads per row in flight, all
+// rows requested before the first store waits. Indices past the end of a row repeat its last item (no branch around
+// load); only the stores are conditional, so all GMAX pointers must be readable.
+template <int GMAX, int K = 4>
+__device__ __forceinline__ void stage_x_rows(float* dst, const float* const (&src)[GMAX], uint32_t G, uint32_t roww, uint32_t n,
+                                             uint32_t tid, uint32_t nt) {
+  const uint32_t n4 = n >> 2;
+  for (uint32_t base = tid; base < n4; base += K * nt) {
+    float4 v[GMAX][K];
+#pragma unroll
+    for (int g = 0; g < GMAX; g++) {  // every src[g] is readable (rows past G are loaded and dropped)
+#pragma unroll
+      for (int k = 0; k < K; k++) v[g][k] = ((const float4*)src[g])[min(base + k * nt, n4 - 1u)];
+    }
+#pragma unroll
+    for (int g = 0; g < GMAX; g++) {
+      if (g < (int)G) {
+#pragma unroll
+        for (int k = 0; k < K; k++) {
+          const uint32_t i = base + k * nt;
+          if (i < n4) *(float4*)(dst + g * roww + 4u * i + (i >> 3) * 4u) = v[g][k];
+        }
+      }
+    }
+  }
+}
 __device__ __forceinline__ void load_x32_consecutive(const float* x, uint32_t* v, int n) {
   const float4* p = (const float4*)x;
 #pragma unroll
@@ -258,6 +342,9 @@ __device__ __forceinline__ float sum_h2(const uint32_t* v, int n) {
 //   UNIT            columns one lane owns per unit
 //   LDS_WORDS       32-bit words of table the workgroup stages in LDS (0 = none)
 //   fill_lds()      cooperative table copy
+//   STAGE_X         a lane's slice is one run of 128 bytes: read straight from device memory every 128-bit load of a
+//                   wave touches 64 cache lines, so the workgroup stages the row in LDS with contiguous loads instead
+//                   (decoders whose slices are runs of 32 or 64 bytes read them directly: 16 or 32 lines per load)
 //   X / load_x()    the lane's activation slice for unit u of a row (x points at the row's first activation)
 //   Raw / load()    the raw block bytes of unit u of a weight row (global loads only, so callers can prefetch)
 //   dot()           sum over the unit's columns of weight * activation, fp32
@@ -265,12 +352,16 @@ __device__ __forceinline__ float sum_h2(const uint32_t* v, int n) {
 // ---- IQ1_S: {fp16 d; u8 qs[32]; u16 qh[8]}, 50 bytes / 256 weights; unit = one 32-weight sub-block
 struct DecIQ1S {
   static constexpr int UNIT = 32, LDS_WORDS = MSQ_IQ1S_GRID_N * 4;
+  static constexpr bool STAGE_X = true;
   typedef X32 X;
   struct Raw { uint32_t qs, qh, d; };
   __device__ static void fill_lds(uint32_t* lds, int tid, int nt) { copy_words16(lds, g_tbl_iq1s.w, LDS_WORDS, tid, nt); }
-  __device__ static X load_x(const float* x, uint32_t u) {
+  static constexpr int NTBL = 1;
+  __device__ static CopyJob tbl_job(int, uint32_t at) { return {(const uint4*)g_tbl_iq1s.w, at, LDS_WORDS / 4, false}; }
+  template <class S>
+  __device__ static X load_x(S x, uint32_t u) {
     X r;
-    load_x32_consecutive(x + 32u * u, r.v, 32);
+    load_x32_consecutive(xat(x, 32u * u), r.v, 32);
     r.sx = sum_h2(r.v, 16);
     return r;
   }
@@ -343,15 +434,22 @@ struct DecIQ1S {
 // ---- IQ2_XXS: {fp16 d; u16 qs[32]}, 66 bytes / 256 weights; unit = one 32-weight sub-block (8 bytes)
 struct DecIQ2XXS {
   static constexpr int UNIT = 32, LDS_WORDS = MSQ_IQ2XXS_GRID_N * 4 + 128 * 4;
+  static constexpr bool STAGE_X = true;
   typedef X32 X;
   struct Raw { uint32_t a0, a1, d; };
   __device__ static void fill_lds(uint32_t* lds, int tid, int nt) {
     copy_words16(lds, g_tbl_iq2xxs.w, MSQ_IQ2XXS_GRID_N * 4, tid, nt);
     copy_words16(lds + MSQ_IQ2XXS_GRID_N * 4, g_tbl_sign.w, 128 * 4, tid, nt);
   }
-  __device__ static X load_x(const float* x, uint32_t u) {
+  static constexpr int NTBL = 2;
+  __device__ static CopyJob tbl_job(int k, uint32_t at) {
+    if (k == 0) return {(const uint4*)g_tbl_iq2xxs.w, at, MSQ_IQ2XXS_GRID_N, false};
+    return {(const uint4*)g_tbl_sign.w, at + MSQ_IQ2XXS_GRID_N * 4, 128, false};
+  }
+  template <class S>
+  __device__ static X load_x(S x, uint32_t u) {
     X r;
-    load_x32_consecutive(x + 32u * u, r.v, 32);
+    load_x32_consecutive(xat(x, 32u * u), r.v, 32);
     r.sx = 0.f;
     return r;
   }
@@ -423,12 +521,14 @@ struct DecIQ2XXS {
 // ---- Q8_0: {fp16 d; int8 qs[32]}, 34 bytes / 32 weights; unit = one block, activations kept in fp32
 struct DecQ8_0 {
   static constexpr int UNIT = 32, LDS_WORDS = 0;
+  static constexpr bool STAGE_X = true;
   struct X { float v[32]; };
   struct Raw { uint32_t q[8]; uint32_t d; };
   __device__ static void fill_lds(uint32_t*, int, int) {}
-  __device__ static X load_x(const float* x, uint32_t u) {
+  template <class S>
+  __device__ static X load_x(S x, uint32_t u) {
     X r;
-    const float4* p = (const float4*)(x + 32u * u);
+    const float4* p = (const float4*)xat(x, 32u * u);
 #pragma unroll
     for (int i = 0; i < 8; i++) { const float4 f = p[i]; r.v[4 * i] = f.x; r.v[4 * i + 1] = f.y; r.v[4 * i + 2] = f.z; r.v[4 * i + 3] = f.w; }
     return r;
@@ -456,12 +556,14 @@ struct DecQ8_0 {
 // ---- IQ4_NL: {fp16 d; u8 qs[16]}, 18 bytes / 32 weights; byte j holds columns j (low nibble) and j + 16 (high)
 struct DecIQ4NL {
   static constexpr int UNIT = 32, LDS_WORDS = 256;
+  static constexpr bool STAGE_X = true;
   struct X { uint32_t v[16]; };  // pair j = (x[j], x[j + 16])
   struct Raw { uint32_t q[4]; uint32_t d; };
   __device__ static void fill_lds(uint32_t* lds, int tid, int nt) { copy_words16(lds, g_tbl_iq4nl.w, 256, tid, nt); }
-  __device__ static X load_x(const float* x, uint32_t u) {
+  template <class S>
+  __device__ static X load_x(S x, uint32_t u) {
     X r;
-    const float4* p = (const float4*)(x + 32u * u);
+    const float4* p = (const float4*)xat(x, 32u * u);
 #pragma unroll
     for (int i = 0; i < 4; i++) {
       const float4 a = p[i], b = p[i + 4];
@@ -492,16 +594,18 @@ struct DecIQ4NL {
 // 128 h + 32 k + l0 .. + 7 (k = 0..3), which share the bytes ql[64 h + l0 ..], ql[64 h + 32 + l0 ..], qh[32 h + l0 ..].
 struct DecQ6K {
   static constexpr int UNIT = 32, LDS_WORDS = 0;
+  static constexpr bool STAGE_X = false;
   struct X { uint32_t v[16]; float sx[4]; };
   struct Raw { uint32_t qa[2], qb[2], qh[2], sc[2], d; };
   __device__ static void fill_lds(uint32_t*, int, int) {}
-  __device__ static X load_x(const float* x, uint32_t u) {
+  template <class S>
+  __device__ static X load_x(S x, uint32_t u) {
     X r;
     const uint32_t j = u & 7u;
-    const float* base = x + 256u * (u >> 3) + 128u * (j >> 2) + 8u * (j & 3u);
+    const uint32_t base = 256u * (u >> 3) + 128u * (j >> 2) + 8u * (j & 3u);
 #pragma unroll
     for (int k = 0; k < 4; k++) {
-      load_x32_consecutive(base + 32 * k, r.v + 4 * k, 8);
+      load_x32_consecutive(xat(x, base + 32u * k), r.v + 4 * k, 8);
       r.sx[k] = sum_h2(r.v + 4 * k, 4);
     }
     return r;
@@ -543,15 +647,17 @@ struct DecQ6K {
 // scale index 2 g) and 64 g + 32 + l0 .. + 15 (high nibbles, scale index 2 g + 1).
 struct DecQ5K {
   static constexpr int UNIT = 32, LDS_WORDS = 0;
+  static constexpr bool STAGE_X = false;
   struct X { uint32_t v[16]; float sx[2]; };
   struct Raw { uint32_t ql[4], qh[4], pa, pb, pc, dd; };
   __device__ static void fill_lds(uint32_t*, int, int) {}
-  __device__ static X load_x(const float* x, uint32_t u) {
+  template <class S>
+  __device__ static X load_x(S x, uint32_t u) {
     X r;
     const uint32_t j = u & 7u;
-    const float* base = x + 256u * (u >> 3) + 64u * (j >> 1) + 16u * (j & 1u);
-    load_x32_consecutive(base, r.v, 16);
-    load_x32_consecutive(base + 32, r.v + 8, 16);
+    const uint32_t base = 256u * (u >> 3) + 64u * (j >> 1) + 16u * (j & 1u);
+    load_x32_consecutive(xat(x, base), r.v, 16);
+    load_x32_consecutive(xat(x, base + 32u), r.v + 8, 16);
     r.sx[0] = sum_h2(r.v, 8);
     r.sx[1] = sum_h2(r.v + 8, 8);
     return r;
@@ -594,12 +700,15 @@ struct DecQ5K {
 template <int QT>
 struct DecDense {
   static constexpr int UNIT = 8, LDS_WORDS = 0;
+  static constexpr bool STAGE_X = false;
   struct X { float v[8]; };
   struct Raw { uint32_t w[QT == MSQ_F32 ? 8 : 4]; };
   __device__ static void fill_lds(uint32_t*, int, int) {}
-  __device__ static X load_x(const float* x, uint32_t u) {
+  template <class S>
+  __device__ static X load_x(S x, uint32_t u) {
     X r;
-    const float4 a = ((const float4*)(x + 8u * u))[0], b = ((const float4*)(x + 8u * u))[1];
+    const float4* p = (const float4*)xat(x, 8u * u);
+    const float4 a = p[0], b = p[1];
     r.v[0] = a.x; r.v[1] = a.y; r.v[2] = a.z; r.v[3] = a.w; r.v[4] = b.x; r.v[5] = b.y; r.v[6] = b.z; r.v[7] = b.w;
     return r;
   }

@@ -32,6 +32,16 @@ inline int hip_fail(hipError_t e, const char* where) {
     if (e_ != hipSuccess) return ::msq::hip_fail(e_, #expr); \
   } while (0)
 
+// LDS of one CU; a kernel that takes more than 64 KB of it as dynamic LDS has to be told so once
+constexpr int kMaxLds = 160 * 1024;
+template <class K>
+void allow_large_lds(K kernel, size_t lds) {
+  static bool done = false;  // per instantiation; idempotent, so a race between first callers is harmless
+  if (lds > 64 * 1024 && !done) {
+    hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, kMaxLds);
+    done = true;
+  }
+}
 inline const uint8_t* bptr(const MsqBuffer* b) { return (const uint8_t*)b->dev + b->off; }
 inline uint8_t* bptr_mut(const MsqBuffer* b) { return (uint8_t*)b->dev + b->off; }
 inline bool buf_ok(const MsqBuffer* b, size_t need) { return b && b->dev && b->size >= need; }

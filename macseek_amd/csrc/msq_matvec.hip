@@ -78,6 +78,19 @@ bool mv_shape(int t, int rows, int cols, int groups, const MsqMvCfg* cfg, MvShap
   return true;
 }
 
+// LDS layout behind the tables and partial sums: the four partial sums of a fused norm, then the padded activation
+// rows the workgroup stages, `tokens` of them, when all of it fits under `limit` bytes (else the activations are read
+// straight from device memory; refused with a fused norm or when the kernel has no such path).
+bool place_x_row(MvArgs& a, size_t& lds, int tokens = 1, size_t limit = 64 * 1024, bool required = false) {
+  size_t at = (lds + 15) / 16 * 16;
+  if (a.norm_w) { a.norm_off = (uint32_t)(at / 4); at += 16; }
+  a.xs_off = (uint32_t)(at / 4);
+  const size_t end = at + (size_t)xlds_words(a.cols) * 4 * tokens;
+  a.stage_x = end <= limit ? 1u : 0u;
+  if (a.stage_x) lds = end;
+  return a.stage_x || !(a.norm_w || required);
+}
+
 template <class D>
 int launch_mv(hipStream_t st, const MvShape& s, MvArgs& a) {
   const int threads = 64 * s.rw * s.ks;
@@ -87,12 +100,7 @@ int launch_mv(hipStream_t st, const MvShape& s, MvArgs& a) {
   a.rpw = s.rpw;
   a.ntiles = (a.rows + tile_rows - 1) / tile_rows;
   size_t lds = (size_t)D::LDS_WORDS * 4 + (size_t)tile_rows * s.ks * 4;
-  if (a.norm_w) {  // fused input norm: partial sums and the normalized activations follow in LDS
-    lds = (lds + 15) / 16 * 16;
-    a.norm_off = (uint32_t)(lds / 4);
-    lds += 16 + (size_t)a.cols * 4;
-    if (lds > 64 * 1024) return MSQ_ERR_UNSUPPORTED;
-  }
+  if ((D::STAGE_X || a.norm_w) && !place_x_row(a, lds)) return MSQ_ERR_UNSUPPORTED;
   // persistent workgroups: as many as can be resident, never more than there are tiles
   const int wg_per_cu = std::max(1, std::min(2048 / threads, (int)((160 * 1024) / std::max<size_t>(lds, 1))));
   const int grid = (int)std::min<long>(a.ntiles, (long)device_info().cus * wg_per_cu);
@@ -177,16 +185,19 @@ int launch_mv_tok(hipStream_t st, const MvShape& s, MvTokArgs& ta) {
   a.ntiles = (a.rows + tile_rows - 1) / tile_rows;
   size_t lds = (size_t)D::LDS_WORDS * 4 + (size_t)tile_rows * s.ks * 4 * T * 4;
   const int gy = ((int)ta.n + T - 1) / T;
-  if (a.norm_w) {  // fused input norm (single token): partial sums and the normalized activations follow in LDS
-    lds = (lds + 15) / 16 * 16;
-    a.norm_off = (uint32_t)(lds / 4);
-    lds += 16 + (size_t)a.cols * 4;
-    if (lds > 64 * 1024) return MSQ_ERR_UNSUPPORTED;
+  if (D::STAGE_X || a.norm_w) {
+    if (!place_x_row(a, lds, tok_round<D, T>(), kMaxLds, true)) return MSQ_ERR_UNSUPPORTED;  // one workgroup per CU: all of its LDS
+  }
+  auto launch = [&](auto kernel, dim3 grid) {
+    allow_large_lds(kernel, lds);
+    hipLaunchKernelGGL(kernel, grid, dim3(threads), lds, st, ta);
+  };
+  if (a.norm_w) {  // fused input norm (single token)
     if constexpr (T != 1 || requires { D::STAGES; }) return MSQ_ERR_UNSUPPORTED;
     else {
-      const int gxn = (int)std::min<long>(a.ntiles, std::max(1, device_info().cus));
-      if (s.iters == 1) hipLaunchKernelGGL((mv_tok_kernel<D, 1, 1, true>), dim3(gxn), dim3(threads), lds, st, ta);
-      else if constexpr (D::UNIT == 8) hipLaunchKernelGGL((mv_tok_kernel<D, 2, 1, true>), dim3(gxn), dim3(threads), lds, st, ta);
+      const dim3 gxn((unsigned)std::min<long>(a.ntiles, std::max(1, device_info().cus)));
+      if (s.iters == 1) launch(mv_tok_kernel<D, 1, 1, true>, gxn);
+      else if constexpr (D::UNIT == 8) launch(mv_tok_kernel<D, 2, 1, true>, gxn);
       else return MSQ_ERR_UNSUPPORTED;
       MSQ_HIP(hipGetLastError());
       return MSQ_OK;
@@ -195,8 +206,8 @@ int launch_mv_tok(hipStream_t st, const MvShape& s, MvTokArgs& ta) {
   // persistent workgroups, one per CU over all token groups
   const int gx = (int)std::min<long>(a.ntiles, std::max(1, device_info().cus / gy));
   const dim3 grid((unsigned)gx, (unsigned)gy);
-  if (s.iters == 1) hipLaunchKernelGGL((mv_tok_kernel<D, 1, T>), grid, dim3(threads), lds, st, ta);
-  else if constexpr (D::UNIT == 8) hipLaunchKernelGGL((mv_tok_kernel<D, 2, T>), grid, dim3(threads), lds, st, ta);
+  if (s.iters == 1) launch(mv_tok_kernel<D, 1, T>, grid);
+  else if constexpr (D::UNIT == 8) launch(mv_tok_kernel<D, 2, T>, grid);
   else return MSQ_ERR_UNSUPPORTED;  // two block-format units per lane and T activation slices do not fit the registers
   MSQ_HIP(hipGetLastError());
   return MSQ_OK;

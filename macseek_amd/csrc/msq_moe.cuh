@@ -38,6 +38,9 @@ struct MoeArgs {
   uint32_t grid_routed;  // gate/up: workgroups [0, grid_routed) take routed rows, the rest shared rows
   uint32_t rows_per_wg_r, rows_per_wg_s;  // gate/up: virtual rows (expert * inter + row) per workgroup
   uint32_t rows_per_wg;  // down: rows of y per workgroup
+  // activations staged through LDS (padded rows of XLds): word offset in dynamic LDS, or read straight from device
+  // memory when stage_x is 0 (rows too long for LDS)
+  uint32_t xs_off, stage_x;
 };
 
 __device__ __forceinline__ float swiglu(float g, float u, float w) {  // quant_moe.metal:23-27
@@ -105,9 +108,16 @@ __device__ __forceinline__ void moe_gu_run_direct(const MoeArgs& a, uint32_t* sm
       }
     }
     if (first) {  // tables and activations arrive while the first weight rows are in flight
-      D::fill_lds(tbl, (int)tid, (int)blockDim.x);
-      xr = D::load_x(a.x, unit);
-      __syncthreads();
+      const CopyJob jobs[3] = {tbl_job_of<D>(0, 0u, true), tbl_job_of<D>(1, 0u, true),
+                               {(const uint4*)a.x, a.xs_off, a.stage_x ? a.dim / 4u : 0u, true}};
+      copy_jobs<4>(smem, jobs, tid, blockDim.x);
+      if (a.stage_x) {
+        __syncthreads();
+        xr = D::load_x(XLds{(const float*)(smem + a.xs_off)}, unit);
+      } else {
+        xr = D::load_x(a.x, unit);
+        __syncthreads();
+      }
       first = false;
     }
     for (uint32_t r0 = w0; r0 < w1; r0 += RPW) {
@@ -218,10 +228,17 @@ __device__ __forceinline__ void moe_gu_run_ring(const MoeArgs& a, uint32_t* smem
 #pragma unroll
     for (int s = 0; s < NR; s++) fetch(s);
     if (first) {  // tables and activations arrive while the first weight rows are in flight
-      D::fill_lds(tbl, (int)tid, (int)blockDim.x);
-      xr = D::load_x(a.x, unit);
+      const CopyJob jobs[3] = {tbl_job_of<D>(0, 0u, true), tbl_job_of<D>(1, 0u, true),
+                               {(const uint4*)a.x, a.xs_off, a.stage_x ? a.dim / 4u : 0u, true}};
+      copy_jobs<4>(smem, jobs, tid, blockDim.x);
+      if (a.stage_x) {
+        __syncthreads();
+        xr = D::load_x(XLds{(const float*)(smem + a.xs_off)}, unit);
+      } else {
+        xr = D::load_x(a.x, unit);
+        __syncthreads();
+      }
       if (!valid) xr = typename D::X{};
-      __syncthreads();
       first = false;
     }
     typename D::Look lk[2];  // stage t of a row pair uses lk[t & 1]; 2 NS stages per row pair keep the parity fixed
@@ -411,17 +428,25 @@ __global__ __launch_bounds__(MAXT) void moe_down_kernel(const MoeArgs a) {
       for (int s = 0; s < NSH; s++) fetch_s(s);
     }
     if (first) {
-      if (NE) {
-        DR::fill_lds(tbl_r, (int)tid, (int)blockDim.x);
-        xr = DR::load_x(a.h + (size_t)e * a.inter, unit_r);
-        if (!valid_r) xr = typename DR::X{};
+      // h rows this launch reads: the routed ones [0, NE), then the shared one at n_routed (NE is 0 or n_routed)
+      const uint32_t lo = NE ? 0u : a.n_routed * a.inter;
+      const uint32_t hi = (a.run_shared ? a.n_routed + 1u : a.n_routed) * a.inter;
+      const CopyJob jobs[5] = {tbl_job_of<DR>(0, 0u, NE), tbl_job_of<DR>(1, 0u, NE),
+                               tbl_job_of<DS>(0, DR::LDS_WORDS, a.run_shared), tbl_job_of<DS>(1, DR::LDS_WORDS, a.run_shared),
+                               {(const uint4*)(a.h + lo), a.xs_off, a.stage_x ? (hi - lo) / 4u : 0u, true}};
+      copy_jobs<(MAXT <= 768 ? 8 : 4)>(smem, jobs, tid, blockDim.x);
+      if (a.stage_x) {
+        const float* hs = (const float*)(smem + a.xs_off);
+        __syncthreads();
+        if (NE) xr = DR::load_x(XLds{hs + xlds_words(e * a.inter)}, unit_r);
+        if (a.run_shared) xs = DS::load_x(XLds{hs + xlds_words(a.n_routed * a.inter - lo)}, unit_s);
+      } else {
+        if (NE) xr = DR::load_x(a.h + (size_t)e * a.inter, unit_r);
+        if (a.run_shared) xs = DS::load_x(a.h + (size_t)a.n_routed * a.inter, unit_s);
+        __syncthreads();
       }
-      if (a.run_shared) {
-        DS::fill_lds(tbl_s, (int)tid, (int)blockDim.x);
-        xs = DS::load_x(a.h + (size_t)a.n_routed * a.inter, unit_s);
-        if (!valid_s) xs = typename DS::X{};
-      }
-      __syncthreads();
+      if (!valid_r) xr = typename DR::X{};
+      if (!valid_s) xs = typename DS::X{};
       first = false;
     }
     // ---- routed expert e, rows w0 .. w1

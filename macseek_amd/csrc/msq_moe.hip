@@ -13,12 +13,18 @@ bool shared_type_ok(int t) { return t == MSQ_Q6_K || t == MSQ_Q8_0 || t == MSQ_I
 
 template <class DR, class DS>
 void launch_gu_t(dim3 g, dim3 b, size_t lds, hipStream_t st, const MoeArgs& a) {
+  allow_large_lds(moe_gu_kernel<DR, DS>, lds);
   hipLaunchKernelGGL((moe_gu_kernel<DR, DS>), g, b, lds, st, a);
 }
 template <class DR, class DS>
 void launch_down_t(dim3 g, dim3 b, size_t lds, hipStream_t st, const MoeArgs& a) {
-  if (b.x <= 768) hipLaunchKernelGGL((moe_down_kernel<DR, DS, 768>), g, b, lds, st, a);
-  else hipLaunchKernelGGL((moe_down_kernel<DR, DS, 1024>), g, b, lds, st, a);
+  if (b.x <= 768) {
+    allow_large_lds(moe_down_kernel<DR, DS, 768>, lds);
+    hipLaunchKernelGGL((moe_down_kernel<DR, DS, 768>), g, b, lds, st, a);
+  } else {
+    allow_large_lds(moe_down_kernel<DR, DS, 1024>, lds);
+    hipLaunchKernelGGL((moe_down_kernel<DR, DS, 1024>), g, b, lds, st, a);
+  }
 }
 // launch-shape knobs for experiments (the reference exposes MACSEEK_MOE_* the same way, quant.mm:274-276)
 int env_int(const char* name, int dflt) {
@@ -35,12 +41,20 @@ size_t lds_words_for_shared(int ts, bool down) {
   }
   return down ? DR::LDS_WORDS + s : std::max<size_t>(DR::LDS_WORDS, s);
 }
+// the staged activations follow the tables and partial sums when everything fits the CU's LDS
+size_t place_x(MoeArgs& a, size_t lds, uint32_t x_cols) {
+  const size_t at = (lds + 15) / 16 * 16, end = at + (size_t)xlds_words(x_cols) * 4;
+  a.xs_off = (uint32_t)(at / 4);
+  a.stage_x = end <= (size_t)kMaxLds ? 1u : 0u;
+  return a.stage_x ? end : lds;
+}
 // dispatch over (routed type, shared type)
 template <bool DOWN>
-size_t dispatch(int tr, int ts, dim3 g, dim3 b, size_t part_bytes, hipStream_t st, const MoeArgs& a) {
+size_t dispatch(int tr, int ts, dim3 g, dim3 b, size_t part_bytes, uint32_t x_cols, hipStream_t st, MoeArgs& a) {
 #define MSQ_MOE_CASE(TR, DRT, TS, DST)                                                            \
   if (tr == TR && ts == TS) {                                                                     \
-    const size_t lds = 4 * lds_words_for_shared<DRT>(ts, DOWN) + part_bytes;                      \
+    size_t lds = 4 * lds_words_for_shared<DRT>(ts, DOWN) + part_bytes;                            \
+    lds = place_x(a, lds, x_cols);                                                                \
     if (DOWN) launch_down_t<DRT, DST>(g, b, lds, st, a); else launch_gu_t<DRT, DST>(g, b, lds, st, a); \
     return lds;                                                                                   \
   }
@@ -139,7 +153,7 @@ int moe_decode_impl(hipStream_t st, const MsqMoeDecodeArgs* p, const MsqBuffer* 
     if (g_r) { a.rows_per_wg_r = (uint32_t)((rows_r + g_r - 1) / g_r); g_r = (rows_r + a.rows_per_wg_r - 1) / a.rows_per_wg_r; }
     if (g_s) { a.rows_per_wg_s = (uint32_t)((rows_s + g_s - 1) / g_s); g_s = (rows_s + a.rows_per_wg_s - 1) / a.rows_per_wg_s; }
     a.grid_routed = (uint32_t)g_r;
-    if (!dispatch<false>(p->t_gate_up, ts, dim3((unsigned)(g_r + g_s)), dim3(threads), part_bytes, st, a))
+    if (!dispatch<false>(p->t_gate_up, ts, dim3((unsigned)(g_r + g_s)), dim3(threads), part_bytes, (uint32_t)dim, st, a))
       return unsupported("moe_decode type combo", p->t_gate_up, 0, 0);
     MSQ_HIP(hipGetLastError());
   }
@@ -161,7 +175,7 @@ int moe_decode_impl(hipStream_t st, const MsqMoeDecodeArgs* p, const MsqBuffer* 
     const long total = std::max<long>(1, (long)cus * std::max(1, env_d_wgs));
     a.rows_per_wg = (uint32_t)((dim + total - 1) / total);
     const long grid = (dim + a.rows_per_wg - 1) / a.rows_per_wg;
-    if (!dispatch<true>(p->t_down, ts, dim3((unsigned)grid), dim3(threads), part_bytes, st, a))
+    if (!dispatch<true>(p->t_down, ts, dim3((unsigned)grid), dim3(threads), part_bytes, (uint32_t)(((run_d_r ? nr : 0) + (d_s ? 1 : 0)) * inter), st, a))
       return unsupported("moe_decode type combo", p->t_down, 0, 0);
     MSQ_HIP(hipGetLastError());
   }

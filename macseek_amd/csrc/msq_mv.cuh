@@ -27,8 +27,30 @@ struct MvArgs {
   // fused input RMSNorm (NORM kernels only): x is replaced by x * rsqrt(mean(x^2) + eps) * norm_w
   const float* norm_w;
   float eps;
-  uint32_t norm_off;  // word offset in dynamic LDS of {partial sums [4], normalized activations [cols]}
+  uint32_t norm_off;  // word offset in dynamic LDS of the norm's four partial sums
+  // Activations staged through LDS (always for NORM kernels): word offset in dynamic LDS of the padded row
+  // (xlds_words(cols) words), and whether the plain kernels stage at all (rows too long for LDS are read directly)
+  uint32_t xs_off;
+  uint32_t stage_x;
 };
+
+// The lane's activation slices of one row, from the workgroup's padded LDS copy (staged here, all threads must call)
+// or straight from device memory.
+template <class D, int ITERS>
+__device__ __forceinline__ void load_x_row(const MvArgs& a, float* xs, const float* xg, const uint32_t (&unit)[ITERS],
+                                           typename D::X (&xr)[ITERS], uint32_t tid, uint32_t nt) {
+  if (D::STAGE_X && a.stage_x) {
+    __syncthreads();  // readers of the previous row are done
+    const float* src[1] = {xg};
+    stage_x_rows<1>(xs, src, 1u, 0u, a.cols, tid, nt);
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < ITERS; i++) xr[i] = D::load_x(XLds{xs}, unit[i]);
+  } else {
+#pragma unroll
+    for (int i = 0; i < ITERS; i++) xr[i] = D::load_x(xg, unit[i]);
+  }
+}
 
 // ---------------------------------------------------------------------------------------------------- RMSNorm
 // scale = 1 / sqrt(mean(x^2) + eps) of one row, computed by a workgroup with a reduction whose order does not depend
@@ -65,19 +87,17 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const float* x, const floa
   }
 }
 
-// Prologue of the NORM matvec kernels: the normalized activations of the (single) input row go to LDS as fp32, from
-// where load_x() converts them exactly as it would from device memory. Returns the LDS row.
-__device__ __forceinline__ const float* stage_normed_x(const MvArgs& a, uint32_t* smem, uint32_t tid, uint32_t lane, uint32_t wave,
-                                                       uint32_t nwaves) {
+// Prologue of the NORM matvec kernels: the normalized activations of the (single) input row go to LDS as fp32 (padded
+// layout of XLds), from where load_x() converts them exactly as it would from device memory.
+__device__ __forceinline__ void stage_normed_x(const MvArgs& a, uint32_t* smem, float* xs, uint32_t tid, uint32_t lane, uint32_t wave,
+                                               uint32_t nwaves) {
   float* red = (float*)(smem + a.norm_off);
-  float* xs = red + 4;
   const float r = rms_scale(a.x, a.cols, a.eps, red, lane, wave, nwaves);
   for (uint32_t i = tid; i < a.cols; i += nwaves * 64u) {
     const float v = a.x[i] * r;
-    xs[i] = v * a.norm_w[i];
+    xs[i + (i >> 5) * 4u] = v * a.norm_w[i];
   }
   __syncthreads();
-  return xs;
 }
 
 template <class D, int ITERS, bool NORM = false>
@@ -102,17 +122,20 @@ __global__ __launch_bounds__(1024) void mv_kernel(const MvArgs a) {
   }
   typename D::X xr[ITERS];
   uint32_t cur_group = 0xFFFFFFFFu;
-  const float* xbase = a.x;
-  if constexpr (NORM) xbase = stage_normed_x(a, smem, tid, lane, wave, nwaves);  // synchronises (one group only)
+  float* xs = (float*)(smem + a.xs_off);
+  if constexpr (NORM) stage_normed_x(a, smem, xs, tid, lane, wave, nwaves);  // synchronises (one group only)
   else if (D::LDS_WORDS) __syncthreads();
 
   for (uint32_t tile = blockIdx.x; tile < a.ntiles; tile += gridDim.x) {
     const uint32_t tile_row0 = tile * tile_rows;
     const uint32_t group = tile_row0 / a.rows_per_group;  // a tile never straddles two groups (host guarantees)
     if (group != cur_group) {
-      const float* xg = xbase + (size_t)group * a.x_group_stride;
+      if constexpr (NORM) {
 #pragma unroll
-      for (int i = 0; i < ITERS; i++) xr[i] = D::load_x(xg, unit[i]);
+        for (int i = 0; i < ITERS; i++) xr[i] = D::load_x(XLds{xs}, unit[i]);
+      } else {
+        load_x_row<D, ITERS>(a, xs, a.x + (size_t)group * a.x_group_stride, unit, xr, tid, blockDim.x);
+      }
       cur_group = group;
     }
     const uint32_t row0 = tile_row0 + rw * a.rpw;
@@ -195,7 +218,10 @@ __global__ __launch_bounds__(1024) void mv_ring_kernel(const MvArgs a) {
     }
     const uint32_t group = tile_row0 / a.rows_per_group;  // a tile never straddles two groups (host guarantees)
     if (group != cur_group) {
-      xr = D::load_x(a.x + (size_t)group * a.x_group_stride, unit);
+      const uint32_t units1[1] = {unit};
+      typename D::X x1[1];
+      load_x_row<D, 1>(a, (float*)(smem + a.xs_off), a.x + (size_t)group * a.x_group_stride, units1, x1, tid, blockDim.x);
+      xr = x1[0];
       if (!valid) xr = typename D::X{};
       cur_group = group;
     }
@@ -258,8 +284,18 @@ struct MvTokArgs {
   uint32_t x_stride, y_stride;   // elements between the activation / output rows of consecutive tokens
 };
 
+// Tokens whose activation rows a workgroup stages in LDS per round (a decoder with a large table leaves less room).
+template <class D, int T>
+constexpr int tok_round() {
+  constexpr int g = D::LDS_WORDS * 4 > 16 * 1024 ? 2 : 4;
+  return T < g ? T : g;
+}
+
+// Decoders with STAGE_X take the activations through LDS (contiguous loads, tok_round() tokens per round); with the
+// others every lane reads its slices from device memory, all T tokens' loads in flight at once.
 template <class D, int ITERS, int T, bool NORM = false>
 __global__ __launch_bounds__(512) void mv_tok_kernel(const MvTokArgs ta) {
+  constexpr bool STAGE = D::STAGE_X;
   const MvArgs& a = ta.m;
   extern __shared__ __attribute__((aligned(16))) uint32_t smem[];
   uint32_t* tbl = smem;
@@ -283,29 +319,48 @@ __global__ __launch_bounds__(512) void mv_tok_kernel(const MvTokArgs ta) {
   }
   typename D::X xr[T][ITERS];
   uint32_t cur_group = 0xFFFFFFFFu;
-  const float* xbase = a.x;
-  if constexpr (NORM) xbase = stage_normed_x(a, smem, tid, lane, wave, nwaves);  // synchronises (one token, one group)
+  float* xs = (float*)(smem + a.xs_off);
+  if constexpr (NORM) stage_normed_x(a, smem, xs, tid, lane, wave, nwaves);  // synchronises (one token, one group)
   else if (D::LDS_WORDS) __syncthreads();
+  const uint32_t roww = xlds_words(a.cols);
 
   for (uint32_t tile = blockIdx.x; tile < a.ntiles; tile += gridDim.x) {
     const uint32_t tile_row0 = tile * tile_rows;
     const uint32_t group = tile_row0 / a.rows_per_group;  // a tile never straddles two groups (host guarantees)
-    if (group != cur_group) {
-#pragma unroll
-      for (int t = 0; t < T; t++) {  // tokens past the last repeat it; their results are never stored
-        const float* xg = xbase + (size_t)min(t0 + t, ta.n - 1) * ta.x_stride + (size_t)group * a.x_group_stride;
-#pragma unroll
-        for (int i = 0; i < ITERS; i++) xr[t][i] = D::load_x(xg, unit[i]);
-      }
-      cur_group = group;
-    }
     const uint32_t row0 = tile_row0 + rw * a.rpw;
     const uint32_t last = min(min(row0 + a.rpw, a.rows) - 1u, a.rows - 1u);  // last row of this wave's run
-    typename D::Raw raw[ITERS];
+    typename D::Raw raw[ITERS];  // the first row is on its way while the activations are staged
     {
       const gptr_t wr = as_global(a.W) + (size_t)min(row0, last) * a.row_bytes;
 #pragma unroll
       for (int i = 0; i < ITERS; i++) raw[i] = D::load(wr, unit[i]);
+    }
+    if (group != cur_group) {
+      // tokens past the last repeat it; their results are never stored
+      auto x_of = [&](int t) { return a.x + (size_t)min(t0 + t, ta.n - 1) * ta.x_stride + (size_t)group * a.x_group_stride; };
+      constexpr int G = tok_round<D, T>();  // tokens staged per round (the host has made room for G padded rows)
+#pragma unroll
+      for (int t = 0; t < T; t++) {
+        if constexpr (NORM) {
+#pragma unroll
+          for (int i = 0; i < ITERS; i++) xr[t][i] = D::load_x(XLds{xs}, unit[i]);
+        } else if constexpr (!STAGE) {
+#pragma unroll
+          for (int i = 0; i < ITERS; i++) xr[t][i] = D::load_x(x_of(t), unit[i]);
+        } else {
+          if (t % G == 0) {
+            __syncthreads();  // readers of the previous round are done
+            const float* src[G];
+#pragma unroll
+            for (int k = 0; k < G; k++) src[k] = x_of(t + k);
+            stage_x_rows<G>(xs, src, G, roww, a.cols, tid, blockDim.x);
+            __syncthreads();
+          }
+#pragma unroll
+          for (int i = 0; i < ITERS; i++) xr[t][i] = D::load_x(XLds{xs + (t % G) * roww}, unit[i]);
+        }
+      }
+      cur_group = group;
     }
     for (uint32_t j = 0; j < a.rpw; j++) {
       typename D::Raw nxt[ITERS];  // the next row's bytes are requested before this row's arithmetic (after the
