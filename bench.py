@@ -30,8 +30,8 @@ HBM_PEAK_GBPS = 8000.0
 
 
 # HBM bytes per launch of the decode gate/up kernel, from the FETCH_SIZE / WRITE_SIZE counter runs of this workload
-# (KiB per dispatch, scaled by what the same counters read for a 1 GiB copy: x2.000 and x1.000): 42.87 MB + 0.06 MB
-GU_TRAFFIC_BYTES = 42935015
+# (KiB per dispatch, scaled by what the same counters read for a 1 GiB copy: x2.000 and x1.000): 42.91 MB + 0.06 MB
+GU_TRAFFIC_BYTES = 42970419
 
 
 def cores():
