@@ -44,20 +44,17 @@ extern "C" int msq_matvec_n(void* stream, int t, const MsqBuffer* W, int rows, i
   const int rpg = rows / groups;
   const double mb = (double)rb * rows / 1e6;
   // Two kernels serve n > 1. The dot-product kernel (weights fetched in contiguous runs, decoded once for up to eight
-  // tokens, dot2 chains per token) wins wherever its shape fits, except for more than eight tokens over a large matrix
-  // of a format whose MFMA fragments are cheap to build: measured on MI355X, IQ4_NL 7168x4096 at n = 16 takes 28.9 us
-  // there and 26.2 us through the MFMA kernel, Q8_0 4096x7168 35.2 and 30.6 us; Q6_K 1536x7168 14.4 against 42.9 us.
-  const bool cheap_fragments = t == MSQ_IQ4_NL || t == MSQ_Q8_0 || t == MSQ_F16 || t == MSQ_BF16;
-  const bool mfma_first = n > 8 && mb > 12.0 && cheap_fragments && !(groups > 1 && rpg % 16);
-  if (!mfma_first) {
+  // tokens, dot2 chains per token) wins wherever its shape fits: measured on MI355X at n = 16, IQ4_NL 7168x4096 takes
+  // 20.7 us there and 25.4 us through the MFMA kernel, Q8_0 4096x7168 28.8 and 29.6 us, Q6_K 1536x7168 14.4 and 42.9 us.
+  {
     const int rc = matvec_tok((hipStream_t)stream, t, bptr(W), rows, cols, (const float*)bptr(X), (float*)bptr_mut(Y), n, accumulate, groups);
     if (rc != MSQ_ERR_UNSUPPORTED) return rc;
   }
-  // Rows too wide for the dot-product kernel: a few tokens over a small matrix are served faster as n decode matvecs
-  // (the matrix stays in the caches after the first) than by the MFMA kernel: a matvec launch costs about
-  // 3 us + 1 us per 1.5 MB of weights, an MFMA launch about 20 us + 1 us per MB (one 16-row tile per workgroup pass,
-  // K split over its waves).
-  const bool few = !mfma_first && n * (3.0 + mb / 1.5) < 20.0 + mb;
+  // Rows too wide for the dot-product kernel (or for its activation staging in LDS): a few tokens over a small matrix
+  // are served faster as n decode matvecs (the matrix stays in the caches after the first) than by the MFMA kernel: a
+  // matvec launch costs about 3 us + 1 us per 1.5 MB of weights, an MFMA launch about 20 us + 1 us per MB (one 16-row
+  // tile per workgroup pass, K split over its waves).
+  const bool few = n * (3.0 + mb / 1.5) < 20.0 + mb;
   if (t == MSQ_F32 || (groups > 1 && rpg % 16) || few) {  // served as n decode matvecs
     for (int i = 0; i < n; i++) {
       const MsqBuffer xi{X->dev, X->off + (size_t)i * xs * 4, xs * 4}, yi{Y->dev, Y->off + (size_t)i * rows * 4, (size_t)rows * 4};

@@ -53,14 +53,19 @@ def test_matvec_n_vs_oracle(dev, t, rows, cols, groups, n, acc):
     got = Yd.cpu().numpy().astype(np.float64).reshape(n, rows)
     assert np.all(np.isfinite(got))
     # the library's dispatch: rows of up to 16384 columns (dense types: 8192) go through the dot-product kernel, which
-    # stages activations like the decode matvec, unless more than eight tokens meet a large matrix of a format with
-    # cheap MFMA fragments; wider rows through the MFMA kernel, or as n decode matvecs when that is cheaper
+    # stages activations like the decode matvec; the formats whose activation rows it stages in LDS also need room for
+    # the rows of a round there (160 KB less tables and partial sums: the latter are left out here). Wider rows go
+    # through the MFMA kernel, or as n decode matvecs when that is cheaper
     dots = cols <= (8192 if t in (O.F32, O.F16, O.BF16) else 16384)
+    if t in (O.IQ1_S, O.IQ2_XXS, O.IQ4_NL, O.Q8_0):
+        T = 1 if n == 1 else 4 if (t == O.Q8_0 or n <= 4) else 8
+        G = min(T, 2 if t == O.IQ1_S else 4)
+        table = {O.IQ1_S: 32768, O.IQ2_XXS: 6144, O.IQ4_NL: 1024, O.Q8_0: 0}[t]
+        dots = dots and table + G * (cols + cols // 32 * 4) * 4 <= 160 * 1024
     mb = q.row_bytes(q.QType(t), cols) * rows / 1e6
     mfma_ok = n > 1 and t != O.F32 and not (groups > 1 and (rows // groups) % 16)
-    mfma_first = mfma_ok and n > 8 and mb > 12.0 and t in (O.IQ4_NL, O.Q8_0, O.F16, O.BF16)
-    few = not mfma_first and n * (3.0 + mb / 1.5) < 20.0 + mb
-    uses_mfma = mfma_first or (mfma_ok and not dots and not few)
+    few = n * (3.0 + mb / 1.5) < 20.0 + mb
+    uses_mfma = mfma_ok and not dots and not few
     Xh = half_round(X, t) if uses_mfma else X
     if not uses_mfma and t not in (O.F32, O.F16, O.BF16, O.Q8_0):
         Xh = X.astype(np.float16).astype(np.float32)  # the decode (n = 1) path stages fp16 pairs for the block formats
