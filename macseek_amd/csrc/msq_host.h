@@ -38,7 +38,7 @@ template <class K>
 void allow_large_lds(K kernel, size_t lds) {
   static bool done = false;  // per instantiation; idempotent, so a race between first callers is harmless
   if (lds > 64 * 1024 && !done) {
-    hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, kMaxLds);
+    (void)hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, kMaxLds);
     done = true;
   }
 }
