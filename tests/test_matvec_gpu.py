@@ -69,6 +69,11 @@ CASES = [
     (O.F16, 1280, 5120, 1, False, "f16 synthetic"), (O.F16, 7, 768, 1, True, "f16 odd rows"),
     (O.Q6_K, 3, 256, 1, False, "tiny"), (O.IQ1_S, 1, 256, 1, False, "one row one block"),
     (O.IQ2_XXS, 5, 512, 1, True, "tiny acc"), (O.Q8_0, 9, 32, 1, False, "one q8 block per row"),
+    # activation rows staged through LDS: block-diagonal groups (one staged row per group), rows too long to stage
+    (O.IQ4_NL, 4096, 1024, 4, False, "staged x, groups"), (O.IQ1_S, 2048, 2048, 2, True, "staged x, groups acc"),
+    (O.Q8_0, 1024, 2048, 2, False, "staged x, groups"), (O.IQ2_XXS, 2048, 1024, 8, False, "staged x, groups"),
+    (O.IQ2_XXS, 16, 36864, 1, False, "row too long for LDS"), (O.Q8_0, 8, 16384, 1, True, "row too long for LDS acc"),
+    (O.IQ1_S, 600, 12288, 1, False, "long staged row"),
 ]
 
 
@@ -88,6 +93,26 @@ def test_matvec_vs_oracle(dev, t, rows, cols, groups, acc, what):
     got = yd.cpu().numpy()
     err_ref, err_ns = matvec_errors(got, ry, mag, wn2 + (y0.astype(np.float64) ** 2 if acc else 0), x, rows, cols, groups)
     print(f"  {O.TYPE_NAMES[t]:8s} {what:24s} [{cols:5d} -> {rows:6d}] g{groups} err/sum|wx| {err_ref:.2e} err/(|w||x|) {err_ns:.2e}")
+    assert err_ns <= TOL_NORTH_STAR
+    assert err_ref <= (TOL_REF_F32_X if t in F32_X_TYPES else TOL_REF_F16_X)
+
+
+@pytest.mark.parametrize("t,rows,cols", [(O.IQ1_S, 4096, 7168), (O.IQ4_NL, 520, 4096), (O.Q8_0, 300, 2048), (O.Q6_K, 1536, 7168)])
+def test_activation_offset_four_bytes(dev, t, rows, cols):
+    # x and y start 4 bytes into their buffers (not 16-byte aligned): the staging copies and the 128-bit slice loads
+    # must not assume more than the 4-byte alignment the operator interface gives
+    Wb = O.random_blocks(t, rows * cols, 17 + rows)
+    x = O.randn(cols, 23)
+    ry, mag, wn2 = O.matvec(t, Wb, rows, cols, x, 1)
+    arena, (W,) = place_in_arena([Wb])
+    xd = up(np.concatenate([np.zeros(1, np.float32), x]))
+    yd = up(np.zeros(rows + 1, np.float32))
+    e = q.Enc()
+    q.encode_matvec(e, t, W, rows, cols, q.Buffer.of(xd).sub(4, cols * 4), q.Buffer.of(yd).sub(4, rows * 4), False, 1)
+    e.wait()
+    got = yd.cpu().numpy()
+    assert got[0] == 0.0
+    err_ref, err_ns = matvec_errors(got[1:], ry, mag, wn2, x, rows, cols, 1)
     assert err_ns <= TOL_NORTH_STAR
     assert err_ref <= (TOL_REF_F32_X if t in F32_X_TYPES else TOL_REF_F16_X)
 

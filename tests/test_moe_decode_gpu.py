@@ -109,6 +109,8 @@ CASES = [  # (gu, down, shared type, n_routed, shared, xscale, dim, inter)
     (T.IQ1_S, T.IQ1_S, T.IQ2_XXS, 6, True, 1.0, 7168, 2048),  # BASELINE batch-1 MoE layer
     (T.IQ2_XXS, T.IQ1_S, T.IQ1_S, 5, True, 1.0, 7168, 2048),
     (T.IQ1_S, T.IQ1_S, T.IQ2_XXS, 1, True, 40.0, 512, 256),   # smallest shapes the kernels accept
+    (T.IQ1_S, T.IQ1_S, T.Q8_0, 2, True, 1.0, 32768, 256),     # x too long to stage in LDS: gate/up reads it directly
+    (T.IQ2_XXS, T.IQ1_S, T.IQ2_XXS, 1, True, 1.0, 256, 16384),  # h rows too long to stage: down reads them directly
 ]
 
 
