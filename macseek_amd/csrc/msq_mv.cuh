@@ -329,11 +329,18 @@ __global__ __launch_bounds__(512) void mv_tok_kernel(const MvTokArgs ta) {
     const uint32_t group = tile_row0 / a.rows_per_group;  // a tile never straddles two groups (host guarantees)
     const uint32_t row0 = tile_row0 + rw * a.rpw;
     const uint32_t last = min(min(row0 + a.rpw, a.rows) - 1u, a.rows - 1u);  // last row of this wave's run
-    typename D::Raw raw[ITERS];  // the first row is on its way while the activations are staged
-    {
-      const gptr_t wr = as_global(a.W) + (size_t)min(row0, last) * a.row_bytes;
+    // The wave's first NR rows are on their way while the activations are staged; a slot is refilled with the row NR
+    // places ahead before its own bytes are used (rows past the run's last repeat it: no branch around a load).
+    // Four rows in flight pay for the codebook formats at one token (a row slice is 8 bytes per lane: IQ1_S 4096x7168
+    // 8.5 -> 7.5 us); the others move 18 to 34 bytes per lane and row, and the rows repeated at the end of a run cost
+    // them more than the deeper ring gains (Q8_0 4096x4096 8.4 -> 9.8 us, Q6_K 1536x7168 6.2 -> 7.8 us).
+    constexpr int NR = (T == 1 && requires { D::STAGES; }) ? 4 : 1;
+    typename D::Raw ring[NR][ITERS];
 #pragma unroll
-      for (int i = 0; i < ITERS; i++) raw[i] = D::load(wr, unit[i]);
+    for (int s = 0; s < NR; s++) {
+      const gptr_t wr = as_global(a.W) + (size_t)min(row0 + s, last) * a.row_bytes;
+#pragma unroll
+      for (int i = 0; i < ITERS; i++) ring[s][i] = D::load(wr, unit[i]);
     }
     if (group != cur_group) {
       // tokens past the last repeat it; their results are never stored
@@ -362,13 +369,7 @@ __global__ __launch_bounds__(512) void mv_tok_kernel(const MvTokArgs ta) {
       }
       cur_group = group;
     }
-    for (uint32_t j = 0; j < a.rpw; j++) {
-      typename D::Raw nxt[ITERS];  // the next row's bytes are requested before this row's arithmetic (after the
-      {                            // run's last row: that row again, which the caches hold)
-        const gptr_t wr = as_global(a.W) + (size_t)min(row0 + j + 1, last) * a.row_bytes;
-#pragma unroll
-        for (int i = 0; i < ITERS; i++) nxt[i] = D::load(wr, unit[i]);
-      }
+    auto row_dot = [&](const typename D::Raw (&raw)[ITERS], uint32_t j) {
       float acc[T];
 #pragma unroll
       for (int t = 0; t < T; t++) {
@@ -382,8 +383,16 @@ __global__ __launch_bounds__(512) void mv_tok_kernel(const MvTokArgs ta) {
       // transposed fold: afterwards acc[0] of lane l is token group8_sel<T>(l) summed over l's 16-lane row
       row16_fold<T>(acc, lane);
       if (!(lane & 8u)) part[(((rw * a.rpw + j) * KS + ks) * 4 + (lane >> 4)) * T + group8_sel<T>(lane)] = acc[0];
+    };
+    for (uint32_t j0 = 0; j0 < a.rpw; j0 += NR) {
 #pragma unroll
-      for (int i = 0; i < ITERS; i++) raw[i] = nxt[i];
+      for (int s = 0; s < NR; s++) {
+        typename D::Raw cur[ITERS];
+        const gptr_t wr = as_global(a.W) + (size_t)min(row0 + j0 + s + NR, last) * a.row_bytes;
+#pragma unroll
+        for (int i = 0; i < ITERS; i++) { cur[i] = ring[s][i]; ring[s][i] = D::load(wr, unit[i]); }
+        if (NR == 1 || j0 + s < a.rpw) row_dot(cur, j0 + s);  // wave-uniform; no load inside
+      }
     }
     __syncthreads();
     for (uint32_t idx = tid; idx < tile_rows * T; idx += blockDim.x) {
