@@ -32,14 +32,15 @@ inline int hip_fail(hipError_t e, const char* where) {
     if (e_ != hipSuccess) return ::msq::hip_fail(e_, #expr); \
   } while (0)
 
-// LDS of one CU; a kernel that takes more than 64 KB of it as dynamic LDS has to be told so once
+// LDS of one CU; a kernel that takes more than 64 KB of it as dynamic LDS has to be told so (the limit granted so far
+// is kept per kernel instantiation; raising it again is idempotent, so a race between callers is harmless)
 constexpr int kMaxLds = 160 * 1024;
 template <class K>
 void allow_large_lds(K kernel, size_t lds) {
-  static bool done = false;  // per instantiation; idempotent, so a race between first callers is harmless
-  if (lds > 64 * 1024 && !done) {
-    (void)hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, kMaxLds);
-    done = true;
+  static size_t granted = 64 * 1024;
+  if (lds > granted) {
+    (void)hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    granted = lds;
   }
 }
 inline const uint8_t* bptr(const MsqBuffer* b) { return (const uint8_t*)b->dev + b->off; }

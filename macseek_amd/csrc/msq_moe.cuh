@@ -64,9 +64,8 @@ __device__ __forceinline__ const void* uniform(const void* p) {
 
 // gate + up + SwiGLU over the virtual rows [wg * per, ...) of one kind of expert (routed: e * inter + r; shared: r).
 template <class D, int RPW>
-__device__ __forceinline__ void moe_gu_run_direct(const MoeArgs& a, uint32_t* smem, const bool shared, const uint32_t wg) {
-  uint32_t* tbl = smem;
-  float* part = (float*)(smem + D::LDS_WORDS);
+__device__ __forceinline__ void moe_gu_run_direct(const MoeArgs& a, uint32_t* tbl, uint32_t* smem, const bool shared, const uint32_t wg) {
+  float* part = (float*)smem;
   const uint32_t tid = threadIdx.x, lane = tid & 63u;
   const uint32_t wave = uniform(tid >> 6), nwaves = blockDim.x >> 6;
   const uint32_t KS = a.ks, ks = wave % KS, rw = wave / KS, RW = nwaves / KS;
@@ -109,8 +108,8 @@ __device__ __forceinline__ void moe_gu_run_direct(const MoeArgs& a, uint32_t* sm
     }
     if (first) {  // tables and activations arrive while the first weight rows are in flight
       const CopyJob jobs[3] = {tbl_job_of<D>(0, 0u, true), tbl_job_of<D>(1, 0u, true),
-                               {(const uint4*)a.x, a.xs_off, a.stage_x ? a.dim / 4u : 0u, true}};
-      copy_jobs<4>(smem, jobs, tid, blockDim.x);
+                               {(const uint4*)a.x, (uint32_t)(smem - tbl) + a.xs_off, a.stage_x ? a.dim / 4u : 0u, true}};
+      copy_jobs<4>(tbl, jobs, tid, blockDim.x);
       if (a.stage_x) {
         __syncthreads();
         xr = D::load_x(XLds{(const float*)(smem + a.xs_off)}, unit);
@@ -175,11 +174,10 @@ __device__ __forceinline__ void moe_gu_run_direct(const MoeArgs& a, uint32_t* sm
 // names an exact number of loads that may stay in flight. Table lookups run one decoder stage ahead of the dot
 // products (two alternating lookup buffers), so LDS latency overlaps the math as well.
 template <class D>
-__device__ __forceinline__ void moe_gu_run_ring(const MoeArgs& a, uint32_t* smem, const bool shared, const uint32_t wg) {
+__device__ __forceinline__ void moe_gu_run_ring(const MoeArgs& a, uint32_t* tbl, uint32_t* smem, const bool shared, const uint32_t wg) {
   constexpr int NR = 4;  // row pairs in flight per wave
   constexpr int NS = D::STAGES;
-  uint32_t* tbl = smem;
-  float* part = (float*)(smem + D::LDS_WORDS);
+  float* part = (float*)smem;
   const uint32_t tid = threadIdx.x, lane = tid & 63u;
   const uint32_t wave = uniform(tid >> 6), nwaves = blockDim.x >> 6;
   const uint32_t KS = a.ks, ks = wave % KS, rw = wave / KS, RW = nwaves / KS;
@@ -229,8 +227,8 @@ __device__ __forceinline__ void moe_gu_run_ring(const MoeArgs& a, uint32_t* smem
     for (int s = 0; s < NR; s++) fetch(s);
     if (first) {  // tables and activations arrive while the first weight rows are in flight
       const CopyJob jobs[3] = {tbl_job_of<D>(0, 0u, true), tbl_job_of<D>(1, 0u, true),
-                               {(const uint4*)a.x, a.xs_off, a.stage_x ? a.dim / 4u : 0u, true}};
-      copy_jobs<4>(smem, jobs, tid, blockDim.x);
+                               {(const uint4*)a.x, (uint32_t)(smem - tbl) + a.xs_off, a.stage_x ? a.dim / 4u : 0u, true}};
+      copy_jobs<4>(tbl, jobs, tid, blockDim.x);
       if (a.stage_x) {
         __syncthreads();
         xr = D::load_x(XLds{(const float*)(smem + a.xs_off)}, unit);
@@ -297,16 +295,21 @@ __device__ __forceinline__ void moe_gu_run_ring(const MoeArgs& a, uint32_t* smem
 }
 
 template <class D>
-__device__ __forceinline__ void moe_gu_run(const MoeArgs& a, uint32_t* smem, const bool shared, const uint32_t wg) {
-  if constexpr (requires { D::STAGES; }) moe_gu_run_ring<D>(a, smem, shared, wg);
-  else moe_gu_run_direct<D, rows_in_flight<D>(2)>(a, smem, shared, wg);
+__device__ __forceinline__ void moe_gu_run(const MoeArgs& a, uint32_t* tbl, uint32_t* smem, const bool shared, const uint32_t wg) {
+  if constexpr (requires { D::STAGES; }) moe_gu_run_ring<D>(a, tbl, smem, shared, wg);
+  else moe_gu_run_direct<D, rows_in_flight<D>(2)>(a, tbl, smem, shared, wg);
 }
 
 template <class DR, class DS>
 __global__ __launch_bounds__(1024) void moe_gu_kernel(const MoeArgs a) {
+  // The codebook table is a static array: its LDS address is a compile-time constant that goes into the offset field
+  // of the lookups (with a table in dynamic LDS every lookup address ends in an addition of the base). Partial sums and
+  // the staged activations follow in dynamic LDS.
+  constexpr int TBL = DR::LDS_WORDS > DS::LDS_WORDS ? DR::LDS_WORDS : DS::LDS_WORDS;
+  __shared__ __attribute__((aligned(16))) uint32_t tbl[TBL > 0 ? TBL : 4];
   extern __shared__ __attribute__((aligned(16))) uint32_t smem[];
-  if (blockIdx.x < a.grid_routed) moe_gu_run<DR>(a, smem, false, blockIdx.x);
-  else moe_gu_run<DS>(a, smem, true, blockIdx.x - a.grid_routed);
+  if (blockIdx.x < a.grid_routed) moe_gu_run<DR>(a, tbl, smem, false, blockIdx.x);
+  else moe_gu_run<DS>(a, tbl, smem, true, blockIdx.x - a.grid_routed);
 }
 
 // down: workgroup = RW row-groups x (NE expert-waves x KS K-split waves). In a row-group, wave (e, ks) owns routed
@@ -361,11 +364,12 @@ __global__ __launch_bounds__(MAXT) void moe_down_kernel(const MoeArgs a) {
   constexpr bool RING_R = requires { DR::STAGES; }, RING_S = requires { DS::STAGES; };
   constexpr int RPW = rows_in_flight<DR>(1);
   constexpr int NR = 4, NSH = 4;  // ring depth: routed rows, shared rows
-  extern __shared__ __attribute__((aligned(16))) uint32_t smem[];
   constexpr int TBL = DR::LDS_WORDS + DS::LDS_WORDS;
-  uint32_t* tbl_r = smem;
-  uint32_t* tbl_s = smem + DR::LDS_WORDS;
-  float* part = (float*)(smem + TBL);
+  __shared__ __attribute__((aligned(16))) uint32_t tbl[TBL > 0 ? TBL : 4];  // static: see moe_gu_kernel
+  extern __shared__ __attribute__((aligned(16))) uint32_t smem[];
+  uint32_t* tbl_r = tbl;
+  uint32_t* tbl_s = tbl + DR::LDS_WORDS;
+  float* part = (float*)smem;
 
   const uint32_t tid = threadIdx.x, lane = tid & 63u;
   const uint32_t wave = uniform(tid >> 6), nwaves = blockDim.x >> 6;
@@ -433,8 +437,8 @@ __global__ __launch_bounds__(MAXT) void moe_down_kernel(const MoeArgs a) {
       const uint32_t hi = (a.run_shared ? a.n_routed + 1u : a.n_routed) * a.inter;
       const CopyJob jobs[5] = {tbl_job_of<DR>(0, 0u, NE), tbl_job_of<DR>(1, 0u, NE),
                                tbl_job_of<DS>(0, DR::LDS_WORDS, a.run_shared), tbl_job_of<DS>(1, DR::LDS_WORDS, a.run_shared),
-                               {(const uint4*)(a.h + lo), a.xs_off, a.stage_x ? (hi - lo) / 4u : 0u, true}};
-      copy_jobs<(MAXT <= 768 ? 8 : 4)>(smem, jobs, tid, blockDim.x);
+                               {(const uint4*)(a.h + lo), (uint32_t)(smem - tbl) + a.xs_off, a.stage_x ? (hi - lo) / 4u : 0u, true}};
+      copy_jobs<(MAXT <= 768 ? 8 : 4)>(tbl, jobs, tid, blockDim.x);
       if (a.stage_x) {
         const float* hs = (const float*)(smem + a.xs_off);
         __syncthreads();

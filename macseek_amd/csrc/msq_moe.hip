@@ -41,11 +41,12 @@ size_t lds_words_for_shared(int ts, bool down) {
   }
   return down ? DR::LDS_WORDS + s : std::max<size_t>(DR::LDS_WORDS, s);
 }
-// the staged activations follow the tables and partial sums when everything fits the CU's LDS
-size_t place_x(MoeArgs& a, size_t lds, uint32_t x_cols) {
+// the staged activations follow the partial sums in dynamic LDS when everything (with the kernel's static table) fits
+// the CU's LDS
+size_t place_x(MoeArgs& a, size_t lds, uint32_t x_cols, size_t static_lds) {
   const size_t at = (lds + 15) / 16 * 16, end = at + (size_t)xlds_words(x_cols) * 4;
   a.xs_off = (uint32_t)(at / 4);
-  a.stage_x = end <= (size_t)kMaxLds ? 1u : 0u;
+  a.stage_x = end + static_lds + 64 <= (size_t)kMaxLds ? 1u : 0u;
   return a.stage_x ? end : lds;
 }
 // dispatch over (routed type, shared type)
@@ -53,8 +54,8 @@ template <bool DOWN>
 size_t dispatch(int tr, int ts, dim3 g, dim3 b, size_t part_bytes, uint32_t x_cols, hipStream_t st, MoeArgs& a) {
 #define MSQ_MOE_CASE(TR, DRT, TS, DST)                                                            \
   if (tr == TR && ts == TS) {                                                                     \
-    size_t lds = 4 * lds_words_for_shared<DRT>(ts, DOWN) + part_bytes;                            \
-    lds = place_x(a, lds, x_cols);                                                                \
+    const size_t tbl = 4 * lds_words_for_shared<DRT>(ts, DOWN);  /* static LDS of the kernel */    \
+    const size_t lds = place_x(a, part_bytes, x_cols, tbl);                                       \
     if (DOWN) launch_down_t<DRT, DST>(g, b, lds, st, a); else launch_gu_t<DRT, DST>(g, b, lds, st, a); \
     return lds;                                                                                   \
   }
