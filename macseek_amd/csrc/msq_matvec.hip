@@ -78,7 +78,11 @@ bool mv_shape(int t, int rows, int cols, int groups, const MsqMvCfg* cfg, MvShap
   return true;
 }
 
-// LDS layout behind the tables and partial sums: the four partial sums of a fused norm, then the padded activation
+// static LDS of the matvec kernels of decoder D: the codebook table (an array of at least four words)
+template <class D>
+constexpr size_t kStaticLds = (D::LDS_WORDS > 0 ? D::LDS_WORDS : 4) * 4 + 64;
+
+// LDS layout behind the partial sums: the four partial sums of a fused norm, then the padded activation
 // rows the workgroup stages, `tokens` of them, when all of it fits under `limit` bytes (else the activations are read
 // straight from device memory; refused with a fused norm or when the kernel has no such path).
 bool place_x_row(MvArgs& a, size_t& lds, int tokens = 1, size_t limit = 64 * 1024, bool required = false) {
@@ -99,10 +103,10 @@ int launch_mv(hipStream_t st, const MvShape& s, MvArgs& a) {
   a.ks = s.ks;
   a.rpw = s.rpw;
   a.ntiles = (a.rows + tile_rows - 1) / tile_rows;
-  size_t lds = (size_t)D::LDS_WORDS * 4 + (size_t)tile_rows * s.ks * 4;
-  if ((D::STAGE_X || a.norm_w) && !place_x_row(a, lds)) return MSQ_ERR_UNSUPPORTED;
+  size_t lds = (size_t)tile_rows * s.ks * 4;  // dynamic LDS: partial sums, staged activations (the table is static)
+  if ((D::STAGE_X || a.norm_w) && !place_x_row(a, lds, 1, 64 * 1024 - kStaticLds<D>)) return MSQ_ERR_UNSUPPORTED;
   // persistent workgroups: as many as can be resident, never more than there are tiles
-  const int wg_per_cu = std::max(1, std::min(2048 / threads, (int)((160 * 1024) / std::max<size_t>(lds, 1))));
+  const int wg_per_cu = std::max(1, std::min(2048 / threads, (int)((size_t)kMaxLds / (lds + kStaticLds<D>))));
   const int grid = (int)std::min<long>(a.ntiles, (long)device_info().cus * wg_per_cu);
   if (a.norm_w) {
     if constexpr (requires { D::STAGES; }) return MSQ_ERR_UNSUPPORTED;  // codebook formats: as in the reference (quant.mm:110)
@@ -183,10 +187,10 @@ int launch_mv_tok(hipStream_t st, const MvShape& s, MvTokArgs& ta) {
   a.ks = s.ks;
   a.rpw = s.rpw;
   a.ntiles = (a.rows + tile_rows - 1) / tile_rows;
-  size_t lds = (size_t)D::LDS_WORDS * 4 + (size_t)tile_rows * s.ks * 4 * T * 4;
+  size_t lds = (size_t)tile_rows * s.ks * 4 * T * 4;  // dynamic LDS: partial sums, staged activations (the table is static)
   const int gy = ((int)ta.n + T - 1) / T;
   if (D::STAGE_X || a.norm_w) {
-    if (!place_x_row(a, lds, tok_round<D, T>(), kMaxLds, true)) return MSQ_ERR_UNSUPPORTED;  // one workgroup per CU: all of its LDS
+    if (!place_x_row(a, lds, tok_round<D, T>(), kMaxLds - kStaticLds<D>, true)) return MSQ_ERR_UNSUPPORTED;  // one workgroup per CU: all of its LDS
   }
   auto launch = [&](auto kernel, dim3 grid) {
     allow_large_lds(kernel, lds);

@@ -103,8 +103,10 @@ __device__ __forceinline__ void stage_normed_x(const MvArgs& a, uint32_t* smem, 
 template <class D, int ITERS, bool NORM = false>
 __global__ __launch_bounds__(1024) void mv_kernel(const MvArgs a) {
   extern __shared__ __attribute__((aligned(16))) uint32_t smem[];
-  uint32_t* tbl = smem;
-  float* part = (float*)(smem + D::LDS_WORDS);
+  // the codebook table is a static array: its LDS address is a compile-time constant, which saves the addition of a base
+  // in every lookup address; partial sums (and staged activations) follow in dynamic LDS
+  __shared__ __attribute__((aligned(16))) uint32_t tbl[D::LDS_WORDS > 0 ? D::LDS_WORDS : 4];
+  float* part = (float*)smem;
 
   const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6, nwaves = blockDim.x >> 6;
   const uint32_t KS = a.ks, ks = wave % KS, rw = wave / KS, RW = nwaves / KS;
@@ -183,8 +185,10 @@ __global__ __launch_bounds__(1024) void mv_ring_kernel(const MvArgs a) {
   constexpr bool BUFFER = requires { D::STAGES; };  // codebook decoders: buffer loads and staged table lookups
   constexpr int NR = 4;
   extern __shared__ __attribute__((aligned(16))) uint32_t smem[];
-  uint32_t* tbl = smem;
-  float* part = (float*)(smem + D::LDS_WORDS);
+  // the codebook table is a static array: its LDS address is a compile-time constant, which saves the addition of a base
+  // in every lookup address; partial sums (and staged activations) follow in dynamic LDS
+  __shared__ __attribute__((aligned(16))) uint32_t tbl[D::LDS_WORDS > 0 ? D::LDS_WORDS : 4];
+  float* part = (float*)smem;
 
   const uint32_t tid = threadIdx.x, lane = tid & 63u, nwaves = blockDim.x >> 6;
   const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
@@ -298,8 +302,10 @@ __global__ __launch_bounds__(512) void mv_tok_kernel(const MvTokArgs ta) {
   constexpr bool STAGE = D::STAGE_X;
   const MvArgs& a = ta.m;
   extern __shared__ __attribute__((aligned(16))) uint32_t smem[];
-  uint32_t* tbl = smem;
-  float* part = (float*)(smem + D::LDS_WORDS);  // [row of tile][ks][16-lane row of the wave][T]
+  // the codebook table is a static array: its LDS address is a compile-time constant, which saves the addition of a base
+  // in every lookup address; partial sums (and staged activations) follow in dynamic LDS
+  __shared__ __attribute__((aligned(16))) uint32_t tbl[D::LDS_WORDS > 0 ? D::LDS_WORDS : 4];
+  float* part = (float*)smem;  // [row of tile][ks][16-lane row of the wave][T]
 
   const uint32_t tid = threadIdx.x, lane = tid & 63u, nwaves = blockDim.x >> 6;
   const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
