@@ -14,7 +14,7 @@ int launch_mvn(hipStream_t st, MvnArgs a) {
   const uint32_t ks = std::min<uint32_t>(16u, a.nsteps);
   a.steps_per_wave = (a.nsteps + ks - 1) / ks;
   const uint32_t waves = (a.nsteps + a.steps_per_wave - 1) / a.steps_per_wave;
-  const size_t lds = (size_t)F::LDS_WORDS * 4 + (size_t)waves * 16 * 17 * 4;
+  const size_t lds = (size_t)waves * 16 * 17 * 4;  // dynamic LDS: the partial results (the table is a static array)
   // resident workgroups per CU (the kernel takes up to 128 registers per lane: 16 waves per CU); a persistent
   // workgroup keeps its activation fragments across tiles, a later one would stage them again
   const int wg_per_cu = std::max(1, 16 / (int)waves);

@@ -31,8 +31,8 @@ __global__ __launch_bounds__(1024) void mvn_kernel(const MvnArgs a) {
   constexpr int MS = kMvnSubSteps;
   constexpr bool HALF_SCALES = requires(const uint8_t* r, float& s) { F::get_scales(r, 0u, s, s); };
   extern __shared__ __attribute__((aligned(16))) uint32_t smem[];
-  uint32_t* tbl = smem;
-  float* red = (float*)(smem + F::LDS_WORDS);  // [wave][token][17]
+  __shared__ __attribute__((aligned(16))) uint32_t tbl[F::LDS_WORDS > 0 ? F::LDS_WORDS : 4];  // static: a known address
+  float* red = (float*)smem;  // [wave][token][17]
 
   const uint32_t tid = threadIdx.x, lane = tid & 63u;
   const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6)), nwaves = blockDim.x >> 6;
