@@ -210,14 +210,16 @@ template <class B>
 constexpr size_t pf_blk_lds(int T) { return (size_t)B::LDS_WORDS * 4 + (T > 3 ? 1 : 2) * (size_t)(T > 3 ? kPfBigTokens : kPfBlkTokens) * kPfBlkPitch; }
 
 template <class B, bool GU, int T>
-__device__ __forceinline__ void pf_block_body(const PfBlkArgs& a, uint32_t* tbl, uint8_t* abuf) {
+__device__ __forceinline__ void pf_block_body(const PfBlkArgs& a) {
   constexpr int WAVES = pf_blk_waves(T), NT = 64 * WAVES;
   constexpr int NM = GU ? 2 : 1, RT = pf_blk_rt(GU, T), R = RT * NM, PITCH = kPfBlkPitch;
   constexpr bool DB = T <= 3;  // two activation buffers
   constexpr int ABUF = (DB ? kPfBlkTokens : kPfBigTokens) * PITCH;
   constexpr int PPS = R / 2, NP = 8 * PPS;  // fragment pairs per K step, per block
   static_assert(R == 2 || R == 4, "fragments are processed in pairs");
-  // tbl: [B::LDS_WORDS]; abuf: [2][T * 16 tokens][PITCH] (one buffer for T > 3); both static LDS of the kernel
+  extern __shared__ __attribute__((aligned(16))) uint32_t smem[];
+  uint32_t* tbl = smem;
+  uint8_t* abuf = (uint8_t*)(smem + B::LDS_WORDS);  // [2][T * 16 tokens][PITCH]
   const uint32_t tid = threadIdx.x, lane = tid & 63u;
   const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
   const uint32_t n16 = lane & 15u, q = lane >> 4;
@@ -396,17 +398,13 @@ __device__ __forceinline__ void pf_block_body(const PfBlkArgs& a, uint32_t* tbl,
 // then decoded half as often; 12 waves, one activation buffer).
 template <class B, bool GU, int T>
 __global__ __launch_bounds__(64 * pf_blk_waves(T)) void moe_pf_block_kernel(const PfBlkArgs a) {
-  // static LDS: table and activation buffers at addresses the compiler knows (they go into the offset fields of the
-  // LDS instructions instead of being added to every lookup address)
-  __shared__ __attribute__((aligned(16))) uint32_t tbl[B::LDS_WORDS];
-  __shared__ __attribute__((aligned(16))) uint8_t abuf[pf_blk_lds<B>(T) - (size_t)B::LDS_WORDS * 4];
   if constexpr (T == 1 || T > 3) {
-    pf_block_body<B, GU, T>(a, tbl, abuf);
+    pf_block_body<B, GU, T>(a);
   } else {
     const uint32_t item = ((blockIdx.x >> 3) / a.row_chunks) * 8u + (blockIdx.x & 7u);
     if (item >= a.nitems) return;
-    if (a.items[3 * item + 2] > 32) pf_block_body<B, GU, 3>(a, tbl, abuf);
-    else pf_block_body<B, GU, 2>(a, tbl, abuf);
+    if (a.items[3 * item + 2] > 32) pf_block_body<B, GU, 3>(a);
+    else pf_block_body<B, GU, 2>(a);
   }
 }
 

@@ -49,8 +49,13 @@ int launch_block_tt(hipStream_t st, PfBlkArgs a) {
   if (!a.nitems) return MSQ_OK;
   const uint32_t rows_per_item = pf_blk_rows(GU, T);
   a.row_chunks = (a.N + rows_per_item - 1) / rows_per_item;
+  static bool attr_set = false;  // per instantiation: allow more than 64 KiB of dynamic LDS
+  if (!attr_set) {
+    MSQ_HIP(hipFuncSetAttribute((const void*)moe_pf_block_kernel<B, GU, T>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+    attr_set = true;
+  }
   const uint32_t grid = ((a.nitems + 7) / 8) * 8 * a.row_chunks;
-  hipLaunchKernelGGL((moe_pf_block_kernel<B, GU, T>), dim3(grid), dim3(64 * pf_blk_waves(T)), 0, st, a);  // all of its LDS is static
+  hipLaunchKernelGGL((moe_pf_block_kernel<B, GU, T>), dim3(grid), dim3(64 * pf_blk_waves(T)), pf_blk_lds<B>(T), st, a);
   MSQ_HIP(hipGetLastError());
   return MSQ_OK;
 }
