@@ -63,7 +63,16 @@ __device__ __forceinline__ float rms_scale(const float* __restrict__ x, uint32_t
                                            uint32_t wave, uint32_t nwaves) {
   for (uint32_t v = wave; v < 4u; v += nwaves) {
     float ss = 0.f;
-    for (uint32_t i = v * 64u + lane; i < dim; i += 256u) ss = __builtin_fmaf(x[i], x[i], ss);
+    // eight elements are requested before the first is used (one at a time the loop is a chain of memory latencies);
+    // indices past the end repeat the last element and are left out of the sum, so the order of additions stays
+    for (uint32_t i0 = v * 64u + lane; i0 < dim; i0 += 8u * 256u) {
+      float t[8];
+#pragma unroll
+      for (int k = 0; k < 8; k++) t[k] = x[min(i0 + 256u * k, dim - 1u)];
+#pragma unroll
+      for (int k = 0; k < 8; k++)
+        if (i0 + 256u * k < dim) ss = __builtin_fmaf(t[k], t[k], ss);
+    }
     ss = wave_sum(ss);
     if (lane == 0) red[v] = ss;
   }
@@ -81,9 +90,19 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const float* x, const floa
   const float* xr = x + (size_t)blockIdx.x * in_stride;
   float* yr = y + (size_t)blockIdx.x * out_stride;
   const float r = rms_scale(xr, dim, eps, red, lane, wave, 4u);
-  for (uint32_t i = tid; i < dim; i += 256u) {
-    const float v = xr[i] * r;
-    yr[i] = w ? v * w[i] : v;
+  for (uint32_t i0 = tid; i0 < dim; i0 += 4u * 256u) {  // four elements in flight per thread
+    float xv[4], wv[4];
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+      const uint32_t i = min(i0 + 256u * k, dim - 1u);
+      xv[k] = xr[i];
+      wv[k] = w ? w[i] : 1.f;
+    }
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+      const uint32_t i = i0 + 256u * k;
+      if (i < dim) { const float v = xv[k] * r; yr[i] = w ? v * wv[k] : v; }
+    }
   }
 }
 
@@ -93,9 +112,20 @@ __device__ __forceinline__ void stage_normed_x(const MvArgs& a, uint32_t* smem, 
                                                uint32_t nwaves) {
   float* red = (float*)(smem + a.norm_off);
   const float r = rms_scale(a.x, a.cols, a.eps, red, lane, wave, nwaves);
-  for (uint32_t i = tid; i < a.cols; i += nwaves * 64u) {
-    const float v = a.x[i] * r;
-    xs[i + (i >> 5) * 4u] = v * a.norm_w[i];
+  const uint32_t nt = nwaves * 64u;
+  for (uint32_t i0 = tid; i0 < a.cols; i0 += 4u * nt) {  // four elements in flight per thread
+    float xv[4], wv[4];
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+      const uint32_t i = min(i0 + nt * k, a.cols - 1u);
+      xv[k] = a.x[i];
+      wv[k] = a.norm_w[i];
+    }
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+      const uint32_t i = i0 + nt * k;
+      if (i < a.cols) { const float v = xv[k] * r; xs[i + (i >> 5) * 4u] = v * wv[k]; }
+    }
   }
   __syncthreads();
 }
