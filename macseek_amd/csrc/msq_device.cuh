@@ -219,6 +219,21 @@ __device__ __forceinline__ uint32_t group8_sel(uint32_t lane) {
   return s;
 }
 
+// Sum of n partial results p[0], p[stride], ... in that order. Eight are read before the first is added: read and
+// added one at a time, the loop is a chain of LDS latencies (28 of them per output row in the MoE down kernel).
+__device__ __forceinline__ float sum_in_order(const float* p, uint32_t n, uint32_t stride = 1) {
+  float s = 0.f;
+  for (uint32_t k0 = 0; k0 < n; k0 += 8u) {
+    float t[8];
+#pragma unroll
+    for (int j = 0; j < 8; j++) t[j] = p[min(k0 + j, n - 1u) * stride];
+#pragma unroll
+    for (int j = 0; j < 8; j++)
+      if (k0 + j < n) s += t[j];
+  }
+  return s;
+}
+
 // ------------------------------------------------------------------------------------------------ LDS table copies
 __device__ __forceinline__ void copy_words16(uint32_t* dst, const uint32_t* src, int nwords, int tid, int nthreads) {
   const uint4* s = (const uint4*)src;

@@ -152,8 +152,7 @@ __device__ __forceinline__ void moe_gu_run_direct(const MoeArgs& a, uint32_t* tb
     for (uint32_t q0 = 0; q0 < 2 * n; q0 += blockDim.x) {
       const uint32_t q = q0 + tid;
       float sum = 0.f;
-      if (q < 2 * n)
-        for (uint32_t k = 0; k < 4 * KS; k++) sum += part[q * PSTRIDE + k];
+      if (q < 2 * n) sum = sum_in_order(part + q * PSTRIDE, 4 * KS);
       const float other = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, sum), 0xB1, 0xF, 0xF, false));
       if (q < 2 * n && !(q & 1u)) {
         const uint32_t v = c0 + (q >> 1);
@@ -280,8 +279,7 @@ __device__ __forceinline__ void moe_gu_run_ring(const MoeArgs& a, uint32_t* tbl,
     for (uint32_t q0 = 0; q0 < 2 * n; q0 += blockDim.x) {
       const uint32_t q = q0 + tid;
       float sum = 0.f;
-      if (q < 2 * n)
-        for (uint32_t k = 0; k < 4 * KS; k++) sum += part[q * PSTRIDE + k];
+      if (q < 2 * n) sum = sum_in_order(part + q * PSTRIDE, 4 * KS);
       const float other = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, sum), 0xB1, 0xF, 0xF, false));
       if (q < 2 * n && !(q & 1u)) {
         const uint32_t v = c0 + (q >> 1);
@@ -500,8 +498,7 @@ __global__ __launch_bounds__(MAXT) void moe_down_kernel(const MoeArgs a) {
     }
     __syncthreads();
     for (uint32_t t = tid; t < n; t += blockDim.x) {
-      float s = 0.f;
-      for (uint32_t k = 0; k < slots; k++) s += part[t * PSTRIDE + k];
+      const float s = sum_in_order(part + t * PSTRIDE, slots);
       a.y[c0 + t] += s;
     }
     __syncthreads();

@@ -195,8 +195,7 @@ __global__ __launch_bounds__(1024) void mv_kernel(const MvArgs a) {
       if (tid < tile_rows) {
         const uint32_t row = tile_row0 + tid;
         if (row < a.rows) {
-          float s = 0.f;
-          for (uint32_t k = 0; k < KS; k++) s += part[tid * KS + k];
+          const float s = sum_in_order(part + tid * KS, KS);
           a.y[row] = a.accumulate ? a.y[row] + s : s;
         }
       }
@@ -296,8 +295,7 @@ __global__ __launch_bounds__(1024) void mv_ring_kernel(const MvArgs a) {
       if (tid < tile_rows) {
         const uint32_t row = tile_row0 + tid;
         if (row < a.rows) {
-          float sum = 0.f;
-          for (uint32_t k = 0; k < KS; k++) sum += part[tid * KS + k];
+          const float sum = sum_in_order(part + tid * KS, KS);
           a.y[row] = a.accumulate ? a.y[row] + sum : sum;
         }
       }
@@ -434,8 +432,7 @@ __global__ __launch_bounds__(512) void mv_tok_kernel(const MvTokArgs ta) {
     for (uint32_t idx = tid; idx < tile_rows * T; idx += blockDim.x) {
       const uint32_t r = idx % tile_rows, t = idx / tile_rows, row = tile_row0 + r;  // consecutive lanes: consecutive rows
       if (row < a.rows && t0 + t < ta.n) {
-        float s = 0.f;
-        for (uint32_t k = 0; k < 4 * KS; k++) s += part[(r * 4 * KS + k) * T + t];
+        const float s = sum_in_order(part + r * 4 * KS * T + t, 4 * KS, T);
         float* y = a.y + (size_t)(t0 + t) * ta.y_stride + row;
         *y = a.accumulate ? *y + s : s;
       }
