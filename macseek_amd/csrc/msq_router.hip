@@ -212,7 +212,7 @@ __global__ __launch_bounds__(256) void route_lists_kernel(const int* __restrict_
   const uint32_t lane = threadIdx.x & 63u;
   const int e = (int)(blockIdx.x * 4u + (threadIdx.x >> 6));
   if (e >= (int)n_exp) return;  // whole waves leave; no barrier follows
-  constexpr uint32_t U = 4;  // ids fetched per lane before they are used: the loop is bound by load latency otherwise
+  constexpr uint32_t U = 16;  // ids fetched per lane before they are used: the loop is bound by load latency otherwise
   uint32_t lt = 0, eq = 0;
   for (uint32_t i0 = 0; i0 < n_entries; i0 += 64u * U) {
     int id[U];
