@@ -421,6 +421,41 @@ def bench_stream(torch, args):
             "cpu_baseline": None, "pct_of_hbm_peak": 100 * best / HBM_PEAK_GBPS}
 
 
+def bench_issue_probe(torch, args):
+    """Instruction-issue probes (msq_issue_probe): ns per instruction group and SIMD for vector ops, matrix-core ops and
+    LDS reads, alone and interleaved, at 1, 2 and 4 waves per SIMD (one workgroup per CU) and 8 (two workgroups)."""
+    from macseek_amd import _lib
+    from macseek_amd import quant as q
+    L = _lib.load()
+    dev = torch.device("cuda:0")
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    sink = torch.zeros(4 * cus * 4, dtype=torch.uint8, device=dev)
+    sb = q.Buffer.of(sink).c()
+    VALU, MFMA16, MFMA4, MFMA8, LDS = 1, 2, 4, 8, 16
+    mixes = [("valu32", VALU), ("mfma16_f16_x8", MFMA16), ("mfma_fp4_fp6_x8", MFMA4), ("mfma_fp8_x8", MFMA8), ("lds_b32_x16", LDS),
+             ("valu32+mfma16_f16_x8", VALU | MFMA16), ("valu32+mfma_fp4_fp6_x8", VALU | MFMA4), ("valu32+lds_b32_x16", VALU | LDS),
+             ("valu32+lds_b32_x16+mfma_fp4_fp6_x8", VALU | LDS | MFMA4)]
+    iters = 4096
+    rows = []
+    for wps, grid, block in ((1, cus, 256), (2, cus, 512), (4, cus, 1024), (8, 2 * cus, 1024)):
+        row = {"waves_per_simd": wps}
+        for name, mask in mixes:
+            def launch(i):
+                rc = L.msq_issue_probe(C.c_void_p(torch.cuda.current_stream().cuda_stream), mask, grid, block, iters, C.byref(sb))
+                if rc != 0:
+                    raise RuntimeError(L.msq_last_error().decode())
+            ms = graph_ms_per_launch(torch, launch, 3)
+            # one iteration of one wave = one group set; a SIMD runs wps waves: ns per group set and SIMD
+            row[name] = round(ms * 1e6 / iters / wps, 2)
+        rows.append(row)
+    v = rows[2]["valu32"] / 32.0
+    return {"value": 0.0, "ms_per_step": 0.0, "dtype": "instruction issue",
+            "config": {"workload": "issue probes: ns per SIMD for one group set of a wave (valu32 = 32 vector ops, mfma*_x8 = 8 matrix ops, "
+                                   "lds_b32_x16 = 16 random ds_read_b32 + 16 v_xor), by waves per SIMD", "rows": rows,
+                       "ns_per_valu_issue_at_4_waves": round(v, 3)},
+            "roofline": None, "cpu_baseline": None, "pct_of_hbm_peak": None}
+
+
 def bench_copy_calibration(torch, args):
     """A device-to-device copy of known size (1 GiB read, 1 GiB written per launch): the reference that the FETCH_SIZE /
     WRITE_SIZE counters of a profiling run are scaled by."""
@@ -619,7 +654,7 @@ def main():
     ap.add_argument("--steps", type=int, default=500)
     ap.add_argument("--warmup", type=int, default=100)
     ap.add_argument("--workload", default="moe_decode",
-                    choices=["moe_decode", "moe_prefill", "matvec_iq1s", "matvec_iq2xxs", "q8_0", "matvec_n", "router", "matmul", "stream", "copy_calibration"])
+                    choices=["moe_decode", "moe_prefill", "matvec_iq1s", "matvec_iq2xxs", "q8_0", "matvec_n", "router", "matmul", "stream", "copy_calibration", "issue_probe"])
     ap.add_argument("--gpu-only", action="store_true",
                     help="profiling runs: skip the CPU baseline leg and the prefill appendix of the default workload")
     args = ap.parse_args()
@@ -657,6 +692,8 @@ def main():
         r = bench_stream(torch, args)
     elif args.workload == "copy_calibration":
         r = bench_copy_calibration(torch, args)
+    elif args.workload == "issue_probe":
+        r = bench_issue_probe(torch, args)
     elif args.workload == "router":
         r = bench_router(torch, args)
     elif args.workload == "matvec_n":
