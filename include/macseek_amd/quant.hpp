@@ -130,6 +130,12 @@ inline void encode_moe_decode_table(Enc& e, const MoeDecodeArgs& a, const Buffer
   const MsqBuffer t = table.c();
   detail::check(msq_moe_decode_table(e.stream, &c, &t));
 }
+// no reference counterpart: the same layer with the h scratch in the library's static device array (nothing is
+// allocated, a.scratch is ignored, inter <= msq_moe_decode_static_max_inter())
+inline void encode_moe_decode_static(Enc& e, const MoeDecodeArgs& a) {
+  const MsqMoeDecodeArgs c = a.c();
+  detail::check(msq_moe_decode_static(e.stream, &c));
+}
 enum class MoePart { All, SharedGu, AfterSharedGu, Shared, Routed, SharedDown };  // reference: quant.hpp:85
 inline void encode_moe_decode_table_part(Enc& e, const MoeDecodeArgs& a, const Buffer& table, MoePart part) {
   const MsqMoeDecodeArgs c = a.c();

@@ -198,6 +198,15 @@ int msq_moe_decode_table(void* stream, const MsqMoeDecodeArgs* a, const MsqBuffe
  * SHARED_DOWN never read `table` (it may be NULL for them). */
 int msq_moe_decode_table_part(void* stream, const MsqMoeDecodeArgs* a, const MsqBuffer* table, int part);
 
+/* No counterpart in the reference. msq_moe_decode for callers that cannot allocate device memory (code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc): `a->scratch` is ignored, the h rows live in a
+ * device array inside the library (7 x 4096 floats = 112 KiB per GPU, held until the process ends), and the call
+ * allocates nothing. inter above msq_moe_decode_static_max_inter() (4096) is refused with MSQ_ERR_SCRATCH. Every call
+ * on a GPU uses that GPU's one array: calls that overlap on one GPU (two streams) race; calls on one stream do not.
+ * Results are bit-identical to msq_moe_decode with caller scratch. */
+int msq_moe_decode_static(void* stream, const MsqMoeDecodeArgs* a);
+int msq_moe_decode_static_max_inter(void);
+
 /* ---------------------------------------------------------------------------------------------- MoE, prefill */
 
 /* reference: ms::q::MoePrefillArgs (quant.hpp:93-116), field for field, plus dim / inter / x_is_bf16.

@@ -81,6 +81,8 @@ SIGNATURES = {
     "msq_moe_decode": (C.c_int, [C.c_void_p, C.POINTER(MsqMoeDecodeArgs)]),
     "msq_moe_decode_table": (C.c_int, [C.c_void_p, C.POINTER(MsqMoeDecodeArgs), _BP]),
     "msq_moe_decode_table_part": (C.c_int, [C.c_void_p, C.POINTER(MsqMoeDecodeArgs), _BP, C.c_int]),
+    "msq_moe_decode_static": (C.c_int, [C.c_void_p, C.POINTER(MsqMoeDecodeArgs)]),
+    "msq_moe_decode_static_max_inter": (C.c_int, []),
     "msq_moe_prefill_scratch_bytes": (C.c_size_t, [C.c_int, C.c_int, C.c_int, C.c_int, C.c_int]),
     "msq_moe_prefill": (C.c_int, [C.c_void_p, C.POINTER(MsqMoePrefillArgs)]),
     "msq_router_topk": (C.c_int, [C.c_void_p, _BP, _BP, _BP, _BP, C.c_int, C.c_int, C.c_float]),

@@ -50,6 +50,9 @@ inline bool buf_ok(const MsqBuffer* b, size_t need) { return b && b->dev && b->s
 struct DeviceInfo { int ok, cus; };
 const DeviceInfo& device_info();  // cached facts of the current device (CU count, gfx950 check)
 
+// looks up this device's copy of the static MoE scratch (msq_moe.hip); called by msq_init() and by the entry point
+int static_scratch_setup(float** out);
+
 // small-N matvec through the dot-product kernels (msq_matvec.hip); MSQ_ERR_UNSUPPORTED, without a message, when the
 // shape does not fit them
 int matvec_tok(hipStream_t st, int t, const uint8_t* W, int rows, int cols, const float* X, float* Y, int n, int accumulate,

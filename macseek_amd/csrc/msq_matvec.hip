@@ -278,7 +278,7 @@ int msq_init(void) {
   g_err[0] = 0;
   const DeviceInfo& d = device_info();
   if (!d.ok) return fail(MSQ_ERR_HIP, "macseek quant: no gfx950 device is current");
-  return MSQ_OK;
+  return static_scratch_setup(nullptr);
 }
 const char* msq_last_error(void) { return g_err; }
 int msq_device_ok(void) { return device_info().ok; }

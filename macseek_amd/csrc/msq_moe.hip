@@ -1,11 +1,38 @@
 // C ABI: fused one-token MoE layer (see include/msq.h; reference host code src/kernels/quant.mm:252-369).
 #include <algorithm>
 #include <cstdlib>
+#include <mutex>
 
 #include "msq_host.h"
 #include "msq_moe.cuh"
 
 namespace msq {
+
+// ---- msq_moe_decode_static: the h scratch of the one-token layer in memory the library's code object carries, for
+// callers that cannot allocate. Every device that loads the library holds its own copy of the array; host code never
+// uses the array's name as an address (it is only a handle for hipGetSymbolAddress), but the per-device pointer that
+// static_scratch_setup() looks up once, with that device current.
+constexpr int kStaticMaxInter = 4096;  // largest expert intermediate size the static scratch serves
+static __device__ __align__(256) float g_moe_static_scratch[(kMaxRouted + 1) * kStaticMaxInter];
+constexpr int kStaticMaxDevices = 64;
+static float* g_static_ptr[kStaticMaxDevices];
+static std::mutex g_static_mu;
+
+int static_scratch_setup(float** out) {
+  int dev = 0;
+  MSQ_HIP(hipGetDevice(&dev));
+  if (dev < 0 || dev >= kStaticMaxDevices) return fail(MSQ_ERR_ARGUMENT, "macseek quant: device ordinal %d is beyond the static scratch table", dev);
+  std::lock_guard<std::mutex> lock(g_static_mu);
+  if (!g_static_ptr[dev]) {
+    void* p = nullptr;
+    MSQ_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(g_moe_static_scratch)));
+    if (!p) return fail(MSQ_ERR_HIP, "macseek quant: hipGetSymbolAddress returned no address for the static MoE scratch");
+    g_static_ptr[dev] = (float*)p;
+  }
+  if (out) *out = g_static_ptr[dev];
+  return MSQ_OK;
+}
+
 namespace {
 
 bool routed_type_ok(int t) { return t == MSQ_IQ1_S || t == MSQ_IQ2_XXS; }
@@ -201,6 +228,21 @@ int msq_moe_decode_table(void* stream, const MsqMoeDecodeArgs* a, const MsqBuffe
 }
 int msq_moe_decode_table_part(void* stream, const MsqMoeDecodeArgs* a, const MsqBuffer* table, int part) {
   return moe_decode_impl((hipStream_t)stream, a, table, part, true);
+}
+int msq_moe_decode_static_max_inter(void) { return kStaticMaxInter; }
+int msq_moe_decode_static(void* stream, const MsqMoeDecodeArgs* a) {
+  if (!a) return fail(MSQ_ERR_ARGUMENT, "macseek quant: moe_decode_static: null arguments");
+  const int inter = a->inter ? a->inter : MSQ_EXPERT_INTER;
+  if (inter > kStaticMaxInter)
+    return fail(MSQ_ERR_SCRATCH, "macseek quant: moe_decode_static: inter %d exceeds the static scratch limit of %d; use msq_moe_decode "
+                "with caller scratch", inter, kStaticMaxInter);
+  float* h = nullptr;
+  if (const int rc = static_scratch_setup(&h)) return rc;
+  MsqMoeDecodeArgs b = *a;
+  b.scratch.dev = h;
+  b.scratch.off = 0;
+  b.scratch.size = sizeof(float) * (size_t)(kMaxRouted + 1) * kStaticMaxInter;
+  return moe_decode_impl((hipStream_t)stream, &b, nullptr, MSQ_PART_ALL, false);
 }
 
 }  // extern "C"

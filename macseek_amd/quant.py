@@ -213,6 +213,16 @@ def encode_moe_decode_table_part(e, a, table, part):  # reference: quant.hpp:79-
     _check(_lib.load().msq_moe_decode_table_part(e.handle, C.byref(a.c()), _bp(table), int(part)))
 
 
+def encode_moe_decode_static(e, a):
+    """encode_moe_decode without caller scratch (no reference counterpart): h lives in the library's static device
+    array, nothing is allocated; a.scratch is ignored. inter <= moe_decode_static_max_inter()."""
+    _check(_lib.load().msq_moe_decode_static(e.handle, C.byref(a.c())))
+
+
+def moe_decode_static_max_inter():
+    return _lib.load().msq_moe_decode_static_max_inter()
+
+
 # ---------------------------------------------------------------------------------------------- MoE, prefill
 class MoePrefillArgs:
     """reference: ms::q::MoePrefillArgs (quant.hpp:93-116) plus dim / inter / x_is_bf16. `slots` is a list of
