@@ -431,10 +431,10 @@ def bench_issue_probe(torch, args):
     cus = torch.cuda.get_device_properties(0).multi_processor_count
     sink = torch.zeros(4 * cus * 4, dtype=torch.uint8, device=dev)
     sb = q.Buffer.of(sink).c()
-    VALU, MFMA16, MFMA4, MFMA8, LDS = 1, 2, 4, 8, 16
+    VALU, MFMA16, MFMA4, MFMA8, LDS, VINT = 1, 2, 4, 8, 16, 32
     mixes = [("valu32", VALU), ("mfma16_f16_x8", MFMA16), ("mfma_fp4_fp6_x8", MFMA4), ("mfma_fp8_x8", MFMA8), ("lds_b32_x16", LDS),
              ("valu32+mfma16_f16_x8", VALU | MFMA16), ("valu32+mfma_fp4_fp6_x8", VALU | MFMA4), ("valu32+lds_b32_x16", VALU | LDS),
-             ("valu32+lds_b32_x16+mfma_fp4_fp6_x8", VALU | LDS | MFMA4)]
+             ("valu32+lds_b32_x16+mfma_fp4_fp6_x8", VALU | LDS | MFMA4), ("vint32", VINT), ("vint32+mfma16_f16_x8", VINT | MFMA16)]
     iters = 4096
     rows = []
     for wps, grid, block in ((1, cus, 256), (2, cus, 512), (4, cus, 1024), (8, 2 * cus, 1024)):

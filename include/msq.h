@@ -134,8 +134,8 @@ int msq_bw_probe(void* stream, const MsqBuffer* src, size_t bytes, const MsqBuff
 /* Instruction-issue probe (no reference counterpart; the reference prices its kernels against a bandwidth probe only):
  * `grid` workgroups of `block` threads each run `iters` iterations of a fixed instruction group per wave. `mask` ORs
  * the groups: 1 = 32 vector ops, 2 = 8 fp16 16x16x32 matrix ops, 4 = 8 block-scaled fp4 x fp6 16x16x128 matrix ops,
- * 8 = 8 fp8 16x16x128 matrix ops, 16 = 16 random 32-bit LDS reads; supported mixes: 1, 2, 4, 8, 16, 1|2, 1|4, 1|16,
- * 1|4|16. `sink` holds >= 4 * grid bytes. The benchmark turns the timings into ns per issue slot. */
+ * 8 = 8 fp8 16x16x128 matrix ops, 16 = 16 random 32-bit LDS reads, 32 = 32 integer vector ops; supported mixes: 1, 2,
+ * 4, 8, 16, 32, 1|2, 1|4, 1|16, 1|4|16, 32|2. `sink` holds >= 4 * grid bytes. The benchmark turns the timings into ns per issue slot. */
 int msq_issue_probe(void* stream, int mask, int grid, int block, int iters, const MsqBuffer* sink);
 
 /* ---------------------------------------------------------------------------------------------- MoE, one token */

@@ -12,9 +12,25 @@
 // LDS; a workgroup synchronises only once per chunk of rows, to add the K-split / per-expert partials in a fixed
 // order and run the epilogue.
 #pragma once
+#include <type_traits>
+
 #include "msq_device.cuh"
+#include "msq_iq1s.cuh"
 
 namespace msq {
+
+#ifdef MSQ_EXP_NOLOOP  // experiment builds: the row loops never run, what remains is the launch's fixed cost
+#define MSQ_EXP_LOOP_COND && a_never
+#else
+#define MSQ_EXP_LOOP_COND
+#endif
+
+#ifdef MSQ_EXP_TIMELINE  // experiment builds: wall-clock stamps (100 MHz) per workgroup, wave and point
+__device__ uint64_t g_timeline[512 * 16 * 8];
+#define MSQ_TL(k) do { if ((threadIdx.x & 63u) == 0 && blockIdx.x < 512u) g_timeline[(blockIdx.x * 16u + (threadIdx.x >> 6)) * 8u + (k)] = wall_clock64(); } while (0)
+#else
+#define MSQ_TL(k) do {} while (0)
+#endif
 
 constexpr int kMaxRouted = 6;
 constexpr int kMoeChunkRows = 128;  // rows a workgroup finishes between two synchronisations
@@ -54,6 +70,26 @@ template <class D>
 constexpr int rows_in_flight(int matrices) {
   const int words = (int)(sizeof(typename D::Raw) / 4) * matrices;
   return words <= 6 ? 4 : words <= 12 ? 2 : 1;
+}
+
+// 32-bit words of LDS that the staged activations of a row of `cols` columns take for decoder D
+template <class D>
+__host__ __device__ constexpr uint32_t x_stage_words(uint32_t cols) {
+  if constexpr (requires { D::QUANT_X; }) return xq_words(cols);
+  else return xlds_words(cols);
+}
+// the lane's activation slice of unit u from a staged row (at word offset `at` of `base`), or from device memory
+template <class D>
+__device__ __forceinline__ typename D::X load_x_staged(const uint32_t* base, uint32_t u) {
+  if constexpr (requires { D::QUANT_X; }) return D::load_x(XQLds{base}, u);
+  else return D::load_x(XLds{(const float*)base}, u);
+}
+
+// Entry i of the expert address table, read through the scalar cache (the index is wave-uniform): one request per wave
+// instead of one per lane, and its result does not queue behind the vector loads in flight.
+__device__ __forceinline__ const void* table_entry(const uint64_t* table, uint32_t i) {
+  typedef const __attribute__((address_space(4))) uint64_t* cptr_t;
+  return (const void*)((cptr_t)(uintptr_t)table)[i];
 }
 
 __device__ __forceinline__ uint32_t uniform(uint32_t v) { return (uint32_t)__builtin_amdgcn_readfirstlane((int)v); }
@@ -195,6 +231,14 @@ __device__ __forceinline__ void moe_gu_run_ring(const MoeArgs& a, uint32_t* tbl,
 
   typename D::X xr;
   bool first = true;
+  // The loads of the prologue (grid items, activations) need nothing but kernel arguments: they are requested before
+  // the expert addresses are looked up, and stored to LDS after the first weight rows have been requested.
+  [[maybe_unused]] DecIQ1SQ::TblRegs tr;
+  [[maybe_unused]] XqBatch<2> xb;
+  if constexpr (requires { D::QUANT_X; }) {
+    tr = D::issue_tables(tid, blockDim.x);
+    if (a.stage_x) xb = xq_issue<2>(a.x, a.dim >> 2, tid, blockDim.x);
+  }
   for (uint32_t c0 = wg_begin; c0 < wg_end; c0 += kMoeChunkRows) {
     const uint32_t c1 = min(wg_end, c0 + kMoeChunkRows), n = c1 - c0;
     const uint32_t run = uniform((n + RW - 1) / RW);  // divisions run on the vector unit: bring the results back
@@ -205,7 +249,7 @@ __device__ __forceinline__ void moe_gu_run_ring(const MoeArgs& a, uint32_t* tbl,
     const void *pg = nullptr, *pu = nullptr;
     auto set_expert = [&]() {
       if (shared) { pg = a.sgate; pu = a.sup; }
-      else if (a.table) { pg = (const void*)a.table[3 * pe]; pu = (const void*)a.table[3 * pe + 1]; }
+      else if (a.table) { pg = table_entry(a.table, 3 * pe); pu = table_entry(a.table, 3 * pe + 1); }
       else { pg = a.gate[pe]; pu = a.up[pe]; }
       pg = uniform(pg); pu = uniform(pu);  // buffer descriptors live in scalar registers
     };
@@ -217,30 +261,102 @@ __device__ __forceinline__ void moe_gu_run_ring(const MoeArgs& a, uint32_t* tbl,
     auto fetch = [&](int s) {  // loads of row pair pv into slot s (nothing is read once pv has passed w1), then advance
       const uint32_t bytes = pv < w1 ? mat_bytes : 0u;
       const uint32_t soff = pr * row_bytes;
+#ifdef MSQ_EXP_NOLOAD
+      if (pv < w0 + NR) {
+#endif
       rg[s] = D::fetch(make_rsrc(pg, bytes), off, soff);
       ru[s] = D::fetch(make_rsrc(pu, bytes), off, soff);
+#ifdef MSQ_EXP_NOLOAD
+      } else { asm volatile("" : "+v"(*(uint32_t*)&rg[s]), "+v"(*(uint32_t*)&ru[s])); }
+#endif
       pv++; pr++;
       if (!shared && pr == a.inter && pv < w1) { pr = 0; pe++; set_expert(); }
     };
+    if (first) MSQ_TL(1);
 #pragma unroll
     for (int s = 0; s < NR; s++) fetch(s);
     if (first) {  // tables and activations arrive while the first weight rows are in flight
-      const CopyJob jobs[3] = {tbl_job_of<D>(0, 0u, true), tbl_job_of<D>(1, 0u, true),
-                               {(const uint4*)a.x, (uint32_t)(smem - tbl) + a.xs_off, a.stage_x ? a.dim / 4u : 0u, true}};
-      copy_jobs<4>(tbl, jobs, tid, blockDim.x);
-      if (a.stage_x) {
-        __syncthreads();
-        xr = D::load_x(XLds{(const float*)(smem + a.xs_off)}, unit);
+      MSQ_TL(2);
+      if constexpr (requires { D::QUANT_X; }) {
+        if (a.stage_x) {
+          D::finish_tables(tbl, tr, tid, blockDim.x);
+          MSQ_TL(3);
+          stage_xq<2>(smem + a.xs_off, a.x, a.dim, tid, blockDim.x, &xb);
+          __syncthreads();
+          xr = D::load_x(XQLds{smem + a.xs_off}, unit);
+        } else {
+          D::finish_tables(tbl, tr, tid, blockDim.x);
+          xr = D::load_x(a.x, unit);
+          __syncthreads();
+        }
       } else {
-        xr = D::load_x(a.x, unit);
-        __syncthreads();
+        const CopyJob jobs[3] = {tbl_job_of<D>(0, 0u, true), tbl_job_of<D>(1, 0u, true),
+                                 {(const uint4*)a.x, (uint32_t)(smem - tbl) + a.xs_off, a.stage_x ? a.dim / 4u : 0u, true}};
+        copy_jobs<4>(tbl, jobs, tid, blockDim.x);
+        if (a.stage_x) {
+          __syncthreads();
+          xr = D::load_x(XLds{(const float*)(smem + a.xs_off)}, unit);
+        } else {
+          xr = D::load_x(a.x, unit);
+          __syncthreads();
+        }
       }
       if (!valid) xr = typename D::X{};
       first = false;
+      MSQ_TL(4);
     }
+    if constexpr (requires { D::HAS_PRE; }) {
+      // Three steps per unit (gate of a row pair, then up): table reads of the unit two places ahead, entry reads of
+      // the next unit, arithmetic of this one. Units past the end of the run decode the zeros that their empty buffer
+      // descriptors returned (every address stays inside the tables, and a zero block scale makes the result zero).
+      static_assert(NS == 1 && NR % 2 == 0, "unit pipeline: one stage per unit, buffers alternate gate / up");
+      const uint32_t lanec = (lane & 1u) * 0x80808080u;
+      typename D::Pre pa[2];
+      typename D::Look lk[2];
+      pa[0] = D::pre(rg[0], tbl);
+      pa[1] = D::pre(ru[0], tbl);
+      D::lookup(rg[0], pa[0], tbl, lanec, lk[0]);
+      [[maybe_unused]] const bool a_never = a.dim == 1u;
+      for (uint32_t r0 = w0; r0 < w1 MSQ_EXP_LOOP_COND; r0 += NR) {
+#pragma unroll
+        for (int half = 0; half < 2; half++) {
+          float acc[NR];  // value 2 j + m: row pair j of this half, m = 0 gate, 1 up
+#pragma unroll
+          for (int j = 0; j < NR / 2; j++) {
+            const int s = half * (NR / 2) + j, sn = (s + 1) % NR;
+            // table reads first: a result is then waited for a whole unit after its request
+            // (scheduling barriers: left alone, the compiler moves a unit's entry reads next to their use)
+            pa[0] = D::pre(rg[sn], tbl);
+            D::lookup(ru[s], pa[1], tbl, lanec, lk[1]);
+            __builtin_amdgcn_sched_barrier(0);
+            float g = D::partial(rg[s], lk[0], xr);
+            __builtin_amdgcn_sched_barrier(0);
+            pa[1] = D::pre(ru[sn], tbl);
+            D::lookup(rg[sn], pa[0], tbl, lanec, lk[0]);
+            __builtin_amdgcn_sched_barrier(0);
+            float u = D::partial(ru[s], lk[1], xr);
+            __builtin_amdgcn_sched_barrier(0);
+            acc[2 * j] = g;
+            acc[2 * j + 1] = u;
+#ifndef MSQ_EXP_NOFETCH
+            fetch(s);  // the slot is free again: fetch the row pair NR places ahead
+#else
+            asm volatile("" : "+v"(rg[s].qs), "+v"(ru[s].qs));
+#endif
+          }
+          const uint32_t rb = r0 + half * (NR / 2);
+          if (rb < w1) {
+            row16_fold<NR>(acc, lane);
+            const uint32_t k = group8_sel<NR>(lane), j = k >> 1, m = k & 1u;
+            if (!(lane & 8u) && rb + j < w1) part[((rb + j - c0) * 2 + m) * PSTRIDE + ks * 4 + (lane >> 4)] = acc[0];
+          }
+        }
+      }
+    } else {
     typename D::Look lk[2];  // stage t of a row pair uses lk[t & 1]; 2 NS stages per row pair keep the parity fixed
     if (w0 < w1) lk[0] = D::lookup(rg[0], 0, tbl);
-    for (uint32_t r0 = w0; r0 < w1; r0 += NR) {
+    [[maybe_unused]] const bool a_never = a.dim == 1u;
+    for (uint32_t r0 = w0; r0 < w1 MSQ_EXP_LOOP_COND; r0 += NR) {
 #pragma unroll
       for (int half = 0; half < 2; half++) {
         float acc[NR];  // value 2 j + m: row pair j of this half, m = 0 gate, 1 up
@@ -274,7 +390,10 @@ __device__ __forceinline__ void moe_gu_run_ring(const MoeArgs& a, uint32_t* tbl,
         }
       }
     }
+    }
+    MSQ_TL(5);
     __syncthreads();
+    MSQ_TL(6);
     // thread q sums the partials of (row q / 2, matrix q % 2); gate and up then meet in the even lane
     for (uint32_t q0 = 0; q0 < 2 * n; q0 += blockDim.x) {
       const uint32_t q = q0 + tid;
@@ -289,6 +408,7 @@ __device__ __forceinline__ void moe_gu_run_ring(const MoeArgs& a, uint32_t* tbl,
       }
     }
     __syncthreads();
+    MSQ_TL(7);
   }
 }
 
@@ -306,6 +426,7 @@ __global__ __launch_bounds__(1024) void moe_gu_kernel(const MoeArgs a) {
   constexpr int TBL = DR::LDS_WORDS > DS::LDS_WORDS ? DR::LDS_WORDS : DS::LDS_WORDS;
   __shared__ __attribute__((aligned(16))) uint32_t tbl[TBL > 0 ? TBL : 4];
   extern __shared__ __attribute__((aligned(16))) uint32_t smem[];
+  MSQ_TL(0);
   if (blockIdx.x < a.grid_routed) moe_gu_run<DR>(a, tbl, smem, false, blockIdx.x);
   else moe_gu_run<DS>(a, tbl, smem, true, blockIdx.x - a.grid_routed);
 }
@@ -385,7 +506,7 @@ __global__ __launch_bounds__(MAXT) void moe_down_kernel(const MoeArgs a) {
   const bool valid_r = NE && u0 < units_r, valid_s = a.run_shared && u0 < units_s;
   const uint32_t unit_r = u0 < units_r ? u0 : units_r - 1, unit_s = u0 < units_s ? u0 : units_s - 1;
   const void* Dr_ = nullptr;
-  if (NE) Dr_ = uniform(a.table ? (const void*)a.table[3 * e + 2] : (const void*)a.down[e]);
+  if (NE) Dr_ = uniform(a.table ? table_entry(a.table, 3 * e + 2) : (const void*)a.down[e]);
   const gptr_t Dr = as_global(Dr_), Dsh = as_global(a.sdown);
 
   const auto off_r = [&] { if constexpr (RING_R) return DR::offsets(unit_r); else return 0; }();

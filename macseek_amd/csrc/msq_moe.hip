@@ -2,9 +2,13 @@
 #include <algorithm>
 #include <cstdlib>
 #include <mutex>
+#include <type_traits>
 
 #include "msq_host.h"
 #include "msq_moe.cuh"
+#ifdef MSQ_EXP_OLDDEC
+#define DecIQ1SQ DecIQ1S
+#endif
 
 namespace msq {
 
@@ -58,42 +62,50 @@ int env_int(const char* name, int dflt) {
   const char* v = getenv(name);
   return v && *v ? atoi(v) : dflt;
 }
-template <class DR>
-size_t lds_words_for_shared(int ts, bool down) {
-  size_t s = 0;
-  switch (ts) {
-    case MSQ_IQ2_XXS: s = DecIQ2XXS::LDS_WORDS; break;
-    case MSQ_IQ1_S: s = DecIQ1S::LDS_WORDS; break;
-    default: s = 0;
-  }
-  return down ? DR::LDS_WORDS + s : std::max<size_t>(DR::LDS_WORDS, s);
-}
-// the staged activations follow the partial sums in dynamic LDS when everything (with the kernel's static table) fits
-// the CU's LDS
-size_t place_x(MoeArgs& a, size_t lds, uint32_t x_cols, size_t static_lds) {
-  const size_t at = (lds + 15) / 16 * 16, end = at + (size_t)xlds_words(x_cols) * 4;
+// The staged activations follow the partial sums in dynamic LDS when everything (with the kernel's static tables) fits
+// the CU's LDS. gate/up: x in the routed decoder's form for the routed workgroups, in the shared decoder's form for
+// the others (one region, sized for the larger); down: the routed h rows in DR's form, then the shared row in DS's.
+template <class DR, class DS, bool DOWN>
+size_t place_x(MoeArgs& a, size_t lds, uint32_t cols_r, uint32_t cols_s) {
+  const size_t static_lds = 4 * (size_t)(DOWN ? DR::LDS_WORDS + DS::LDS_WORDS
+                                              : std::max<int>(DR::LDS_WORDS, DS::LDS_WORDS));
+  const size_t wr = cols_r ? x_stage_words<DR>(cols_r) : 0, ws = cols_s ? x_stage_words<DS>(cols_s) : 0;
+  const size_t words = DOWN ? wr + ws : std::max(wr, ws);
+  const size_t at = (lds + 15) / 16 * 16, end = at + words * 4;
   a.xs_off = (uint32_t)(at / 4);
   a.stage_x = end + static_lds + 64 <= (size_t)kMaxLds ? 1u : 0u;
   return a.stage_x ? end : lds;
 }
-// dispatch over (routed type, shared type)
+// The down kernel (rows of `inter` columns: one wave per row, a dozen rows per wave and launch) keeps the fp16 form of
+// the IQ1_S decoder: the integer form's larger tables and activation quantization cost its prologue more than its
+// shorter decode saves there.
+template <class D> struct DownDec { using T = D; };
+template <> struct DownDec<DecIQ1SQ> { using T = DecIQ1S; };
+// dispatch over (routed type, shared type); cols_r / cols_s: activations the routed / shared part stages (0 = none)
 template <bool DOWN>
-size_t dispatch(int tr, int ts, dim3 g, dim3 b, size_t part_bytes, uint32_t x_cols, hipStream_t st, MoeArgs& a) {
+size_t dispatch(int tr, int ts, dim3 g, dim3 b, size_t part_bytes, uint32_t cols_r, uint32_t cols_s, hipStream_t st, MoeArgs& a) {
 #define MSQ_MOE_CASE(TR, DRT, TS, DST)                                                            \
   if (tr == TR && ts == TS) {                                                                     \
-    const size_t tbl = 4 * lds_words_for_shared<DRT>(ts, DOWN);  /* static LDS of the kernel */    \
-    const size_t lds = place_x(a, part_bytes, x_cols, tbl);                                       \
-    if (DOWN) launch_down_t<DRT, DST>(g, b, lds, st, a); else launch_gu_t<DRT, DST>(g, b, lds, st, a); \
-    return lds;                                                                                   \
+    if constexpr (DOWN) {                                                                         \
+      using R = typename DownDec<DRT>::T;                                                         \
+      using S = typename DownDec<DST>::T;                                                         \
+      const size_t lds = place_x<R, S, true>(a, part_bytes, cols_r, cols_s);                      \
+      launch_down_t<R, S>(g, b, lds, st, a);                                                      \
+      return lds;                                                                                 \
+    } else {                                                                                      \
+      const size_t lds = place_x<DRT, DST, false>(a, part_bytes, cols_r, cols_s);                 \
+      launch_gu_t<DRT, DST>(g, b, lds, st, a);                                                    \
+      return lds;                                                                                 \
+    }                                                                                             \
   }
-  MSQ_MOE_CASE(MSQ_IQ1_S, DecIQ1S, MSQ_Q6_K, DecQ6K)
-  MSQ_MOE_CASE(MSQ_IQ1_S, DecIQ1S, MSQ_Q8_0, DecQ8_0)
-  MSQ_MOE_CASE(MSQ_IQ1_S, DecIQ1S, MSQ_IQ2_XXS, DecIQ2XXS)
-  MSQ_MOE_CASE(MSQ_IQ1_S, DecIQ1S, MSQ_IQ1_S, DecIQ1S)
+  MSQ_MOE_CASE(MSQ_IQ1_S, DecIQ1SQ, MSQ_Q6_K, DecQ6K)
+  MSQ_MOE_CASE(MSQ_IQ1_S, DecIQ1SQ, MSQ_Q8_0, DecQ8_0)
+  MSQ_MOE_CASE(MSQ_IQ1_S, DecIQ1SQ, MSQ_IQ2_XXS, DecIQ2XXS)
+  MSQ_MOE_CASE(MSQ_IQ1_S, DecIQ1SQ, MSQ_IQ1_S, DecIQ1SQ)
   MSQ_MOE_CASE(MSQ_IQ2_XXS, DecIQ2XXS, MSQ_Q6_K, DecQ6K)
   MSQ_MOE_CASE(MSQ_IQ2_XXS, DecIQ2XXS, MSQ_Q8_0, DecQ8_0)
   MSQ_MOE_CASE(MSQ_IQ2_XXS, DecIQ2XXS, MSQ_IQ2_XXS, DecIQ2XXS)
-  MSQ_MOE_CASE(MSQ_IQ2_XXS, DecIQ2XXS, MSQ_IQ1_S, DecIQ1S)
+  MSQ_MOE_CASE(MSQ_IQ2_XXS, DecIQ2XXS, MSQ_IQ1_S, DecIQ1SQ)
 #undef MSQ_MOE_CASE
   return 0;
 }
@@ -181,7 +193,8 @@ int moe_decode_impl(hipStream_t st, const MsqMoeDecodeArgs* p, const MsqBuffer* 
     if (g_r) { a.rows_per_wg_r = (uint32_t)((rows_r + g_r - 1) / g_r); g_r = (rows_r + a.rows_per_wg_r - 1) / a.rows_per_wg_r; }
     if (g_s) { a.rows_per_wg_s = (uint32_t)((rows_s + g_s - 1) / g_s); g_s = (rows_s + a.rows_per_wg_s - 1) / a.rows_per_wg_s; }
     a.grid_routed = (uint32_t)g_r;
-    if (!dispatch<false>(p->t_gate_up, ts, dim3((unsigned)(g_r + g_s)), dim3(threads), part_bytes, (uint32_t)dim, st, a))
+    if (!dispatch<false>(p->t_gate_up, ts, dim3((unsigned)(g_r + g_s)), dim3(threads), part_bytes, g_r ? (uint32_t)dim : 0u,
+                         g_s ? (uint32_t)dim : 0u, st, a))
       return unsupported("moe_decode type combo", p->t_gate_up, 0, 0);
     MSQ_HIP(hipGetLastError());
   }
@@ -203,7 +216,8 @@ int moe_decode_impl(hipStream_t st, const MsqMoeDecodeArgs* p, const MsqBuffer* 
     const long total = std::max<long>(1, (long)cus * std::max(1, env_d_wgs));
     a.rows_per_wg = (uint32_t)((dim + total - 1) / total);
     const long grid = (dim + a.rows_per_wg - 1) / a.rows_per_wg;
-    if (!dispatch<true>(p->t_down, ts, dim3((unsigned)grid), dim3(threads), part_bytes, (uint32_t)(((run_d_r ? nr : 0) + (d_s ? 1 : 0)) * inter), st, a))
+    if (!dispatch<true>(p->t_down, ts, dim3((unsigned)grid), dim3(threads), part_bytes, (uint32_t)((run_d_r ? nr : 0) * inter),
+                        d_s ? (uint32_t)inter : 0u, st, a))
       return unsupported("moe_decode type combo", p->t_down, 0, 0);
     MSQ_HIP(hipGetLastError());
   }
@@ -214,6 +228,12 @@ int moe_decode_impl(hipStream_t st, const MsqMoeDecodeArgs* p, const MsqBuffer* 
 }  // namespace msq
 
 using namespace msq;
+
+#ifdef MSQ_EXP_TIMELINE
+extern "C" int msq_exp_timeline(void* host_out) {
+  return (int)hipMemcpyFromSymbol(host_out, HIP_SYMBOL(g_timeline), sizeof(uint64_t) * 512 * 16 * 8, 0, hipMemcpyDeviceToHost);
+}
+#endif
 
 extern "C" {
 
