@@ -333,13 +333,15 @@ __device__ __forceinline__ void stage_x_rows(float* dst, const float* const (&sr
     }
   }
 }
-__device__ __forceinline__ void load_x32_consecutive(const float* x, uint32_t* v, int n) {
+// s: an exact power-of-two factor applied before the rounding to fp16 (callers undo it on their sums); it moves small
+// activations out of the fp16 denormal range
+__device__ __forceinline__ void load_x32_consecutive(const float* x, uint32_t* v, int n, float s = 1.f) {
   const float4* p = (const float4*)x;
 #pragma unroll
   for (int i = 0; i < n / 4; i++) {
     const float4 f = p[i];
-    v[2 * i] = pack_h2(f.x, f.y);
-    v[2 * i + 1] = pack_h2(f.z, f.w);
+    v[2 * i] = pack_h2(f.x * s, f.y * s);
+    v[2 * i + 1] = pack_h2(f.z * s, f.w * s);
   }
 }
 __device__ __forceinline__ float sum_h2(const uint32_t* v, int n) {
@@ -374,9 +376,9 @@ struct DecIQ1S {
   static constexpr int NTBL = 1;
   __device__ static CopyJob tbl_job(int, uint32_t at) { return {(const uint4*)g_tbl_iq1s.w, at, LDS_WORDS / 4, false}; }
   template <class S>
-  __device__ static X load_x(S x, uint32_t u) {
+  __device__ static X load_x(S x, uint32_t u, float s = 1.f) {
     X r;
-    load_x32_consecutive(xat(x, 32u * u), r.v, 32);
+    load_x32_consecutive(xat(x, 32u * u), r.v, 32, s);
     r.sx = sum_h2(r.v, 16);
     return r;
   }
@@ -462,9 +464,9 @@ struct DecIQ2XXS {
     return {(const uint4*)g_tbl_sign.w, at + MSQ_IQ2XXS_GRID_N * 4, 128, false};
   }
   template <class S>
-  __device__ static X load_x(S x, uint32_t u) {
+  __device__ static X load_x(S x, uint32_t u, float s = 1.f) {
     X r;
-    load_x32_consecutive(xat(x, 32u * u), r.v, 32);
+    load_x32_consecutive(xat(x, 32u * u), r.v, 32, s);
     r.sx = 0.f;
     return r;
   }
@@ -541,11 +543,11 @@ struct DecQ8_0 {
   struct Raw { uint32_t q[8]; uint32_t d; };
   __device__ static void fill_lds(uint32_t*, int, int) {}
   template <class S>
-  __device__ static X load_x(S x, uint32_t u) {
+  __device__ static X load_x(S x, uint32_t u, float s = 1.f) {
     X r;
     const float4* p = (const float4*)xat(x, 32u * u);
 #pragma unroll
-    for (int i = 0; i < 8; i++) { const float4 f = p[i]; r.v[4 * i] = f.x; r.v[4 * i + 1] = f.y; r.v[4 * i + 2] = f.z; r.v[4 * i + 3] = f.w; }
+    for (int i = 0; i < 8; i++) { const float4 f = p[i]; r.v[4 * i] = f.x * s; r.v[4 * i + 1] = f.y * s; r.v[4 * i + 2] = f.z * s; r.v[4 * i + 3] = f.w * s; }
     return r;
   }
   template <class P>
@@ -614,13 +616,13 @@ struct DecQ6K {
   struct Raw { uint32_t qa[2], qb[2], qh[2], sc[2], d; };
   __device__ static void fill_lds(uint32_t*, int, int) {}
   template <class S>
-  __device__ static X load_x(S x, uint32_t u) {
+  __device__ static X load_x(S x, uint32_t u, float s = 1.f) {
     X r;
     const uint32_t j = u & 7u;
     const uint32_t base = 256u * (u >> 3) + 128u * (j >> 2) + 8u * (j & 3u);
 #pragma unroll
     for (int k = 0; k < 4; k++) {
-      load_x32_consecutive(xat(x, base + 32u * k), r.v + 4 * k, 8);
+      load_x32_consecutive(xat(x, base + 32u * k), r.v + 4 * k, 8, s);
       r.sx[k] = sum_h2(r.v + 4 * k, 4);
     }
     return r;

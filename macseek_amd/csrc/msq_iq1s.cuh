@@ -125,7 +125,9 @@ struct DecIQ1SQ {
   static constexpr bool STAGE_X = true, QUANT_X = true, HAS_PRE = true;
   static constexpr int STAGES = 1;
   struct X { uint32_t lo[8], hi[8]; float xs8; };
-  struct Raw { uint32_t qs; uint16_t qh, d; };  // 16-bit fields stay 16-bit: their users read bytes / the low half only
+  // qh and d are held as halves (bit containers): a 16-bit integer would be zero-extended, by an extra instruction,
+  // before each use, and their users read bytes / the low half only
+  struct Raw { uint32_t qs; _Float16 qh, d; };
 
   // ---- tables. The grid comes from device memory (32 KB, two entries per 16-byte item; issue_tables requests a
   // thread's items, finish_tables writes each into both copies); the two small tables are computed.
@@ -191,8 +193,8 @@ struct DecIQ1SQ {
     return {b + 2 + 4 * ib, b + 34 + 2 * ib, b};
   }
   __device__ static Raw fetch(rsrc_t rs, const Off& o, uint32_t soff) {
-    return {buf_ld32(rs, o.qs, soff), (uint16_t)__builtin_amdgcn_raw_buffer_load_b16(rs, (int)o.qh, (int)soff, 0),
-            (uint16_t)__builtin_amdgcn_raw_buffer_load_b16(rs, (int)o.d, (int)soff, 0)};
+    return {buf_ld32(rs, o.qs, soff), __builtin_bit_cast(_Float16, __builtin_amdgcn_raw_buffer_load_b16(rs, (int)o.qh, (int)soff, 0)),
+            __builtin_bit_cast(_Float16, __builtin_amdgcn_raw_buffer_load_b16(rs, (int)o.d, (int)soff, 0))};
   }
 
   // ---- three-step decode: pre() reads the two qh tables, lookup() turns them into the four entry addresses and
@@ -205,22 +207,12 @@ struct DecIQ1SQ {
     uint32_t ahi, alo;
     asm("v_lshlrev_b32_sdwa %0, %1, %2 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:BYTE_1" : "=v"(ahi) : "s"(3u), "v"(r.qh));
     asm("v_lshlrev_b32_sdwa %0, %1, %2 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:BYTE_0" : "=v"(alo) : "s"(2u), "v"(r.qh));
-#ifdef MSQ_EXP_NOLUT
-    return {uint2{ahi & 0x38383838u, 0x3f800000u}, alo & 0x38383838u};
-#else
     return {*(const uint2*)(t + LUT_HI_AT * 4 + ahi), *(const uint32_t*)(t + LUT_LO_AT * 4 + alo)};
-#endif
   }
   // lanec: (lane & 1) * 0x80808080, the lane's grid copy in every byte
   __device__ static void lookup(const Raw& r, const Pre& a, const uint32_t* lds, uint32_t lanec, Look& k) {
     const uint8_t* t = (const uint8_t*)lds;
     const uint32_t T = a.hi.x | a.lo | lanec;
-#ifdef MSQ_EXP_NOGRID
-    k.g[0] = uint2{__builtin_amdgcn_perm(r.qs, T, 0x0c0c0400u), T}; k.g[1] = uint2{__builtin_amdgcn_perm(r.qs, T, 0x0c0c0501u), T};
-    k.g[2] = uint2{__builtin_amdgcn_perm(r.qs, T, 0x0c0c0602u), T}; k.g[3] = uint2{__builtin_amdgcn_perm(r.qs, T, 0x0c0c0703u), T};
-    k.sc = __builtin_bit_cast(float, a.hi.y);
-    return;
-#endif
     k.g[0] = *(const uint2*)(t + GRID_AT * 4 + __builtin_amdgcn_perm(r.qs, T, 0x0c0c0400u));
     k.g[1] = *(const uint2*)(t + GRID_AT * 4 + __builtin_amdgcn_perm(r.qs, T, 0x0c0c0501u));
     k.g[2] = *(const uint2*)(t + GRID_AT * 4 + __builtin_amdgcn_perm(r.qs, T, 0x0c0c0602u));
@@ -230,10 +222,6 @@ struct DecIQ1SQ {
   __device__ static float partial(const Raw& r, const Look& k, const X& x) {
     // the first product of each chain takes a literal zero addend (three-operand form): no accumulator to clear
     int lo, hi;
-#ifdef MSQ_EXP_NODOT
-    lo = (int)(k.g[0].x ^ k.g[1].x ^ k.g[2].x ^ k.g[3].x); hi = (int)(k.g[0].y ^ k.g[1].y ^ k.g[2].y ^ k.g[3].y);
-    if (false)
-#endif
     {
     asm("v_dot4_i32_i8 %0, %1, %2, 0" : "=v"(lo) : "v"(k.g[0].x), "v"(x.lo[0]));
     asm("v_dot4_i32_i8 %0, %1, %2, 0" : "=v"(hi) : "v"(k.g[0].x), "v"(x.hi[0]));
@@ -247,11 +235,40 @@ struct DecIQ1SQ {
       hi = __builtin_amdgcn_sdot4((int)k.g[l].y, (int)x.hi[2 * l + 1], hi, false);
     }
     }
+    return finish(r, k, x, lo, hi);
+  }
+  __device__ static float finish(const Raw& r, const Look& k, const X& x, int lo, int hi) {
     const float t = (float)((hi << 8) + lo);  // sum of (8 g +- 1) * n over the unit, exact
     const float w = (t * x.xs8) * k.sc;
     float y;  // d * w with the fp16 d converted inside the multiply
     asm("v_fma_mix_f32 %0, %1, %2, 0 op_sel_hi:[1,0,0]" : "=v"(y) : "v"(r.d), "v"(w));
     return y;
+  }
+  // two units against the same activations (gate and up of a row), their four chains interleaved: a wave on its own
+  // issues a dependent product only every other slot
+  __device__ static void partial2(const Raw& ra, const Look& ka, const Raw& rb, const Look& kb, const X& x, float& ya, float& yb) {
+    int la, ha, lb, hb;
+    asm("v_dot4_i32_i8 %0, %1, %2, 0" : "=v"(la) : "v"(ka.g[0].x), "v"(x.lo[0]));
+    asm("v_dot4_i32_i8 %0, %1, %2, 0" : "=v"(ha) : "v"(ka.g[0].x), "v"(x.hi[0]));
+    asm("v_dot4_i32_i8 %0, %1, %2, 0" : "=v"(lb) : "v"(kb.g[0].x), "v"(x.lo[0]));
+    asm("v_dot4_i32_i8 %0, %1, %2, 0" : "=v"(hb) : "v"(kb.g[0].x), "v"(x.hi[0]));
+    la = __builtin_amdgcn_sdot4((int)ka.g[0].y, (int)x.lo[1], la, false);
+    ha = __builtin_amdgcn_sdot4((int)ka.g[0].y, (int)x.hi[1], ha, false);
+    lb = __builtin_amdgcn_sdot4((int)kb.g[0].y, (int)x.lo[1], lb, false);
+    hb = __builtin_amdgcn_sdot4((int)kb.g[0].y, (int)x.hi[1], hb, false);
+#pragma unroll
+    for (int l = 1; l < 4; l++) {
+      la = __builtin_amdgcn_sdot4((int)ka.g[l].x, (int)x.lo[2 * l], la, false);
+      ha = __builtin_amdgcn_sdot4((int)ka.g[l].x, (int)x.hi[2 * l], ha, false);
+      lb = __builtin_amdgcn_sdot4((int)kb.g[l].x, (int)x.lo[2 * l], lb, false);
+      hb = __builtin_amdgcn_sdot4((int)kb.g[l].x, (int)x.hi[2 * l], hb, false);
+      la = __builtin_amdgcn_sdot4((int)ka.g[l].y, (int)x.lo[2 * l + 1], la, false);
+      ha = __builtin_amdgcn_sdot4((int)ka.g[l].y, (int)x.hi[2 * l + 1], ha, false);
+      lb = __builtin_amdgcn_sdot4((int)kb.g[l].y, (int)x.lo[2 * l + 1], lb, false);
+      hb = __builtin_amdgcn_sdot4((int)kb.g[l].y, (int)x.hi[2 * l + 1], hb, false);
+    }
+    ya = finish(ra, ka, x, la, ha);
+    yb = finish(rb, kb, x, lb, hb);
   }
 };
 

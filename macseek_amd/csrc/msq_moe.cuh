@@ -34,6 +34,10 @@ __device__ uint64_t g_timeline[512 * 16 * 8];
 
 constexpr int kMaxRouted = 6;
 constexpr int kMoeChunkRows = 128;  // rows a workgroup finishes between two synchronisations
+// The down kernel multiplies h by this power of two before it is rounded to fp16 pairs and divides the row sums by it:
+// |h| <= 100 |w| (the clamps of SwiGLU), so routing weights up to 5 keep 128 h inside the fp16 range, and h down to
+// 5e-7 stays out of its denormals.
+constexpr float kHScale = 128.f;
 
 struct MoeArgs {
   const float* x;        // [dim]
@@ -261,14 +265,8 @@ __device__ __forceinline__ void moe_gu_run_ring(const MoeArgs& a, uint32_t* tbl,
     auto fetch = [&](int s) {  // loads of row pair pv into slot s (nothing is read once pv has passed w1), then advance
       const uint32_t bytes = pv < w1 ? mat_bytes : 0u;
       const uint32_t soff = pr * row_bytes;
-#ifdef MSQ_EXP_NOLOAD
-      if (pv < w0 + NR) {
-#endif
       rg[s] = D::fetch(make_rsrc(pg, bytes), off, soff);
       ru[s] = D::fetch(make_rsrc(pu, bytes), off, soff);
-#ifdef MSQ_EXP_NOLOAD
-      } else { asm volatile("" : "+v"(*(uint32_t*)&rg[s]), "+v"(*(uint32_t*)&ru[s])); }
-#endif
       pv++; pr++;
       if (!shared && pr == a.inter && pv < w1) { pr = 0; pe++; set_expert(); }
     };
@@ -306,48 +304,39 @@ __device__ __forceinline__ void moe_gu_run_ring(const MoeArgs& a, uint32_t* tbl,
       MSQ_TL(4);
     }
     if constexpr (requires { D::HAS_PRE; }) {
-      // Three steps per unit (gate of a row pair, then up): table reads of the unit two places ahead, entry reads of
-      // the next unit, arithmetic of this one. Units past the end of the run decode the zeros that their empty buffer
-      // descriptors returned (every address stays inside the tables, and a zero block scale makes the result zero).
-      static_assert(NS == 1 && NR % 2 == 0, "unit pipeline: one stage per unit, buffers alternate gate / up");
+      // Three steps per row pair (gate and up together, four interleaved chains): table reads of the pair two places
+      // ahead, entry reads of the next pair, arithmetic of this one. Pairs past the end of the run decode the zeros that
+      // their empty buffer descriptors returned (every address stays inside the tables, and a zero block scale makes
+      // the result zero).
       const uint32_t lanec = (lane & 1u) * 0x80808080u;
-      typename D::Pre pa[2];
-      typename D::Look lk[2];
-      pa[0] = D::pre(rg[0], tbl);
-      pa[1] = D::pre(ru[0], tbl);
-      D::lookup(rg[0], pa[0], tbl, lanec, lk[0]);
+      typename D::Pre pg_[2], pu_[2];    // [pair & 1]
+      typename D::Look lg[2], lu[2];
+      pg_[0] = D::pre(rg[0], tbl); pu_[0] = D::pre(ru[0], tbl);
+      pg_[1] = D::pre(rg[1], tbl); pu_[1] = D::pre(ru[1], tbl);
+      D::lookup(rg[0], pg_[0], tbl, lanec, lg[0]); D::lookup(ru[0], pu_[0], tbl, lanec, lu[0]);
       [[maybe_unused]] const bool a_never = a.dim == 1u;
+      static_assert(NS == 1 && NR % 2 == 0 && NR >= 4, "two row pairs per fold, table reads two pairs ahead");
       for (uint32_t r0 = w0; r0 < w1 MSQ_EXP_LOOP_COND; r0 += NR) {
 #pragma unroll
-        for (int half = 0; half < 2; half++) {
-          float acc[NR];  // value 2 j + m: row pair j of this half, m = 0 gate, 1 up
+        for (int half = 0; half < NR / 2; half++) {
+          float acc[4];  // value 2 j + m: row pair j of this half, m = 0 gate, 1 up
 #pragma unroll
-          for (int j = 0; j < NR / 2; j++) {
-            const int s = half * (NR / 2) + j, sn = (s + 1) % NR;
-            // table reads first: a result is then waited for a whole unit after its request
-            // (scheduling barriers: left alone, the compiler moves a unit's entry reads next to their use)
-            pa[0] = D::pre(rg[sn], tbl);
-            D::lookup(ru[s], pa[1], tbl, lanec, lk[1]);
+          for (int j = 0; j < 2; j++) {
+            const int s = half * 2 + j, s1 = (s + 1) % NR, s2 = (s + 2) % NR, b = s & 1;
+            D::lookup(rg[s1], pg_[b ^ 1], tbl, lanec, lg[b ^ 1]);
+            D::lookup(ru[s1], pu_[b ^ 1], tbl, lanec, lu[b ^ 1]);
+            pg_[b] = D::pre(rg[s2], tbl);
+            pu_[b] = D::pre(ru[s2], tbl);
+            // (scheduling barriers: left alone, the compiler moves a pair's entry reads next to their use)
             __builtin_amdgcn_sched_barrier(0);
-            float g = D::partial(rg[s], lk[0], xr);
+            D::partial2(rg[s], lg[b], ru[s], lu[b], xr, acc[2 * j], acc[2 * j + 1]);
             __builtin_amdgcn_sched_barrier(0);
-            pa[1] = D::pre(ru[sn], tbl);
-            D::lookup(rg[sn], pa[0], tbl, lanec, lk[0]);
-            __builtin_amdgcn_sched_barrier(0);
-            float u = D::partial(ru[s], lk[1], xr);
-            __builtin_amdgcn_sched_barrier(0);
-            acc[2 * j] = g;
-            acc[2 * j + 1] = u;
-#ifndef MSQ_EXP_NOFETCH
             fetch(s);  // the slot is free again: fetch the row pair NR places ahead
-#else
-            asm volatile("" : "+v"(rg[s].qs), "+v"(ru[s].qs));
-#endif
           }
-          const uint32_t rb = r0 + half * (NR / 2);
+          const uint32_t rb = r0 + half * 2;
           if (rb < w1) {
-            row16_fold<NR>(acc, lane);
-            const uint32_t k = group8_sel<NR>(lane), j = k >> 1, m = k & 1u;
+            row16_fold<4>(acc, lane);
+            const uint32_t k = group8_sel<4>(lane), j = k >> 1, m = k & 1u;
             if (!(lane & 8u) && rb + j < w1) part[((rb + j - c0) * 2 + m) * PSTRIDE + ks * 4 + (lane >> 4)] = acc[0];
           }
         }
@@ -561,11 +550,11 @@ __global__ __launch_bounds__(MAXT) void moe_down_kernel(const MoeArgs a) {
       if (a.stage_x) {
         const float* hs = (const float*)(smem + a.xs_off);
         __syncthreads();
-        if (NE) xr = DR::load_x(XLds{hs + xlds_words(e * a.inter)}, unit_r);
-        if (a.run_shared) xs = DS::load_x(XLds{hs + xlds_words(a.n_routed * a.inter - lo)}, unit_s);
+        if (NE) xr = DR::load_x(XLds{hs + xlds_words(e * a.inter)}, unit_r, kHScale);
+        if (a.run_shared) xs = DS::load_x(XLds{hs + xlds_words(a.n_routed * a.inter - lo)}, unit_s, kHScale);
       } else {
-        if (NE) xr = DR::load_x(a.h + (size_t)e * a.inter, unit_r);
-        if (a.run_shared) xs = DS::load_x(a.h + (size_t)a.n_routed * a.inter, unit_s);
+        if (NE) xr = DR::load_x(a.h + (size_t)e * a.inter, unit_r, kHScale);
+        if (a.run_shared) xs = DS::load_x(a.h + (size_t)a.n_routed * a.inter, unit_s, kHScale);
         __syncthreads();
       }
       if (!valid_r) xr = typename DR::X{};
@@ -620,7 +609,7 @@ __global__ __launch_bounds__(MAXT) void moe_down_kernel(const MoeArgs a) {
     __syncthreads();
     for (uint32_t t = tid; t < n; t += blockDim.x) {
       const float s = sum_in_order(part + t * PSTRIDE, slots);
-      a.y[c0 + t] += s;
+      a.y[c0 + t] += s * (1.f / kHScale);
     }
     __syncthreads();
   }

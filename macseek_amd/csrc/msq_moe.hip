@@ -6,9 +6,6 @@
 
 #include "msq_host.h"
 #include "msq_moe.cuh"
-#ifdef MSQ_EXP_OLDDEC
-#define DecIQ1SQ DecIQ1S
-#endif
 
 namespace msq {
 
@@ -184,9 +181,10 @@ int moe_decode_impl(hipStream_t st, const MsqMoeDecodeArgs* p, const MsqBuffer* 
     // persistent workgroups, dealt to the routed experts and the shared expert in proportion to their bytes
     const long rows_r = (long)n_gu_r * inter, rows_s = gu_s ? inter : 0;
     const long total = std::max<long>(2, (long)cus * std::max(1, env_gu_wgs));
-    // ... weighted by the decode work per byte (IQ2_XXS takes two table lookups and sign flips per 8 weights: measured
-    // about 1.2x IQ1_S per byte)
-    auto cost = [](int t) { return t == MSQ_IQ2_XXS ? 1.2 : 1.0; };
+    // ... weighted by the decode work per byte (IQ2_XXS takes two 16-byte table lookups and sign flips per 8 weights:
+    // the layer of 6 IQ1_S + 1 IQ2_XXS experts is fastest with its bytes counted 1.4 times)
+    static const int env_iq2_cost = env_int("MSQ_MOE_IQ2_COST", 140);  // percent
+    auto cost = [](int t) { return t == MSQ_IQ2_XXS ? 0.01 * env_iq2_cost : 1.0; };
     const double br = (double)n_gu_r * a.rb_gu_r * cost(p->t_gate_up), bs = gu_s ? (double)a.rb_gu_s * cost(ts) : 0.0;
     long g_s = gu_s ? std::max<long>(1, (long)(total * bs / (br + bs) + 0.5)) : 0;
     long g_r = n_gu_r ? std::max<long>(1, total - g_s) : 0;

@@ -10,7 +10,7 @@ import torch
 
 import oracle as O
 from macseek_amd import quant as q
-from util import (F32_X_TYPES, TOL_NORTH_STAR, TOL_REF_F16_X, TOL_REF_F32_X, matvec_errors, place_in_arena, same_floats, up)
+from util import TOL_NORTH_STAR, matvec_errors, place_in_arena, same_floats, tol_ref, up
 
 pytestmark = pytest.mark.gpu
 GOLD = np.load(os.path.join(os.path.dirname(__file__), "golden", "dequant_golden.npz"))
@@ -94,7 +94,7 @@ def test_matvec_vs_oracle(dev, t, rows, cols, groups, acc, what):
     err_ref, err_ns = matvec_errors(got, ry, mag, wn2 + (y0.astype(np.float64) ** 2 if acc else 0), x, rows, cols, groups)
     print(f"  {O.TYPE_NAMES[t]:8s} {what:24s} [{cols:5d} -> {rows:6d}] g{groups} err/sum|wx| {err_ref:.2e} err/(|w||x|) {err_ns:.2e}")
     assert err_ns <= TOL_NORTH_STAR
-    assert err_ref <= (TOL_REF_F32_X if t in F32_X_TYPES else TOL_REF_F16_X)
+    assert err_ref <= tol_ref(t, cols)
 
 
 @pytest.mark.parametrize("t,rows,cols", [(O.IQ1_S, 4096, 7168), (O.IQ4_NL, 520, 4096), (O.Q8_0, 300, 2048), (O.Q6_K, 1536, 7168)])
@@ -114,7 +114,7 @@ def test_activation_offset_four_bytes(dev, t, rows, cols):
     assert got[0] == 0.0
     err_ref, err_ns = matvec_errors(got[1:], ry, mag, wn2, x, rows, cols, 1)
     assert err_ns <= TOL_NORTH_STAR
-    assert err_ref <= (TOL_REF_F32_X if t in F32_X_TYPES else TOL_REF_F16_X)
+    assert err_ref <= tol_ref(t, cols)
 
 
 def test_output_head_shape(dev):
@@ -129,7 +129,7 @@ def test_output_head_shape(dev):
     q.encode_matvec(e, t, q.Buffer.of(Wd), rows, cols, q.Buffer.of(xd), q.Buffer.of(yd))
     e.wait()
     err_ref, err_ns = matvec_errors(yd.cpu().numpy(), ry, mag, wn2, x, rows, cols, 1)
-    assert err_ns <= TOL_NORTH_STAR and err_ref <= TOL_REF_F16_X
+    assert err_ns <= TOL_NORTH_STAR and err_ref <= tol_ref(t, cols)
 
 
 @pytest.mark.parametrize("t", [O.IQ1_S, O.Q6_K, O.Q8_0], ids=ids)

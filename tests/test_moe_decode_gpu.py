@@ -65,7 +65,7 @@ class Layer:
         return O.moe_decode(*self.types, self.n_routed, self.shared, self.dim, self.inter, self.G, self.U, self.D,
                             W6, self.x, self.y0)
 
-    def check(self, y, h=None, what=""):
+    def check(self, y, h=None, what="", h_tol=2e-5, y_tol=5e-5):
         """Stage-wise parity (the reference test checks h, then y: tests/test_quant_moe.mm:82-92):
         h against the oracle's h; y against the float64 down projection of the h the GPU produced (so stage 2 is
         judged on its own inputs), both in the reference's metric and in the north-star metric
@@ -92,8 +92,8 @@ class Layer:
             y_err = float(np.max(np.abs(got - y2) / (mag2 + 1e-12)))
             ns_err = float(np.max(np.abs(got - y2) / (scale + 1e-30)))
         print(f"  {what} h_err {h_err:.2e} y_err {y_err:.2e} north-star {ns_err:.2e} chain {chain_err:.2e}")
-        # reference bounds are 2e-5 (h) and 5e-5 (y) with F32 activations; activations are fp16-staged here
-        assert h_err <= 2e-4 and y_err <= 2e-4 and ns_err <= 1e-3 and chain_err <= 5e-3
+        # the reference's own bounds for its F32-activation kernels: h 2e-5, y 5e-5 (tests/test_quant_moe.mm:82-93)
+        assert h_err <= h_tol and y_err <= y_tol and ns_err <= 1e-3 and chain_err <= 5e-3
         return ry
 
 
@@ -111,7 +111,15 @@ CASES = [  # (gu, down, shared type, n_routed, shared, xscale, dim, inter)
     (T.IQ1_S, T.IQ1_S, T.IQ2_XXS, 1, True, 40.0, 512, 256),   # smallest shapes the kernels accept
     (T.IQ1_S, T.IQ1_S, T.Q8_0, 2, True, 1.0, 32768, 256),     # x too long to stage in LDS: gate/up reads it directly
     (T.IQ2_XXS, T.IQ1_S, T.IQ2_XXS, 1, True, 1.0, 256, 16384),  # h rows too long to stage: down reads them directly
+    (T.IQ1_S, T.IQ1_S, T.IQ2_XXS, 6, True, 1500.0, 7168, 2048),  # activations near the top of the fp16 range (max |x| about 6e3)
+    (T.IQ1_S, T.IQ1_S, T.IQ2_XXS, 6, True, 0.02, 7168, 2048),    # small activations: h of the order of 1e-6 .. 1e-4
 ]
+# Cases that miss the reference's F32-activation bounds because activations are staged as fp16 pairs, with the bound
+# asserted instead (measured value in brackets):
+#   IQ2_XXS gate/up over 256 columns (one block per row): h 6e-5 [4.0e-5]
+#   down over h = products of two small Gaussians (heavy-tailed, xs = 0.02): y 8e-5 [5.6e-5]
+H_TOL = {(T.IQ2_XXS, T.IQ1_S, T.IQ2_XXS, 1, True, 1.0, 256, 16384): 6e-5}
+Y_TOL = {(T.IQ1_S, T.IQ1_S, T.IQ2_XXS, 6, True, 0.02, 7168, 2048): 8e-5}
 
 
 @pytest.mark.parametrize("gu,dn,sh,nr,shared,xs,dim,inter", CASES)
@@ -121,7 +129,8 @@ def test_moe_decode_vs_oracle(dev, gu, dn, sh, nr, shared, xs, dim, inter):
     e = q.Enc()
     q.encode_moe_decode(e, L.args(y))
     e.wait()
-    L.check(y, L.scratch, f"gu={O.TYPE_NAMES[gu]} down={O.TYPE_NAMES[dn]} shared={O.TYPE_NAMES[sh] if shared else '-'} routed={nr}")
+    L.check(y, L.scratch, f"gu={O.TYPE_NAMES[gu]} down={O.TYPE_NAMES[dn]} shared={O.TYPE_NAMES[sh] if shared else '-'} routed={nr} xs={xs}",
+            h_tol=H_TOL.get((gu, dn, sh, nr, shared, xs, dim, inter), 2e-5), y_tol=Y_TOL.get((gu, dn, sh, nr, shared, xs, dim, inter), 5e-5))
 
 
 @pytest.mark.parametrize("dim,inter,sh", [(5120, 2304, O.Q6_K), (7168, 2048, O.IQ2_XXS)])

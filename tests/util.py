@@ -7,11 +7,21 @@ from macseek_amd import quant as q
 
 # north-star tolerance: max |gpu - ref| <= 1e-3 * ||w_row||_2 * ||x||_2
 TOL_NORTH_STAR = 1e-3
-# reference-style tolerance (|gpu - ref| / sum_c |w_c x_c|): the reference allows 2e-5 for F32 activations
+# reference-style tolerance (|gpu - ref| / sum_c |w_c x_c|): the reference allows 2e-5 for its F32-activation n = 1 kernels
 # (tests/test_quant_matvec.mm:42) and 2e-4 against an F32 reference when activations are staged as fp16
-# (tests/test_quant_matvec_n.mm:45); the block formats here stage activations as fp16.
+# (tests/test_quant_matvec_n.mm:45). The block formats here stage activations as fp16 at n = 1 too: the rounding noise of
+# a row averages down with the square root of its length, so the bound asserted for them is tol_ref(cols) below --
+# the reference's 2e-5 from 9216 columns on, 3e-5 at 4096 columns (measured: 2.6e-5), 6e-5 at 1024 (measured: 4.8e-5).
 TOL_REF_F32_X = 2e-5
 TOL_REF_F16_X = 2e-4
+
+
+def tol_ref(t, cols):
+    if t in F32_X_TYPES:
+        return TOL_REF_F32_X
+    return max(TOL_REF_F32_X, 3e-5 * (4096.0 / cols) ** 0.5)
+
+
 F32_X_TYPES = (O.F32, O.F16, O.BF16, O.Q8_0)
 
 
