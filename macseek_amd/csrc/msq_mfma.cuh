@@ -215,14 +215,12 @@ struct FragDense16 {
 };
 
 // ================================================================================================ block fragments
-// For the 256-weight codebook formats the large-token GEMM uses a second decomposition: weight = block_scale * n with
-// n a small integer (or a multiple of 1/8) that fp16 holds exactly -- the sub-block factor (2 s + 1) is folded into the
-// payload. A wave then accumulates a whole 256-column block in the matrix cores and applies the fp32 block scale once
-// per block instead of once per K step. Lane (row n, chunk q) owns the sub-blocks 2 q and 2 q + 1 of its row's block
+// For the 256-weight codebook formats the large-token GEMM uses a second decomposition: the payload is the whole weight,
+// scale included, rounded to fp16 (what the reference's prefill kernels feed their matrix units), so a wave accumulates
+// all of K in the matrix cores without touching the accumulators in between. Lane (row n, chunk q) owns the sub-blocks 2 q and 2 q + 1 of its row's block
 // (16 contiguous bytes of IQ2_XXS), so no lane loads a byte twice; step j (0..7) of a block therefore covers, for chunk
 // q, the 8 columns col_of(q, j) .. + 7 of the block, and the activation operand is read with the same mapping.
 //   Raw / load(block pointer, q)    the lane's bytes of one block
-//   scale(raw)                      fp32 block scale
 //   lookup(raw, j, tbl, col)        table reads of step j (col = lane % 16), issued ahead of their use
 //   finish(raw, j, look, h)         payloads of step j
 __device__ __forceinline__ uint32_t pk_mul_f16(uint32_t a, uint32_t b) {
@@ -270,7 +268,6 @@ struct BlkIQ2XXS {
     r.d = ld16(blk);
     return r;
   }
-  __device__ static float scale(const Raw& r) { return half_bits_to_float(r.d) * 0.125f; }  // db = d (2 s + 1) / 8
   struct Look { uint4 g, s; };
   // byte offsets in the replicated tables: entry << 8 | column << 4
   __device__ static Look lookup(const Raw& r, int j, const uint32_t* tbl, uint32_t col) {
@@ -282,9 +279,12 @@ struct BlkIQ2XXS {
     const uint8_t* t8 = (const uint8_t*)tbl;
     return {*(const uint4*)(t8 + ((g8 & 0xFF00u) | cg)), *(const uint4*)(t8 + ((s8 & 0x7F00u) | cs))};
   }
+  // weight = fp16(d (2 s + 1) / 8) * (+-grid), rounded to fp16 like the reference's dequantized tiles
+  // (src/kernels/quant_moe_prefill.metal:153-167): the whole scale rides in the payload
   __device__ static void finish(const Raw& r, int j, const Look& k, uint32_t (&h)[4]) {
     const uint32_t a1 = r.w[2 * (j >> 2) + 1];
-    const uint32_t m2 = pk_small_int_f16(((a1 >> 27) & 0x1Eu) | 1u);  // 2 s + 1 <= 31; grid <= 43: products are exact
+    const float m = (half_bits_to_float(r.d) * 0.125f) * (float)(((a1 >> 27) & 0x1Eu) | 1u);
+    const uint32_t m2 = pack_h2(m, m);
     h[0] = pk_mul_f16(k.g.x ^ k.s.x, m2); h[1] = pk_mul_f16(k.g.y ^ k.s.y, m2);
     h[2] = pk_mul_f16(k.g.z ^ k.s.z, m2); h[3] = pk_mul_f16(k.g.w ^ k.s.w, m2);
   }
@@ -303,17 +303,19 @@ struct BlkIQ1S {
     r.d = ld16(blk);
     return r;
   }
-  __device__ static float scale(const Raw& r) { return half_bits_to_float(r.d); }  // w = d (2 s + 1) (g + delta)
   struct Look { uint4 g; };
   __device__ static Look lookup(const Raw& r, int j, const uint32_t* tbl, uint32_t) {
     const uint32_t qs = r.qs[j >> 2], qh = (j >> 2) ? r.qh >> 16 : r.qh & 0xFFFFu;
     const int l = j & 3;
     return {((const uint4*)tbl)[((qs >> (8 * l)) & 0xFFu) | (((qh >> (3 * l)) & 7u) << 8)]};
   }
+  // weight = fp16(d (2 s + 1)) * (grid + delta), rounded to fp16 like the reference's dequantized tiles
+  // (src/kernels/quant_moe_prefill.metal:137-147)
   __device__ static void finish(const Raw& r, int j, const Look& k, uint32_t (&h)[4]) {
     const uint32_t qh = (j >> 2) ? r.qh >> 16 : r.qh & 0xFFFFu;
     const uint32_t d2 = (qh & 0x8000u) ? 0xB000B000u : 0x30003000u;          // -+ 1/8 in both halves
-    const uint32_t m2 = pk_small_int_f16(((qh >> 11) & 0xEu) | 1u);          // 2 s + 1 <= 15; |g + delta| <= 9/8
+    const float m = half_bits_to_float(r.d) * (float)(((qh >> 11) & 0xEu) | 1u);
+    const uint32_t m2 = pack_h2(m, m);
     h[0] = pk_mul_f16(pk_add_f16(k.g.x, d2), m2); h[1] = pk_mul_f16(pk_add_f16(k.g.y, d2), m2);
     h[2] = pk_mul_f16(pk_add_f16(k.g.z, d2), m2); h[3] = pk_mul_f16(pk_add_f16(k.g.w, d2), m2);
   }

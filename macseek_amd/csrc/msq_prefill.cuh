@@ -198,11 +198,11 @@ struct PfBlkArgs {
   uint32_t row_chunks;      // chunks of pf_blk_rows() weight rows
 };
 
-constexpr int kPfBlkTokens = 48, kPfBigTokens = 80, kPfBlkPitch = 256 * 2 + 16;
-// waves per workgroup by token tiles per item: four per SIMD for the one-tile variant, three for the others
+constexpr int kPfBlkTokens = 48, kPfBigTokens = 112, kPfBigTiles = kPfBigTokens / 16, kPfBlkPitch = 256 * 2 + 16;
+// waves per workgroup by token tiles per item: four per SIMD for up to three tiles, three for more (registers)
 constexpr int pf_blk_waves(int T) { return T > 3 ? 12 : 16; }
-// weight-row tiles per wave: two fragments per K step (gate + up of one tile, or two tiles of the down matrix) keep
-// the register count low enough for three or four waves per SIMD, which is what overlaps decode, matrix and LDS work
+// weight-row tiles per wave: two fragments per K step (gate + up of one tile, or two tiles of the down matrix) keep the
+// register count low enough for three or four waves per SIMD, which is what overlaps decode, matrix and LDS work
 constexpr int pf_blk_rt(bool gu, int) { return gu ? 1 : 2; }
 constexpr int pf_blk_rows(bool gu, int T) { return pf_blk_waves(T) * pf_blk_rt(gu, T) * 16; }  // weight rows per work item
 // activation staging: double-buffered for up to three token tiles, a single buffer (two barriers per block) for six
@@ -217,6 +217,7 @@ __device__ __forceinline__ void pf_block_body(const PfBlkArgs& a) {
   constexpr int ABUF = (DB ? kPfBlkTokens : kPfBigTokens) * PITCH;
   constexpr int PPS = R / 2, NP = 8 * PPS;  // fragment pairs per K step, per block
   static_assert(R == 2 || R == 4, "fragments are processed in pairs");
+  static_assert(T <= 3 || T == kPfBigTiles, "the single-buffer variant is sized for kPfBigTokens");
   extern __shared__ __attribute__((aligned(16))) uint32_t smem[];
   uint32_t* tbl = smem;
   uint8_t* abuf = (uint8_t*)(smem + B::LDS_WORDS);  // [2][T * 16 tokens][PITCH]
@@ -277,12 +278,54 @@ __device__ __forceinline__ void pf_block_body(const PfBlkArgs& a) {
   for (int t = 0; t < T; t++)
 #pragma unroll
     for (int r = 0; r < R; r++) acc[t][r] = f4_t{0.f, 0.f, 0.f, 0.f};
-  const f4_t zero = {0.f, 0.f, 0.f, 0.f};
 
   for (uint32_t kc = 0; kc < a.nblocks; kc++) {
     const uint32_t kn = kc + 1 < a.nblocks ? kc + 1 : kc;  // the last block fetches itself again: no branch around the loads
     const uint8_t* arow = abuf + (DB ? (kc & 1u) * ABUF : 0u) + n16 * PITCH;
-    f4_t blk[T][R];
+    if constexpr (T > 3) {
+      // many token tiles: a step's fragments are all decoded first, then every tile's activation fragment (read from
+      // LDS two tiles ahead of its use) feeds one matrix instruction per fragment
+      uint32_t af[3][4];
+#pragma unroll
+      for (int j = 0; j < 8; j++) {
+        // the next block's bytes are requested a few at a time between the steps: requested all at once by all waves
+        // right after the barrier, they queue up in the texture addresser and hold the waves at issue
+        if (j == 1) {
+          __builtin_amdgcn_sched_barrier(0);  // keep the requests here: the scheduler would sink them to their first use
+          a_issue(kn);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+        if (j >= 2 && j - 2 < R) {
+          __builtin_amdgcn_sched_barrier(0);
+          nxt[j - 2] = B::load(wrow[j - 2] + (size_t)kn * B::BLOCK_BYTES, q);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+        typename B::Look lk[R];
+#pragma unroll
+        for (int r = 0; r < R; r++) lk[r] = B::lookup(cur[r], j, tbl, n16);
+#pragma unroll
+        for (int u = 0; u < 2; u++) {
+          const uint4 av = *(const uint4*)(arow + u * 16 * PITCH + 2u * blk_col_of(q, j));
+          af[u][0] = av.x; af[u][1] = av.y; af[u][2] = av.z; af[u][3] = av.w;
+        }
+        uint32_t h[R][4];
+#pragma unroll
+        for (int r = 0; r < R; r++) B::finish(cur[r], j, lk[r], h[r]);
+#pragma unroll
+        for (int t = 0; t < T; t++) {
+          const uint32_t(&x)[4] = af[t % 3];
+          if (t + 2 < T) {
+            const uint4 av = *(const uint4*)(arow + (t + 2) * 16 * PITCH + 2u * blk_col_of(q, j));
+            uint32_t(&y)[4] = af[(t + 2) % 3];
+            y[0] = av.x; y[1] = av.y; y[2] = av.z; y[3] = av.w;
+          }
+          if (16u * t < cnt) {  // (uniform) a block of fewer entries leaves its last tiles out
+#pragma unroll
+            for (int r = 0; r < R; r++) acc[t][r] = mfma_f16(x, h[r], acc[t][r]);
+          }
+        }
+      }
+    } else {
     // table reads run one fragment pair ahead where registers allow (pair p = 2 j + half uses lk[p & 1]: fragments
     // 2 half, 2 half + 1 of step j): the one-tile variant has four waves per SIMD to hide them behind instead, the
     // three-tile variant six matrix instructions per pair
@@ -292,7 +335,7 @@ __device__ __forceinline__ void pf_block_body(const PfBlkArgs& a) {
       lk[0][0] = B::lookup(cur[0], 0, tbl, n16);
       lk[0][1] = B::lookup(cur[1], 0, tbl, n16);
     }
-    uint32_t af[T > 3 ? 3 : T][4];
+    uint32_t af[T][4];
 #pragma unroll
     for (int p = 0; p < NP; p++) {
       const int j = p / PPS, r0 = 2 * (p % PPS);
@@ -308,7 +351,7 @@ __device__ __forceinline__ void pf_block_body(const PfBlkArgs& a) {
         nxt[p / 2 - 1] = B::load(wrow[p / 2 - 1] + (size_t)kn * B::BLOCK_BYTES, q);
         __builtin_amdgcn_sched_barrier(0);
       }
-      if (p % PPS == 0 && T <= 3) {  // activations of step j, read with the fragments' column mapping
+      if (p % PPS == 0) {  // activations of step j, read with the fragments' column mapping
 #pragma unroll
         for (int t = 0; t < T; t++) {
           const uint4 av = *(const uint4*)(arow + t * 16 * PITCH + 2u * blk_col_of(q, j));
@@ -328,30 +371,11 @@ __device__ __forceinline__ void pf_block_body(const PfBlkArgs& a) {
       B::finish(cur[r0 + 1], j, lk[p & 1][1], h[1]);
 #pragma unroll
       for (int t = 0; t < T; t++) {
-        if (T > 3) {  // six tiles: short of registers, each tile's activations are read two tiles ahead of their use
-          if (t == 0) {
-#pragma unroll
-            for (int u = 0; u < 2; u++) {
-              const uint4 av = *(const uint4*)(arow + u * 16 * PITCH + 2u * blk_col_of(q, j));
-              af[u][0] = av.x; af[u][1] = av.y; af[u][2] = av.z; af[u][3] = av.w;
-            }
-          }
-        }
-        const uint32_t(&x)[4] = af[T > 3 ? t % 3 : t];
-        if (T > 3 && t + 2 < T) {
-          const uint4 av = *(const uint4*)(arow + (t + 2) * 16 * PITCH + 2u * blk_col_of(q, j));
-          uint32_t(&y)[4] = af[(t + 2) % 3];
-          y[0] = av.x; y[1] = av.y; y[2] = av.z; y[3] = av.w;
-        }
-        blk[t][r0] = mfma_f16(x, h[0], j == 0 ? zero : blk[t][r0]);
-        blk[t][r0 + 1] = mfma_f16(x, h[1], j == 0 ? zero : blk[t][r0 + 1]);
+        const uint32_t(&x)[4] = af[t];
+        acc[t][r0] = mfma_f16(x, h[0], acc[t][r0]);
+        acc[t][r0 + 1] = mfma_f16(x, h[1], acc[t][r0 + 1]);
       }
     }
-#pragma unroll
-    for (int r = 0; r < R; r++) {
-      const float sc = B::scale(cur[r]);
-#pragma unroll
-      for (int t = 0; t < T; t++) acc[t][r] += sc * blk[t][r];
     }
     // the other activation buffer was last read one block ago, before the previous barrier: free to refill (with a
     // single buffer every wave has to be done with the block first)

@@ -67,7 +67,7 @@ int launch_block_t(hipStream_t st, PfBlkArgs a, uint32_t n6, uint32_t n3, uint32
   const uint32_t n = a.nitems;
   int rc;
   a.items = items; a.nitems = n6;
-  if ((rc = launch_block_tt<B, GU, 5>(st, a))) return rc;
+  if ((rc = launch_block_tt<B, GU, kPfBigTiles>(st, a))) return rc;
   a.items = items + 3 * (size_t)n6; a.nitems = n3 + n2;
   if ((rc = launch_block_tt<B, GU, 3>(st, a))) return rc;
   a.items = items + 3 * (size_t)(n6 + n3 + n2); a.nitems = n - n6 - n3 - n2;
