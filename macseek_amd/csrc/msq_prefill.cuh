@@ -432,6 +432,13 @@ __global__ __launch_bounds__(64 * pf_blk_waves(T)) void moe_pf_block_kernel(cons
   }
 }
 
+// A piece of the scratch header, handed over by value in the kernel arguments (the argument block holds 4 KB)
+constexpr int kHdrChunkWords = 960;
+struct HdrChunk { uint32_t w[kHdrChunkWords]; };
+__global__ __launch_bounds__(256) void moe_pf_header_kernel(uint32_t* dst, const HdrChunk c, uint32_t n) {
+  for (uint32_t i = threadIdx.x; i < n; i += blockDim.x) dst[i] = c.w[i];
+}
+
 // Xg[i] = fp16(X[src(i)]): i < total gathers token tok[i]; rows total .. total + n - 1 are the tokens themselves
 template <bool X_BF16>
 __global__ __launch_bounds__(256) void moe_pf_gather_kernel(const void* __restrict__ X, uint16_t* __restrict__ Xg,

@@ -2,6 +2,7 @@
 #include <algorithm>
 #include <array>
 #include <cstdlib>
+#include <cstring>
 #include <vector>
 
 #include "msq_host.h"
@@ -196,9 +197,20 @@ int msq_moe_prefill(void* stream, const MsqMoePrefillArgs* p) {
     ni_shared = emit(v, items + 3 * (size_t)ni_routed, nc_shared);
   }
   uint8_t* sc = bptr_mut(&p->scratch);
-  // pageable source: the copy is staged by the runtime before this call returns, and ordered on the stream
-  MSQ_HIP(hipMemcpyAsync(sc, hdr.data(), 24 * (size_t)(ne + 1) + 4 * (size_t)(ne + 2) + 8 * (size_t)(nt_routed + nt_shared) +
-                             12 * (size_t)(ni_routed + ni_shared), hipMemcpyHostToDevice, st));
+  // The header travels in kernel arguments, a few KB per launch: nothing is read from host memory after this call
+  // returns, the call never waits for the stream, and a stream capture records the values themselves.
+  {
+    const size_t used = 24 * (size_t)(ne + 1) + 4 * (size_t)(ne + 2) + 8 * (size_t)(nt_routed + nt_shared) +
+                        12 * (size_t)(ni_routed + ni_shared);
+    const size_t words = (used + 3) / 4;
+    for (size_t w0 = 0; w0 < words; w0 += kHdrChunkWords) {
+      HdrChunk c;
+      const uint32_t n = (uint32_t)std::min<size_t>(kHdrChunkWords, words - w0);
+      memcpy(c.w, hdr.data() + 4 * w0, 4 * (size_t)n);  // hdr is padded to a multiple of 256 bytes
+      hipLaunchKernelGGL(moe_pf_header_kernel, dim3(1), dim3(256), 0, st, (uint32_t*)sc + w0, c, n);
+    }
+    MSQ_HIP(hipGetLastError());
+  }
   const size_t rows = (size_t)total + n;
   uint16_t* Xg = (uint16_t*)(sc + hbytes);
   uint16_t* H = (uint16_t*)((uint8_t*)Xg + align256(rows * dim * 2));

@@ -106,10 +106,21 @@ def test_prefill_gemm_2048_tokens_over_384_resident_experts(dev):
     e.wait()
     assert torch.equal(y1, Y)
 
-    # tokens to check: the first two, one routed to the most popular expert (cut into 80-entry blocks), one routed to a
-    # least popular expert (a one-tile item), the last token
+    # tokens to check (the reference checks up to 40 plus the tile-boundary ones, tests/test_quant_moe_prefill.mm:165-177):
+    # the first two and the last; in the most popular expert (its 1545 entries are cut into blocks of 112 entries = seven
+    # 16-entry tiles) the entries around tile and block boundaries and its last ones; one token of a least popular expert
     popular, rare = int(np.argmax(counts)), int(used[np.argmin(counts[used])])
-    chk = sorted({0, 1, int(np.nonzero((ids == popular).any(1))[0][-1]), int(np.nonzero((ids == rare).any(1))[0][0]), N - 1})
+    pe = int(np.nonzero(used == popular)[0][0])
+    m = int(counts[popular])
+    inside = [0, 1, 15, 16, 17, 47, 48, 49, 79, 80, 81, 95, 96, 111, 112, 113, 223, 224, 225, 335, 336, 337,
+              112 * (m // 112) - 1, 112 * (m // 112), 112 * (m // 112) + 1, m - 17, m - 16, m - 2, m - 1]
+    chk = {0, 1, N - 1, int(np.nonzero((ids == rare).any(1))[0][0])}
+    chk |= {int(tok[offs[pe] + i]) for i in inside if 0 <= i < m}
+    # and the first entry of ten mid-sized experts (two- and three-tile items)
+    mid = [j for j in range(len(used)) if 17 <= counts[used[j]] <= 48][:10]
+    chk |= {int(tok[offs[j]]) for j in mid}
+    chk = sorted(chk)
+    assert len(chk) >= 40
     need = sorted(set(int(x) for x in ids[chk].ravel()))
     mats = {x: (host(arena[x * per_exp:x * per_exp + gu_b]), host(arena[x * per_exp + gu_b:x * per_exp + 2 * gu_b]),
                 host(arena[x * per_exp + 2 * gu_b:(x + 1) * per_exp])) for x in need}
@@ -124,6 +135,6 @@ def test_prefill_gemm_2048_tokens_over_384_resident_experts(dev):
     Yf, _ = O.moe_prefill(*args, 0, Y0)
     err_h = float(np.max(np.abs(got - Yh) / (Ym + 1e-9)))
     err_f = float(np.max(np.abs(got - Yf) / (Ym + 1e-9)))
-    print(f"  2048 tokens, {len(used)} experts used, entries {total} (max {counts.max()} per expert), checked tokens {chk.tolist()}: "
+    print(f"  2048 tokens, {len(used)} experts used, entries {total} (max {counts.max()} per expert), {len(chk)} tokens checked: "
           f"err(fp16-staged ref) {err_h:.2e} err(vs F32) {err_f:.2e}")
     assert err_h <= 1e-3 and err_f <= 5e-3  # the bounds of the small cases (tests/test_quant_moe_prefill.mm:223)

@@ -99,6 +99,49 @@ def run_gpu(c, x_bf16=False):
     return y1, torch.equal(y1, Yd)
 
 
+def test_moe_prefill_in_a_captured_graph(dev):
+    """The call only enqueues (quant.hpp:3,91-92): captured into a HIP graph -- nothing may be read from host memory at
+    replay time -- every replay repeats the eager result bit for bit, with eager work and synchronizations between the
+    replays and the host-side argument structures destroyed after the capture."""
+    c = build(O.IQ2_XXS, O.IQ1_S, O.Q8_0, 600, 6, 20, True, "sizes", 512, 256)
+    y_eager, same = run_gpu(c)
+    assert same
+    total = len(c["tok"])
+    Xd, Yd = up(c["X"]), up(c["Y0"].copy())
+    keep = [up(c["tok"]), up(c["wt"]), up(c["slot_of"])]
+    scratch = torch.empty(q.moe_prefill_scratch_bytes(total, c["n"], c["n_exp"], c["dim"], c["inter"]), dtype=torch.uint8, device="cuda:0")
+
+    def args():
+        a = q.MoePrefillArgs()
+        a.t_gate_up, a.t_down, a.t_shared = c["types"]
+        a.n_tokens, a.n_exp, a.slots, a.offs = c["n"], c["n_exp"], c["slots"][:c["n_exp"]], list(c["offs"])
+        a.tok, a.wt, a.slot_of = q.Buffer.of(keep[0]), q.Buffer.of(keep[1]), q.Buffer.of(keep[2])
+        a.k_per_token, a.has_shared, a.shared = c["k"], True, c["slots"][c["n_exp"]]
+        a.X, a.Y, a.scratch = q.Buffer.of(Xd), q.Buffer.of(Yd), q.Buffer.of(scratch)
+        a.dim, a.inter, a.x_is_bf16 = c["dim"], c["inter"], False
+        return a
+
+    g = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        q.encode_moe_prefill(q.Enc(side), args())  # warm-up outside the capture
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    with torch.cuda.graph(g):
+        q.encode_moe_prefill(q.Enc(torch.cuda.current_stream()), args())
+    import gc
+    gc.collect()
+    for rep in range(4):
+        Yd.copy_(up(c["Y0"]))
+        scratch.random_(0, 255)  # the header must be rewritten by the replay itself
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(Yd, y_eager), f"replay {rep} differs from the eager result"
+        _ = (Xd * 2).sum().item()  # eager work between the replays
+
+
 def check(c, y, n_check, x_bf16=False):
     n = c["n"]
     if n_check <= 0 or n_check >= n:
