@@ -32,6 +32,8 @@ HBM_PEAK_GBPS = 8000.0
 # HBM bytes per launch of the decode gate/up kernel, from the FETCH_SIZE / WRITE_SIZE counter runs of this workload
 # (KiB per dispatch, scaled by what the same counters read for a 1 GiB copy: x2.000 and x1.000): 42.91 MB + 0.06 MB
 GU_TRAFFIC_BYTES = 42970419
+# HBM bytes of the three launches of the prefill gate/up GEMM together (same counters, same scaling), configs[3]
+PF_GU_TRAFFIC_BYTES = None
 
 
 def cores():
@@ -94,7 +96,7 @@ def graph_ms_per_launch(torch, launch, n):
 
 def timed_graph(torch, enqueue_steps, steps, warmup):
     """Captures `steps` back-to-back steps in one HIP graph (the loop is launch-bound from Python otherwise), replays
-    it `warmup` times untimed, then times one replay = exactly `steps` steps between device synchronisations."""
+    it `warmup` times untimed, then times five replays one by one and returns (the fastest, all five) in ms per step."""
     g = torch.cuda.CUDAGraph()
     side = torch.cuda.Stream()
     side.wait_stream(torch.cuda.current_stream())
@@ -108,10 +110,13 @@ def timed_graph(torch, enqueue_steps, steps, warmup):
     for _ in range(reps):
         g.replay()
     torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    g.replay()
-    torch.cuda.synchronize()
-    return (time.perf_counter() - t0) * 1e3 / steps
+    reps_ms = []
+    for _ in range(5):  # each timed region is one replay = exactly `steps` steps between device synchronisations
+        t0 = time.perf_counter()
+        g.replay()
+        torch.cuda.synchronize()
+        reps_ms.append((time.perf_counter() - t0) * 1e3 / steps)
+    return min(reps_ms), reps_ms
 
 
 # ------------------------------------------------------------------------------------------------ MoE decode layer
@@ -170,7 +175,7 @@ def bench_moe_decode(torch, args):
         for i in range(n):
             run_part(i, q.MoePart.All)
 
-    ms_step = timed_graph(torch, enqueue, args.steps, args.warmup)
+    ms_step, ms_reps = timed_graph(torch, enqueue, args.steps, args.warmup)
     w_bytes = TOPK * per_exp + 2 * sgu_b + sdn_b
     h_bytes = (TOPK + 1) * INTER * 4
     step_bytes = w_bytes + DIM * 4 + 2 * h_bytes + 2 * DIM * 4
@@ -207,14 +212,33 @@ def bench_moe_decode(torch, args):
             break
     el = time.perf_counter() - t0
     cpu_value = step_bytes * n_cpu / el / 1e9 if n_cpu else None
+    # the reference's own form of the CPU path is single-threaded (tests/ref/dequant.cpp:122-131): same port, one thread
+    t1 = time.perf_counter()
+    n_cpu1 = 0
+    while not args.gpu_only:
+        O.moe_decode(int(tr), int(tr), int(ts), TOPK, True, DIM, INTER, G, U, D, wts[i0], xh, np.zeros(DIM, np.float32), nthreads=1)
+        n_cpu1 += 1
+        if time.perf_counter() - t1 > 8.0 or n_cpu1 >= 50:
+            break
+    el1 = time.perf_counter() - t1
+    cpu_value1 = step_bytes * n_cpu1 / el1 / 1e9 if n_cpu1 else None
+    # what this device gives a kernel that only reads, at the layer's and the dominant kernel's size and at 1 GiB
+    stream = None
+    if not args.gpu_only:
+        del G, U, D
+        s_layer, s_gu, s_big = (stream_read_GBps(torch, b, arena) for b in (step_bytes, gu_bytes, 1 << 30))
+        stream = {"read_GBps_at_layer_bytes": s_layer, "read_GBps_at_kernel_bytes": s_gu, "read_GBps_at_1GiB": s_big,
+                  "layer_pct_of_stream_read": 100 * value / s_layer, "kernel_pct_of_stream_read": 100 * achieved / s_gu,
+                  "layer_pct_of_1GiB_stream_read": 100 * value / s_big}
 
     return {
-        "value": value, "ms_per_step": ms_step, "dtype": "f16 activations x IQ1_S/IQ2_XXS codebook weights, f32 accumulate",
+        "value": value, "ms_per_step": ms_step, "ms_per_step_of_each_replay": ms_reps,
+        "dtype": "int8 IQ1_S codebook x 16-bit block-fixed-point activations (i32, gate/up), f16 x f16 (IQ2_XXS shared expert, down); f32 accumulate",
         "config": {"workload": "BASELINE configs[2]: batch-1 MoE decode layer, 384 experts IQ1_S 7168x2048 (3.3 GB resident), "
                                "top-6 of a seeded softmax router + 1 shared IQ2_XXS expert, SwiGLU; fresh top-6 per step",
                    "bytes_per_step": step_bytes, "experts": NE, "top_k": TOPK, "dim": DIM, "inter": INTER},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBPS,
-                     "traffic": GU_TRAFFIC_BYTES, "kernel": "moe_gu_kernel<DecIQ1S,DecIQ2XXS>", "bytes_per_launch": gu_bytes,
+                     "traffic": GU_TRAFFIC_BYTES, "traffic_source": "profiles/moe_hbm_traffic_fetch_write.txt", "kernel": "moe_gu_kernel<DecIQ1SQ,DecIQ2XXS>", "bytes_per_launch": gu_bytes,
                      "avg_launch_us": gu_graph * 1e3,
                      "timing": "HIP event pair around one graph replay of %d back-to-back launches of this kernel" % n_ev,
                      "eager_event_pair_us": {"mean": gu_mean * 1e3, "median": gu_med * 1e3, "min": gu_min * 1e3},
@@ -222,8 +246,11 @@ def bench_moe_decode(torch, args):
                                        "avg_launch_us": dn_graph * 1e3, "achieved": dn_bytes / (dn_graph * 1e-3) / 1e9,
                                        "eager_event_pair_us": {"mean": dn_mean * 1e3, "median": dn_med * 1e3, "min": dn_min * 1e3}}},
         "cpu_baseline": {"value": cpu_value, "unit": "GB/s", "cores": nth, "kind": "port",
-                         "sample": "%d tokens of the same layer (token 0's experts) through oracle.c moe_decode, %.1f s" % (n_cpu, el)},
+                         "sample": "%d tokens of the same layer (token 0's experts) through oracle.c moe_decode, %.1f s" % (n_cpu, el),
+                         "one_thread": {"value": cpu_value1, "cores": 1,
+                                        "sample": "%d tokens, %.1f s (the form of the reference's own CPU path)" % (n_cpu1, el1)}},
         "pct_of_hbm_peak": 100 * value / HBM_PEAK_GBPS,
+        "stream_read_reference": stream,
     }
 
 
@@ -248,7 +275,7 @@ def bench_matvec(torch, args, t, rows, cols, d_sigma, label):
         if rc != 0:
             raise RuntimeError(L.msq_last_error().decode())
 
-    ms_step = timed_graph(torch, lambda n: [launch(i) for i in range(n)], args.steps, args.warmup)
+    ms_step, ms_reps = timed_graph(torch, lambda n: [launch(i) for i in range(n)], args.steps, args.warmup)
     step_bytes = mat_b + 4 * cols + 4 * rows
     value = step_bytes / (ms_step * 1e-3) / 1e9
     e_mean, e_med, e_min = event_ms_per_launch(torch, launch, min(max(args.steps, 50), 400))
@@ -264,8 +291,18 @@ def bench_matvec(torch, args, t, rows, cols, d_sigma, label):
         el = time.perf_counter() - t0
         if el > (0.2 if args.gpu_only else 10.0) or n_cpu >= 2000:  # profiling runs: a token CPU leg
             break
+    t1 = time.perf_counter()
+    n_cpu1 = 0
+    while True:  # the reference's own CPU path is single-threaded (tests/ref/dequant.cpp:122-131)
+        O.matvec(int(t), Wh, rows, cols, xh, 1, nthreads=1)
+        n_cpu1 += 1
+        el1 = time.perf_counter() - t1
+        if el1 > (0.2 if args.gpu_only else 5.0) or n_cpu1 >= 500:
+            break
+    s_read = stream_read_GBps(torch, step_bytes, arena)
     return {
-        "value": value, "ms_per_step": ms_step, "dtype": "f32" if t == q.QType.Q8_0 else "f16 activations, f32 accumulate",
+        "value": value, "ms_per_step": ms_step, "ms_per_step_of_each_replay": ms_reps,
+        "dtype": "f32" if t == q.QType.Q8_0 else "f16 activations, f32 accumulate",
         "config": {"workload": label, "bytes_per_step": step_bytes, "rows": rows, "cols": cols, "weight_copies": copies},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBPS,
                      "traffic": None, "kernel": "decode matvec <%s> (mv_tok_kernel, mv_kernel or mv_ring_kernel by shape)" % q.type_name(t),
@@ -273,8 +310,10 @@ def bench_matvec(torch, args, t, rows, cols, d_sigma, label):
                      "timing": "HIP event pair around one graph replay of 400 back-to-back launches",
                      "eager_event_pair_us": {"mean": e_mean * 1e3, "median": e_med * 1e3, "min": e_min * 1e3}},
         "cpu_baseline": {"value": step_bytes * n_cpu / el / 1e9, "unit": "GB/s", "cores": nth, "kind": "port",
-                         "sample": "%d matvecs of the same matrix through oracle.c (dequant row + double dot), %.1f s" % (n_cpu, el)},
+                         "sample": "%d matvecs of the same matrix through oracle.c (dequant row + double dot), %.1f s" % (n_cpu, el),
+                         "one_thread": {"value": step_bytes * n_cpu1 / el1 / 1e9, "cores": 1, "sample": "%d matvecs, %.1f s" % (n_cpu1, el1)}},
         "pct_of_hbm_peak": 100 * value / HBM_PEAK_GBPS,
+        "stream_read_reference": {"read_GBps_at_step_bytes": s_read, "pct_of_stream_read": 100 * achieved / s_read},
     }
 
 
@@ -350,18 +389,31 @@ def bench_moe_prefill(torch, steps, warmup, with_cpu=True):
     gu_mean, gu_med, gu_min = event_ms_per_launch(torch, lambda i: call(), max(3, min(steps, 10)))
     os.environ["MSQ_MOEP_SKIP"] = str(1 | 2 | 4 | 16 | 32)
     dn_mean, _, _ = event_ms_per_launch(torch, lambda i: call(), max(3, min(steps, 10)))
+    # the three launches of the gate/up GEMM on their own: one-tile items, two- and three-tile items, popular experts' blocks
+    split = {}
+    for name, keep in (("one_tile_items", 64), ("two_three_tile_items", 128), ("blocks_of_popular_experts", 256)):
+        os.environ["MSQ_MOEP_SKIP"] = str((1 | 4 | 8 | 16 | 32) | ((64 | 128 | 256) & ~keep))
+        split[name + "_us"] = event_ms_per_launch(torch, lambda i: call(), 3)[0] * 1e3
     os.environ["MSQ_MOEP_SKIP"] = "0"
+    n_one = int(np.sum((counts[used] <= 16)))
+    n_mid = int(np.sum((counts[used] > 16) & (counts[used] <= 48)))
+    split["experts_by_class"] = {"one_tile": n_one, "two_three_tiles": n_mid, "more": int(len(used)) - n_one - n_mid}
+    split["entries_by_class"] = {"one_tile": int(counts[used][counts[used] <= 16].sum()),
+                                 "two_three_tiles": int(counts[used][(counts[used] > 16) & (counts[used] <= 48)].sum()),
+                                 "more": int(counts[used][counts[used] > 48].sum())}
     gu_flops = 2.0 * 2 * DIM * INTER * total
     achieved = gu_flops / (gu_mean * 1e-3) / 1e12
     out = {
-        "value": value, "unit": "TFLOP/s", "ms_per_step": ms_step, "dtype": "f16 MFMA (bf16 activations staged as f16, exact IQ2_XXS weights), f32 accumulate",
+        "value": value, "unit": "TFLOP/s", "ms_per_step": ms_step, "dtype": "f16 MFMA (bf16 activations staged as f16, IQ2_XXS weights dequantized to f16 tiles), f32 accumulate",
         "config": {"workload": "BASELINE configs[3]: prefill grouped MoE GEMM, 2048 tokens x 7168 bf16, top-6 of 384 experts, "
                                "Zipf(1.1) popularity, IQ2_XXS gate/up 2048x7168 + down 7168x2048, outputs combined with routing weights",
                    "entries": total, "experts_used": int(len(used)), "tokens_per_expert_max": int(counts.max()),
                    "tokens_per_expert_median": float(np.median(counts[used])), "flops_per_step": flops,
                    "weight_bytes_touched": int(len(used)) * per_exp},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": achieved / MFMA_PEAK_TFLOPS,
-                     "traffic": None, "kernel": "moe_pf_block_kernel<BlkIQ2XXS, gate/up> (three launches: 49..80-entry blocks, two- and three-tile items, one-tile items)",
+                     "traffic": PF_GU_TRAFFIC_BYTES, "traffic_source": "profiles/moe_prefill_hbm_traffic_fetch_write.txt",
+                     "kernel": "moe_pf_block_kernel<BlkIQ2XXS, gate/up> (three launches: blocks of 49..112 entries of the popular experts, two- and three-tile items, one-tile items)",
+                     "gate_up_time_split": split,
                      "flops_per_launch": gu_flops,
                      "avg_launch_us": gu_mean * 1e3, "min_launch_us": gu_min * 1e3,
                      "weight_GBps": int(len(used)) * 2 * gu_b / (gu_mean * 1e-3) / 1e9,
@@ -384,13 +436,40 @@ def bench_moe_prefill(torch, steps, warmup, with_cpu=True):
                       np.zeros((N, DIM), np.float32), nthreads=nth)
         el = time.perf_counter() - t0
         cpu_flops = 2.0 * 3 * DIM * INTER * n_chk * TOPK
+        t1 = time.perf_counter()
+        O.moe_prefill(int(t), int(t), int(t), N, len(used), False, DIM, INTER, G, U, D, offs, tok, wt, Xh, chk[:1], 1,
+                      np.zeros((N, DIM), np.float32), nthreads=1)
+        el1 = time.perf_counter() - t1
         out["cpu_baseline"] = {"value": cpu_flops / el / 1e12, "unit": "TFLOP/s", "cores": nth, "kind": "port",
                                "sample": "%d tokens x top-6 of the same routing through oracle.c moe_prefill (dequant each needed "
-                                         "expert row, double dots), %.1f s; whole job = x%d" % (n_chk, el, N // n_chk)}
+                                         "expert row, double dots), %.1f s; whole job = x%d" % (n_chk, el, N // n_chk),
+                               "one_thread": {"value": cpu_flops / n_chk / el1 / 1e12, "cores": 1, "sample": "1 token x top-6, %.1f s" % el1}}
     return out
 
 
 # ------------------------------------------------------------------------------------------------ stream / copy references
+def stream_read_GBps(torch, nbytes, arena=None):
+    """What a kernel that only reads (msq_bw_probe) gets for `nbytes` per launch, launches back to back over distinct memory."""
+    from macseek_amd import _lib
+    from macseek_amd import quant as q
+    L = _lib.load()
+    dev = torch.device("cuda:0")
+    if arena is None:
+        arena = torch.randint(0, 256, (2 << 30,), dtype=torch.uint8, device=dev)
+    sink = torch.zeros(4096, dtype=torch.uint8, device=dev)
+    sb = q.Buffer.of(sink).c()
+    nbytes = int(nbytes) // 4096 * 4096
+    ncopies = max(1, arena.numel() // nbytes)
+    bufs = [q.Buffer.of(arena).sub(i * nbytes, nbytes).c() for i in range(ncopies)]
+
+    def launch(i):
+        rc = L.msq_bw_probe(C.c_void_p(torch.cuda.current_stream().cuda_stream), C.byref(bufs[i % ncopies]), nbytes, C.byref(sb))
+        if rc != 0:
+            raise RuntimeError(L.msq_last_error().decode())
+    ms = graph_ms_per_launch(torch, launch, min(200, max(20, 3 * ncopies)))
+    return nbytes / (ms * 1e-3) / 1e9
+
+
 def bench_stream(torch, args):
     """Plain streaming reads (msq_bw_probe: every lane sums 128-bit loads) at a few sizes: what this device delivers to
     a kernel that does nothing but read, next to the 8 TB/s the rooflines are priced against."""
@@ -672,11 +751,11 @@ def main():
         print("bench.py: " + L.msq_last_error().decode(), file=sys.stderr)
         sys.exit(1)
     if args.workload == "moe_prefill":
-        r = bench_moe_prefill(torch, max(1, min(args.steps, 20)), max(1, min(args.warmup, 3)))
+        r = bench_moe_prefill(torch, max(1, min(args.steps, 20)), max(1, min(args.warmup, 3)), with_cpu=not args.gpu_only)
         out = {"metric": METRIC, "value": r["value"], "unit": "TFLOP/s", "n_gpus": 1, "steps": max(1, min(args.steps, 20)),
                "warmup": max(1, min(args.warmup, 3)), "ms_per_step": r["ms_per_step"], "higher_is_better": True, "scaling": "weak",
                "vs_baseline": None, "dtype": r["dtype"], "data": "synthetic", "config": r["config"], "roofline": r["roofline"],
-               "cpu_baseline": r["cpu_baseline"], "pct_of_mfma_peak": r["pct_of_mfma_peak"]}
+               "cpu_baseline": r.get("cpu_baseline"), "pct_of_mfma_peak": r["pct_of_mfma_peak"]}
         print(json.dumps(out))
         return
     if args.workload == "matmul":
@@ -708,12 +787,16 @@ def main():
            "ms_per_step": r["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
            "dtype": r["dtype"], "data": "synthetic", "config": r["config"], "roofline": r["roofline"],
            "cpu_baseline": r["cpu_baseline"], "pct_of_hbm_peak": r["pct_of_hbm_peak"]}
+    for k in ("ms_per_step_of_each_replay", "stream_read_reference"):
+        if k in r:
+            out[k] = r[k]
     if args.workload == "moe_decode" and not args.gpu_only:
         # the metric's second half, measured in the same run on the same device (BASELINE configs[3])
         torch.cuda.empty_cache()
-        p = bench_moe_prefill(torch, 5, 2, with_cpu=False)
+        p = bench_moe_prefill(torch, 5, 2, with_cpu=True)
         out["prefill_moe_gemm"] = {"value": p["value"], "unit": "TFLOP/s", "ms_per_step": p["ms_per_step"],
-                                   "pct_of_mfma_peak": p["pct_of_mfma_peak"], "config": p["config"], "roofline": p["roofline"]}
+                                   "pct_of_mfma_peak": p["pct_of_mfma_peak"], "config": p["config"], "roofline": p["roofline"],
+                                   "cpu_baseline": p["cpu_baseline"]}
     print(json.dumps(out))
 
 

@@ -14,7 +14,7 @@ namespace {
 size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
 size_t header_bytes(int total, int n, int n_exp) {
   const size_t tiles = (size_t)n_exp + total / 16 + n / 16 + 4;  // token tiles of up to 16 entries
-  const size_t items = 2 * (size_t)n_exp + total / kPfBlkTokens + n / kPfBlkTokens + 4;  // blocks of up to 96 entries + remainders
+  const size_t items = 2 * (size_t)n_exp + total / kPfBlkTokens + n / kPfBlkTokens + 4;  // blocks of more than 48 entries + remainders
   return align256(24 * (size_t)(n_exp + 1) + 4 * (size_t)(n_exp + 2) + 8 * tiles + 12 * items);
 }
 bool routed_ok(int t) { return t == MSQ_IQ1_S || t == MSQ_IQ2_XXS; }
@@ -61,23 +61,24 @@ int launch_block_tt(hipStream_t st, PfBlkArgs a) {
   return MSQ_OK;
 }
 // items are sorted by size, largest first: n6 blocks of more than 48 entries, n3 items of three token tiles, n2 of two,
-// then the one-tile items
+// then the one-tile items; skip: profiling mask (see msq_moe_prefill)
 template <class B, bool GU>
-int launch_block_t(hipStream_t st, PfBlkArgs a, uint32_t n6, uint32_t n3, uint32_t n2) {
+int launch_block_t(hipStream_t st, PfBlkArgs a, uint32_t n6, uint32_t n3, uint32_t n2, int skip) {
   const uint32_t* items = a.items;
   const uint32_t n = a.nitems;
   int rc;
   a.items = items; a.nitems = n6;
-  if ((rc = launch_block_tt<B, GU, kPfBigTiles>(st, a))) return rc;
+  if (!(skip & 256) && (rc = launch_block_tt<B, GU, kPfBigTiles>(st, a))) return rc;
   a.items = items + 3 * (size_t)n6; a.nitems = n3 + n2;
-  if ((rc = launch_block_tt<B, GU, 3>(st, a))) return rc;
+  if (!(skip & 128) && (rc = launch_block_tt<B, GU, 3>(st, a))) return rc;
   a.items = items + 3 * (size_t)(n6 + n3 + n2); a.nitems = n - n6 - n3 - n2;
+  if (skip & 64) return MSQ_OK;
   return launch_block_tt<B, GU, 1>(st, a);
 }
 bool block_path(int t) { return t == MSQ_IQ1_S || t == MSQ_IQ2_XXS; }
 template <bool GU>
-int launch_block(int t, hipStream_t st, const PfBlkArgs& a, uint32_t n6, uint32_t n3, uint32_t n2) {
-  return t == MSQ_IQ1_S ? launch_block_t<BlkIQ1S, GU>(st, a, n6, n3, n2) : launch_block_t<BlkIQ2XXS, GU>(st, a, n6, n3, n2);
+int launch_block(int t, hipStream_t st, const PfBlkArgs& a, uint32_t n6, uint32_t n3, uint32_t n2, int skip) {
+  return t == MSQ_IQ1_S ? launch_block_t<BlkIQ1S, GU>(st, a, n6, n3, n2, skip) : launch_block_t<BlkIQ2XXS, GU>(st, a, n6, n3, n2, skip);
 }
 
 template <bool GU>
@@ -142,7 +143,9 @@ int msq_moe_prefill(void* stream, const MsqMoePrefillArgs* p) {
   hipStream_t st = (hipStream_t)stream;
   const int cus = device_info().cus;
   // PROFILING ONLY (wrong output): MSQ_MOEP_SKIP bit mask 1 gather, 2 routed gate/up, 4 shared gate/up, 8 routed down,
-  // 16 shared down, 32 reduce -- read on every call (reference: MACSEEK_MOEP_SKIP, src/kernels/quant.mm:520-522)
+  // 16 shared down, 32 reduce; of the block GEMMs' three launches 64 the one-tile items, 128 the two- and three-tile
+  // items, 256 the blocks of the popular experts -- read on every call (reference: MACSEEK_MOEP_SKIP,
+  // src/kernels/quant.mm:520-522)
   const char* skip_env = getenv("MSQ_MOEP_SKIP");
   const int skip = skip_env && *skip_env ? atoi(skip_env) : 0;
   // ---- header: expert pointer table, offsets, token-tile tables (routed tiles first, then the shared expert's)
@@ -169,12 +172,13 @@ int msq_moe_prefill(void* stream, const MsqMoePrefillArgs* p) {
     for (int t0 = 0; t0 < p->offs[j + 1] - p->offs[j]; t0 += 16) { tiles[2 * nt_routed] = (uint32_t)j; tiles[2 * nt_routed + 1] = (uint32_t)t0; nt_routed++; }
   if (p->has_shared)
     for (int t0 = 0; t0 < n; t0 += 16) { tiles[2 * (nt_routed + nt_shared)] = (uint32_t)ne; tiles[2 * (nt_routed + nt_shared) + 1] = (uint32_t)t0; nt_shared++; }
-  // work items of the block GEMM: blocks of up to 64 entries, largest first (they take longest)
+  // work items of the block GEMM, largest first (they take longest)
   uint32_t* items = tiles + 2 * (size_t)(nt_routed + nt_shared);
   uint32_t ni_routed = 0, ni_shared = 0;
   uint32_t nc_routed[3] = {0, 0, 0}, nc_shared[3] = {0, 0, 0};  // items of more than 48 entries / three tiles / two tiles
   {
-    // an expert's entries are cut into blocks of 96 while more than 48 remain, then one block of at most 48
+    // an expert's entries are cut into blocks of kPfBigTokens while more than kPfBlkTokens remain, then one block of
+    // at most kPfBlkTokens
     auto cut = [](std::vector<std::array<uint32_t, 3>>& v, uint32_t e, int m) {
       int t0 = 0;
       while (m - t0 > kPfBlkTokens) { const int c = std::min(kPfBigTokens, m - t0); v.push_back({e, (uint32_t)t0, (uint32_t)c}); t0 += c; }
@@ -247,7 +251,7 @@ int msq_moe_prefill(void* stream, const MsqMoePrefillArgs* p) {
       b.A = A; b.K = K; b.N = N; b.nblocks = K / 256; b.row_bytes = (uint32_t)row_bytes;
       b.items = d_items + (shared ? 3 * (size_t)ni_routed : 0); b.nitems = shared ? ni_shared : ni_routed;
       const uint32_t* nc = shared ? nc_shared : nc_routed;
-      return launch_block<GU>(type, st, b, nc[0], nc[1], nc[2]);
+      return launch_block<GU>(type, st, b, nc[0], nc[1], nc[2], skip);
     }
     a.A = A; a.N = N; steps(K); a.row_bytes = (uint32_t)row_bytes;
     a.tiles = d_tiles + (shared ? 2 * (size_t)nt_routed : 0); a.ntiles = shared ? nt_shared : nt_routed;
