@@ -681,10 +681,12 @@ def bench_matmul(torch, args):
     import oracle as O
     from macseek_amd import quant as q
     dev = torch.device("cuda:0")
-    n = 2048
     rows_out = []
-    for t, name, rows, cols in ((q.QType.Q6_K, "Q6_K", 1536, 7168), (q.QType.Q5_K, "Q5_K", 512, 7168),
-                                (q.QType.IQ4_NL, "IQ4_NL", 7168, 4096), (q.QType.BF16, "BF16", 384, 7168)):
+    # n = 2048: dequantize-then-GEMM; n = 256 and 512: the fused kernel (mm_fused_kernel)
+    for n, t, name, rows, cols in ((2048, q.QType.Q6_K, "Q6_K", 1536, 7168), (2048, q.QType.Q5_K, "Q5_K", 512, 7168),
+                                   (2048, q.QType.IQ4_NL, "IQ4_NL", 7168, 4096), (2048, q.QType.BF16, "BF16", 384, 7168),
+                                   (512, q.QType.Q6_K, "Q6_K", 1536, 7168), (256, q.QType.Q6_K, "Q6_K", 1536, 7168),
+                                   (512, q.QType.IQ4_NL, "IQ4_NL", 7168, 4096), (256, q.QType.IQ4_NL, "IQ4_NL", 7168, 4096)):
         if int(t) == 30:
             W = (torch.randn(rows * cols, device=dev) * 0.02).to(torch.bfloat16).view(torch.uint8)
         else:
@@ -707,6 +709,7 @@ def bench_matmul(torch, args):
         flops = 2.0 * n * rows * cols
         rows_out.append({"type": name, "rows": rows, "cols": cols, "n": n, "us_per_call": ms * 1e3, "TFLOPs": flops / (ms * 1e-3) / 1e12})
     head = rows_out[0]
+    n = 2048
     cpu = None
     if not args.gpu_only:
         rows, cols, nt = 1536, 7168, 64
@@ -722,7 +725,7 @@ def bench_matmul(torch, args):
     return {"value": head["TFLOPs"], "ms_per_step": head["us_per_call"] * 1e-3, "dtype": "f16 x f16 MFMA (weights and activations rounded to fp16), f32 accumulate",
             "config": {"workload": "prefill matmul, 2048 tokens, BASELINE configs[4] shapes; one step = one msq_matmul call of the Q6_K 1536x7168 case", "cases": rows_out},
             "roofline": {"bound": "mfma", "achieved": head["TFLOPs"], "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": head["TFLOPs"] / MFMA_PEAK_TFLOPS,
-                         "traffic": None, "kernel": "dequant_kernel<Q6_K, fp16> + rocBLAS fp16 GEMM (whole call)", "flops_per_launch": 2.0 * n * 1536 * 7168,
+                         "traffic": None, "kernel": "f32_to_f16_kernel + dequant_kernel<Q6_K, fp16> + rocBLAS fp16 GEMM (whole call; up to 512 tokens: mm_fused_kernel, see cases)", "flops_per_launch": 2.0 * n * 1536 * 7168,
                          "avg_launch_us": head["us_per_call"]},
             "cpu_baseline": cpu}
 

@@ -32,16 +32,14 @@ inline int hip_fail(hipError_t e, const char* where) {
     if (e_ != hipSuccess) return ::msq::hip_fail(e_, #expr); \
   } while (0)
 
-// LDS of one CU; a kernel that takes more than 64 KB of it as dynamic LDS has to be told so (the limit granted so far
-// is kept per kernel instantiation; raising it again is idempotent, so a race between callers is harmless)
+// LDS of one CU; a kernel that takes more than 64 KB of it as dynamic LDS has to be told so. The limit granted so far
+// is kept per kernel (keyed by the kernel's address: instantiations of one template share their function type) and
+// per device.
 constexpr int kMaxLds = 160 * 1024;
+int grant_large_lds(const void* kernel, size_t lds);  // msq_matvec.hip
 template <class K>
-void allow_large_lds(K kernel, size_t lds) {
-  static size_t granted = 64 * 1024;
-  if (lds > granted) {
-    (void)hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    granted = lds;
-  }
+int allow_large_lds(K kernel, size_t lds) {
+  return lds > 64 * 1024 ? grant_large_lds((const void*)kernel, lds) : MSQ_OK;
 }
 inline const uint8_t* bptr(const MsqBuffer* b) { return (const uint8_t*)b->dev + b->off; }
 inline uint8_t* bptr_mut(const MsqBuffer* b) { return (uint8_t*)b->dev + b->off; }

@@ -1,19 +1,25 @@
 // C ABI: prefill matmul Y[n x rows] (+)= X[n x cols] . W^T over raw GGUF block rows (see include/msq.h; reference
 // host code src/kernels/quant.mm:159-248, kernels src/kernels/quant_mm.metal:81-185).
 //
-// The reference multiplies fp16 activations by weight tiles dequantized to fp16 and, from n >= 512, dequantizes the
-// whole matrix to fp16 once and runs a dense GEMM (quant.mm:204-221). Here the second route serves every n: with
-// 8 TB/s of HBM the fp16 copy of an attention projection (7168 x 1536: 22 MB) is written and read back in a few
-// microseconds, after which the product is a plain fp16 x fp16 -> fp32 GEMM, which is left to rocBLAS (MFMA kernels
-// tuned per shape). The fp16 copies of X and W live in scratch the library owns and grows on demand; like the
-// reference's (docs/modules/quant.md:265-268) it is shared by all calls, so calls must be enqueued on one stream at a
-// time, and a call that has to grow it synchronises that stream and allocates (never inside a stream capture).
+// The reference multiplies fp16 activations by weight tiles dequantized to fp16 inside its GEMM kernel and, from
+// n >= 512, dequantizes the whole matrix to fp16 once and runs a dense GEMM (quant.mm:204-221). The same split is used
+// here. Up to 512 tokens: mm_fused_kernel (msq_mm.cuh) decodes each weight tile once per 128 tokens straight into
+// matrix-core fragments -- no fp16 copy of W or X, no scratch, the call only enqueues. Above: the bit-exact
+// dequantizer writes W as fp16 into library-owned scratch (22 MB for a 7168 x 1536 projection, a few microseconds at
+// 8 TB/s) and the product is a plain fp16 x fp16 -> fp32 GEMM left to rocBLAS. That scratch only grows: a larger
+// request allocates a new block and the old one stays alive until the process ends (work already enqueued may still
+// read it), so growing never waits for the stream; it does allocate, so the first call of a larger shape must not be
+// inside a stream capture, and like the reference's scratch (docs/modules/quant.md:265-268) it is shared by all calls:
+// calls above 512 tokens must be enqueued on one stream at a time.
 #include <rocblas/rocblas.h>
 
+#include <cstdlib>
 #include <mutex>
+#include <vector>
 
 #include "msq_deq.cuh"
 #include "msq_host.h"
+#include "msq_mm.cuh"
 
 namespace msq {
 namespace {
@@ -31,18 +37,27 @@ struct Scratch {
 };
 std::mutex g_mu;
 Scratch g_x16, g_w16;
+std::vector<void*> g_retired;  // outgrown blocks: kept until the process ends
 rocblas_handle g_blas = nullptr;
+// tokens up to which the fused kernel serves the call (the reference's threshold is 512, quant.mm:204); MSQ_MM_FUSED_MAX
+// overrides it for experiments
+int fused_max_tokens() {
+  static const int v = [] { const char* e = getenv("MSQ_MM_FUSED_MAX"); return e && *e ? atoi(e) : 512; }();
+  return v;
+}
 
-// at least `bytes` of device memory in s (>= 64 MiB like the reference's, quant.mm:176-183); growing waits for the
-// stream first, since enqueued work may still use the old allocation
+// at least `bytes` of device memory in s (>= 64 MiB like the reference's, quant.mm:176-183)
 int reserve(Scratch& s, size_t bytes, hipStream_t st) {
   if (s.bytes >= bytes) return MSQ_OK;
-  MSQ_HIP(hipStreamSynchronize(st));
-  if (s.p) MSQ_HIP(hipFree(s.p));
-  s.p = nullptr;
-  s.bytes = 0;
+  hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(st, &cs) == hipSuccess && cs != hipStreamCaptureStatusNone)
+    return fail(MSQ_ERR_SCRATCH, "macseek quant: matmul: the fp16 scratch has to grow, which cannot happen inside a stream capture "
+                                 "(run the shape once before capturing)");
+  void* p = nullptr;
   const size_t want = std::max(bytes, (size_t)64 << 20);
-  MSQ_HIP(hipMalloc(&s.p, want));
+  MSQ_HIP(hipMalloc(&p, want));
+  if (s.p) g_retired.push_back(s.p);
+  s.p = p;
   s.bytes = want;
   return MSQ_OK;
 }
@@ -98,10 +113,52 @@ int gemm_f16(hipStream_t st, const uint16_t* W16, const uint16_t* X16, float* Y,
   return MSQ_OK;
 }
 
-int matmul_h(hipStream_t st, int t, const MsqBuffer* W, int rows, int cols, const uint16_t* X16, float* Y, int n, bool accumulate,
-             int x_stride) {
+template <class F, bool X_F32>
+int launch_mm_t(hipStream_t st, const MmArgs& a) {
+  auto go = [&](auto wv_tag, auto tm_tag) {
+    constexpr int WV = decltype(wv_tag)::value, TM = decltype(tm_tag)::value;
+    const size_t lds = (size_t)F::LDS_WORDS * 4 + 2 * (size_t)16 * TM * kMmPitch;
+    allow_large_lds(mm_fused_kernel<F, WV, TM, X_F32>, lds);
+    hipLaunchKernelGGL((mm_fused_kernel<F, WV, TM, X_F32>), dim3((a.rows + 16 * WV - 1) / (16 * WV), (a.n + 16 * TM - 1) / (16 * TM)),
+                       dim3(64 * WV), lds, st, a);
+  };
+  // the largest tile (a weight tile is decoded once per workgroup, an activation tile staged once) that still gives
+  // every CU a workgroup; with fewer, the call is bound by the latency of one workgroup's K loop
+  const long cus = device_info().cus;
+  auto wgs = [&](long wv, long tm) { return ((a.rows + 16 * wv - 1) / (16 * wv)) * ((a.n + 16 * tm - 1) / (16 * tm)); };
+  using I1 = std::integral_constant<int, 1>; using I2 = std::integral_constant<int, 2>;
+  using I4 = std::integral_constant<int, 4>; using I8 = std::integral_constant<int, 8>;
+  const long want = cus;
+  if (a.n > 64 && wgs(8, 8) >= want) go(I8{}, I8{});
+  else if (a.n > 64 && wgs(4, 8) >= want) go(I4{}, I8{});
+  else if (a.n > 32 && wgs(4, 4) >= want) go(I4{}, I4{});
+  else if (a.n > 16 && wgs(4, 2) >= want) go(I4{}, I2{});
+  else if (a.n > 16 && wgs(4, 1) < want) go(I4{}, I2{});
+  else go(I4{}, I1{});
+  MSQ_HIP(hipGetLastError());
+  return MSQ_OK;
+}
+template <bool X_F32>
+int launch_mm(hipStream_t st, int t, const MmArgs& a) {
+  switch (t) {
+    case MSQ_F32: return launch_mm_t<FragF32H, X_F32>(st, a);
+    case MSQ_F16: return launch_mm_t<FragDense16<MSQ_F16>, X_F32>(st, a);
+    case MSQ_BF16: return launch_mm_t<FragBF16H, X_F32>(st, a);
+    case MSQ_Q8_0: return launch_mm_t<FragQ8_0, X_F32>(st, a);
+    case MSQ_Q5_K: return launch_mm_t<FragQ5K, X_F32>(st, a);
+    case MSQ_Q6_K: return launch_mm_t<FragQ6K, X_F32>(st, a);
+    case MSQ_IQ4_NL: return launch_mm_t<FragIQ4NL, X_F32>(st, a);
+    case MSQ_IQ1_S: return launch_mm_t<FragIQ1S, X_F32>(st, a);
+    case MSQ_IQ2_XXS: return launch_mm_t<FragIQ2XXS, X_F32>(st, a);
+  }
+  return unsupported("matmul", t, (int)a.rows, (int)a.cols);
+}
+
+// more tokens than the fused kernel takes: W as fp16 in scratch (F16 weights are the GEMM operand as they are), then the dense GEMM
+int matmul_big(hipStream_t st, int t, const MsqBuffer* W, int rows, int cols, const uint16_t* X16, float* Y, int n, bool accumulate,
+               int x_stride) {
   const uint16_t* w16 = (const uint16_t*)bptr(W);
-  if (t != MSQ_F16) {  // F16 weights are the GEMM operand as they are
+  if (t != MSQ_F16) {
     const int rc = reserve(g_w16, (size_t)rows * cols * 2, st);
     if (rc != MSQ_OK) return rc;
     const int rd = launch_deq_f16(st, t, bptr(W), (uint16_t*)g_w16.p, (int64_t)rows * cols);
@@ -134,8 +191,14 @@ int msq_matmul_h(void* stream, int t, const MsqBuffer* W, int rows, int cols, co
       !buf_ok(Y, (size_t)n * rows * 4) || ((uintptr_t)bptr(X16) & 1) || ((uintptr_t)bptr(Y) & 3))
     return fail(MSQ_ERR_ARGUMENT, "macseek quant: matmul: buffer missing, too small or misaligned (type %s rows %d cols %d n %d)",
                 msq_type_name_of(t), rows, cols, n);
+  hipStream_t st = (hipStream_t)stream;
+  if (n <= fused_max_tokens()) {
+    const MmArgs a{bptr(X16), bptr(W), (float*)bptr_mut(Y), (uint32_t)n, (uint32_t)rows, (uint32_t)cols, (uint32_t)xs,
+                   (uint32_t)msq_type_row_bytes(t, cols), accumulate ? 1u : 0u};
+    return launch_mm<false>(st, t, a);
+  }
   std::lock_guard<std::mutex> lock(g_mu);
-  return matmul_h((hipStream_t)stream, t, W, rows, cols, (const uint16_t*)bptr(X16), (float*)bptr_mut(Y), n, accumulate != 0, xs);
+  return matmul_big(st, t, W, rows, cols, (const uint16_t*)bptr(X16), (float*)bptr_mut(Y), n, accumulate != 0, xs);
 }
 
 int msq_matmul(void* stream, int t, const MsqBuffer* W, int rows, int cols, const MsqBuffer* X, const MsqBuffer* Y, int n,
@@ -146,12 +209,17 @@ int msq_matmul(void* stream, int t, const MsqBuffer* W, int rows, int cols, cons
     return fail(MSQ_ERR_ARGUMENT, "macseek quant: matmul: buffer missing, too small or misaligned (type %s rows %d cols %d n %d)",
                 msq_type_name_of(t), rows, cols, n);
   hipStream_t st = (hipStream_t)stream;
+  if (n <= fused_max_tokens()) {
+    const MmArgs a{bptr(X), bptr(W), (float*)bptr_mut(Y), (uint32_t)n, (uint32_t)rows, (uint32_t)cols, (uint32_t)cols,
+                   (uint32_t)msq_type_row_bytes(t, cols), accumulate ? 1u : 0u};
+    return launch_mm<true>(st, t, a);  // X is rounded to fp16 on its way into LDS
+  }
   std::lock_guard<std::mutex> lock(g_mu);
   const int rc = reserve(g_x16, (size_t)n * cols * 2, st);
   if (rc != MSQ_OK) return rc;
   const int rx = launch_f32_to_f16(st, (const float*)bptr(X), (uint16_t*)g_x16.p, (size_t)n * cols);
   if (rx != MSQ_OK) return rx;
-  return matmul_h(st, t, W, rows, cols, (const uint16_t*)g_x16.p, (float*)bptr_mut(Y), n, accumulate != 0, cols);
+  return matmul_big(st, t, W, rows, cols, (const uint16_t*)g_x16.p, (float*)bptr_mut(Y), n, accumulate != 0, cols);
 }
 
 }  // extern "C"

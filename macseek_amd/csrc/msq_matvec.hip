@@ -1,5 +1,8 @@
 // C ABI: library bring-up, geometry queries, decode matvec and dequantization (see include/msq.h).
 #include <algorithm>
+#include <map>
+#include <mutex>
+#include <utility>
 
 #include "msq_deq.cuh"
 #include "msq_host.h"
@@ -21,6 +24,20 @@ const DeviceInfo& device_info() {
     return d;
   }();
   return info;
+}
+
+int grant_large_lds(const void* kernel, size_t lds) {
+  static std::mutex mu;
+  static std::map<std::pair<const void*, int>, size_t> granted;
+  int dev = 0;
+  MSQ_HIP(hipGetDevice(&dev));
+  std::lock_guard<std::mutex> lock(mu);
+  size_t& g = granted[{kernel, dev}];
+  if (lds > g) {
+    MSQ_HIP(hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    g = lds;
+  }
+  return MSQ_OK;
 }
 
 // Plain streaming read: every workgroup walks contiguous 16 KiB chunks grid-stride, one 128-bit load per lane per step.

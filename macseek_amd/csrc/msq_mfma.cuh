@@ -122,6 +122,7 @@ struct FragIQ4NL {
   static constexpr int LDS_WORDS = 256;
   __device__ static void fill_lds(uint32_t* lds, int tid, int nt) { copy_words16(lds, g_tbl_iq4nl.w, 256, tid, nt); }
   __device__ static uint32_t col_of(uint32_t q, uint32_t p) { return 4u * q + (p >> 1) + 16u * (p & 1u); }
+  __device__ static uint32_t pos_of(uint32_t c) { return 8u * ((c & 15u) >> 2) + 2u * (c & 3u) + (c >> 4); }  // inverse of col_of
   template <class P>
   __device__ static FragOut get(P row, uint32_t step, uint32_t q, const uint32_t* tbl) {
     const P b = row + step * 18u;
@@ -199,7 +200,7 @@ struct FragQ5K {
 
 template <int QT>  // MSQ_F16 or MSQ_BF16
 struct FragDense16 {
-  static constexpr bool BF16_MATH = QT == MSQ_BF16, HAS_ADD = false;
+  static constexpr bool BF16_MATH = QT == MSQ_BF16, HAS_ADD = false, PLAIN = true;  // PLAIN: the payload is the weight
   static constexpr int LDS_WORDS = 0;
   __device__ static void fill_lds(uint32_t*, int, int) {}
   __device__ static uint32_t col_of(uint32_t q, uint32_t p) { return 8u * q + p; }

@@ -1,0 +1,209 @@
+// Prefill matmul Y[n x rows] (+)= X[n x cols] . W^T with the dequantization fused into the GEMM tiles (reference
+// operator: ms::q::encode_matmul / encode_matmul_h, src/kernels/quant.mm:159-248; reference kernel q_mm,
+// src/kernels/quant_mm.metal:87-115). Numerics are the reference's: activations and weights rounded to fp16, fp32
+// accumulation (quant.hpp:36-39).
+//
+// A workgroup of WV waves owns 16 WV weight rows x 16 TM tokens (the host picks the largest tile that still gives the
+// device a workgroup per CU: below that the call is bound by the latency of a workgroup's K loop). A wave owns one 16-row tile of W: per K step
+// (32 columns) it decodes the lane's eight weights into exact fp16 payloads + fp32 scale (the fragment decoders of
+// msq_mfma.cuh), rounds scale * payload (+ add) to fp16 once (v_fma_mix: fp32 arithmetic, one rounding -- the value
+// the reference's dequantized tile holds) and feeds TM matrix instructions, one per token tile. The activation tile
+// [16 TM tokens][128 columns] is staged in LDS for all waves, double-buffered, one barrier per 128 columns;
+// F32 activations are rounded to fp16 on their way into LDS, so no fp16 copy of X or W is ever materialised.
+#pragma once
+#include "msq_mfma.cuh"
+
+namespace msq {
+
+struct MmArgs {
+  const void* X;       // activations [n][x_stride]: fp16, or fp32 (X_F32)
+  const uint8_t* W;    // raw block rows
+  float* Y;            // [n][rows]
+  uint32_t n, rows, cols, x_stride, row_bytes, accumulate;
+};
+
+// F32 and BF16 weight rows as fp16 payloads (the matmul multiplies every type as fp16)
+struct FragF32H {
+  static constexpr bool BF16_MATH = false, HAS_ADD = false, PLAIN = true;
+  static constexpr int LDS_WORDS = 0;
+  __device__ static void fill_lds(uint32_t*, int, int) {}
+  __device__ static uint32_t col_of(uint32_t q, uint32_t p) { return 8u * q + p; }
+  template <class P>
+  __device__ static FragOut get(P row, uint32_t step, uint32_t q, const uint32_t*) {
+    const u128_a2 a = ld128(row + 128u * step + 32u * q), b = ld128(row + 128u * step + 32u * q + 16);
+    auto f = [](uint32_t v) { return __builtin_bit_cast(float, v); };
+    FragOut o;
+    o.h[0] = pack_h2(f(a.x), f(a.y)); o.h[1] = pack_h2(f(a.z), f(a.w));
+    o.h[2] = pack_h2(f(b.x), f(b.y)); o.h[3] = pack_h2(f(b.z), f(b.w));
+    o.scale = 1.f; o.add = 0.f;
+    return o;
+  }
+};
+struct FragBF16H {
+  static constexpr bool BF16_MATH = false, HAS_ADD = false, PLAIN = true;
+  static constexpr int LDS_WORDS = 0;
+  __device__ static void fill_lds(uint32_t*, int, int) {}
+  __device__ static uint32_t col_of(uint32_t q, uint32_t p) { return 8u * q + p; }
+  template <class P>
+  __device__ static FragOut get(P row, uint32_t step, uint32_t q, const uint32_t*) {
+    const u128_a2 v = ld128(row + 64u * step + 16u * q);
+    auto two = [](uint32_t w) { return pack_h2(__builtin_bit_cast(float, w << 16), __builtin_bit_cast(float, w & 0xFFFF0000u)); };
+    FragOut o;
+    o.h[0] = two(v.x); o.h[1] = two(v.y); o.h[2] = two(v.z); o.h[3] = two(v.w);
+    o.scale = 1.f; o.add = 0.f;
+    return o;
+  }
+};
+
+// fp16(scale * payload + add) for both halves of a payload word: fp32 arithmetic on the fp16 payloads, one rounding
+__device__ __forceinline__ uint32_t scale_round_h2(uint32_t h, float scale, float add) {
+  uint32_t r;
+  asm("v_fma_mixlo_f16 %0, %1, %2, %3 op_sel_hi:[1,0,0]" : "=v"(r) : "v"(h), "v"(scale), "v"(add));
+  asm("v_fma_mixhi_f16 %0, %1, %2, %3 op_sel:[1,0,0] op_sel_hi:[1,0,0]" : "+v"(r) : "v"(h), "v"(scale), "v"(add));
+  return r;
+}
+
+constexpr int kMmKStage = 128, kMmPitch = kMmKStage * 2 + 16;  // bytes per staged token row
+
+// WV waves (16 weight rows each) x TM token tiles per workgroup
+template <class F, int WV, int TM, bool X_F32>
+__global__ __launch_bounds__(64 * WV) void mm_fused_kernel(const MmArgs a) {
+  constexpr int NT = 64 * WV, TOK = 16 * TM, ABUF = TOK * kMmPitch;
+  constexpr int GRAN = TOK * (kMmKStage / 8);           // 16-byte granules (8 halves) per stage
+  constexpr int AG = (GRAN + NT - 1) / NT;              // per thread
+  extern __shared__ __attribute__((aligned(16))) uint32_t smem[];
+  uint32_t* tbl = smem;
+  uint8_t* abuf = (uint8_t*)(smem + F::LDS_WORDS);
+  const uint32_t tid = threadIdx.x, lane = tid & 63u;
+  const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
+  const uint32_t n16 = lane & 15u, q = lane >> 4;
+  const uint32_t row = (blockIdx.x * WV + wave) * 16u + n16;
+  const uint32_t m0 = blockIdx.y * TOK;
+  const gptr_t wrow = as_global(a.W) + (size_t)min(row, a.rows - 1) * a.row_bytes;
+  const uint32_t nstages = a.cols / kMmKStage;
+
+  // activation stage loader: granule g = (token g / 16, columns 8 (g % 16) ..); tokens past n repeat the last one
+  u32x4 pa[AG][X_F32 ? 2 : 1];
+  auto a_issue = [&](uint32_t st) {
+#pragma unroll
+    for (int i = 0; i < AG; i++) {
+      const uint32_t g = min(tid + i * NT, (uint32_t)GRAN - 1u);
+      const uint32_t tok = min(m0 + (g >> 4), a.n - 1), col = st * kMmKStage + (g & 15u) * 8u;
+      if constexpr (X_F32) {
+        const MSQ_GLOBAL float* p = (const MSQ_GLOBAL float*)a.X + (size_t)tok * a.x_stride + col;
+        pa[i][0] = *(const MSQ_GLOBAL u32x4*)p;
+        pa[i][1] = *(const MSQ_GLOBAL u32x4*)(p + 4);
+      } else {
+        // rows of fp16 activations are only 2-byte aligned in general (any x_stride)
+        const u128_a2 v = ld128(as_global((const uint16_t*)a.X + (size_t)tok * a.x_stride + col));
+        pa[i][0] = u32x4{v.x, v.y, v.z, v.w};
+      }
+    }
+  };
+  auto a_store = [&](uint32_t buf) {
+#pragma unroll
+    for (int i = 0; i < AG; i++) {
+      const uint32_t g = tid + i * NT;
+      if (g >= (uint32_t)GRAN) continue;
+      u32x4 v;
+      if constexpr (X_F32) {
+        auto f = [](uint32_t w) { return __builtin_bit_cast(float, w); };
+        v = u32x4{pack_h2(f(pa[i][0].x), f(pa[i][0].y)), pack_h2(f(pa[i][0].z), f(pa[i][0].w)),
+                  pack_h2(f(pa[i][1].x), f(pa[i][1].y)), pack_h2(f(pa[i][1].z), f(pa[i][1].w))};
+      } else {
+        v = pa[i][0];
+      }
+      uint8_t* dst = abuf + buf * ABUF + (g >> 4) * kMmPitch;
+      const uint32_t c0 = (g & 15u) * 8u;  // first of the granule's eight columns inside the stage
+      if constexpr (requires { F::pos_of(0u); }) {
+        // position p of chunk q in a step stands for column col_of(q, p): every column is stored where its fragment
+        // reads it (pos_of is the inverse of col_of)
+        const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+        for (int e = 0; e < 8; e++)
+          *(uint16_t*)(dst + 2u * ((c0 & ~31u) + F::pos_of((c0 & 31u) + e))) = (uint16_t)(w[e >> 1] >> (16 * (e & 1)));
+      } else {
+        *(u32x4*)(dst + 2u * c0) = v;
+      }
+    }
+  };
+
+  a_issue(0);
+  F::fill_lds(tbl, (int)tid, NT);
+  a_store(0);
+  __syncthreads();
+
+  f4_t acc[TM];
+#pragma unroll
+  for (int t = 0; t < TM; t++) acc[t] = f4_t{0.f, 0.f, 0.f, 0.f};
+  uint32_t touch = 0;
+
+  for (uint32_t st = 0; st < nstages; st++) {
+    const uint32_t sn = st + 1 < nstages ? st + 1 : st;  // the last stage fetches itself again: no branch around the loads
+    a_issue(sn);
+    // the next stage's weight bytes are touched now (a lane per 32 bytes of its row's stage), so that the fragment
+    // loads of that stage, which sit right in front of their decode, find them in the nearest cache
+    {
+      const uint32_t stage_bytes = a.row_bytes / nstages;  // rows are whole blocks: every stage has the same byte count
+      const uint32_t off = min(sn * stage_bytes + 32u * q, a.row_bytes - 4u) & ~3u;
+      touch ^= *(const MSQ_GLOBAL uint32_t*)(wrow - ((uintptr_t)wrow & 3u) + off);
+      if (stage_bytes > 128u) touch ^= *(const MSQ_GLOBAL uint32_t*)(wrow - ((uintptr_t)wrow & 3u) + (min(off + 128u, a.row_bytes - 4u) & ~3u));
+    }
+    const uint8_t* arow = abuf + (st & 1u) * ABUF + n16 * kMmPitch + 16u * q;
+    // the four steps' fragments first: their loads are then in flight together (one trip to memory per stage)
+    constexpr int NS = kMmKStage / 32;
+    uint32_t h[NS][4];
+    {
+      FragOut f[NS];
+      float sc[NS];
+#pragma unroll
+      for (int js = 0; js < NS; js++) {
+        const uint32_t step = st * NS + js;
+        f[js] = F::get(wrow, step, q, tbl);
+        sc[js] = f[js].scale;
+        if constexpr (requires(float& s) { F::get_scales(wrow, step, s, s); }) {  // two scale groups per step (Q6_K)
+          float sa, sb;
+          F::get_scales(wrow, step, sa, sb);
+          sc[js] = q < 2 ? sa : sb;
+        }
+      }
+#pragma unroll
+      for (int js = 0; js < NS; js++) {
+#pragma unroll
+        for (int p = 0; p < 4; p++) {
+          if constexpr (requires { F::PLAIN; }) h[js][p] = f[js].h[p];
+          else h[js][p] = scale_round_h2(f[js].h[p], sc[js], F::HAS_ADD ? f[js].add : 0.f);
+        }
+      }
+    }
+#pragma unroll
+    for (int js = 0; js < NS; js++) {
+#pragma unroll
+      for (int t = 0; t < TM; t++) {
+        const uint4 av = *(const uint4*)(arow + t * 16 * kMmPitch + 64u * js);
+        const uint32_t x[4] = {av.x, av.y, av.z, av.w};
+        acc[t] = mfma_f16(x, h[js], acc[t]);
+      }
+    }
+    a_store((st & 1u) ^ 1u);  // the other buffer was last read one stage ago, before the previous barrier
+    __syncthreads();
+  }
+
+  if (touch == 0x9E3779B9u && a.n == 0) a.Y[0] = 0.f;  // never true: keeps the touching loads
+  // D: lane holds weight row n16 (column of D), tokens 4 q + i of every tile
+  if (row < a.rows) {
+#pragma unroll
+    for (int t = 0; t < TM; t++) {
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+        const uint32_t tok = m0 + 16u * t + 4u * q + i;
+        if (tok < a.n) {
+          float* y = a.Y + (size_t)tok * a.rows + row;
+          *y = a.accumulate ? *y + acc[t][i] : acc[t][i];
+        }
+      }
+    }
+  }
+}
+
+}  // namespace msq
