@@ -43,16 +43,18 @@ const TypeRow* type_row(int t) {
 
 enum Kv : uint32_t { U8 = 0, I8, U16, I16, U32, I32, F32, BOOL, STR, ARR, U64, I64, F64 };
 
+// One metadata value. Scalars land in i (every integer and bool kind), f (both float kinds) or s; an array keeps its
+// elements in the one list that fits its element kind.
 struct Value {
   uint32_t type = U8, arr_type = U8;
   int64_t i = 0;
   double f = 0;
   std::string s;
-  std::vector<int64_t> ai;
-  std::vector<double> af;
-  std::vector<std::string> as;
-  std::vector<Value> aa;
-  size_t size() const { return type == ARR ? ai.size() + af.size() + as.size() + aa.size() : 0; }
+  std::vector<int64_t> ints;
+  std::vector<double> floats;
+  std::vector<std::string> strings;
+  std::vector<Value> nested;
+  size_t size() const { return type == ARR ? ints.size() + floats.size() + strings.size() + nested.size() : 0; }
 };
 
 struct Tensor {
@@ -69,18 +71,17 @@ struct File {
   uint64_t size = 0, data_off = 0;
 };
 
-long long pread_full(int fd, void* dst, size_t len, uint64_t off) {
-  size_t got = 0;
-  while (got < len) {
-    const ssize_t r = pread(fd, (char*)dst + got, len - got, (off_t)(off + got));
-    if (r < 0) {
-      if (errno == EINTR) continue;
-      return -1;
-    }
-    if (r == 0) break;
-    got += (size_t)r;
+// Reads len bytes at file offset off; returns how many arrived (fewer only at the end of the file) or -1 on an error.
+long long read_at(int fd, void* dst, size_t len, uint64_t off) {
+  char* out = (char*)dst;
+  size_t left = len;
+  for (;;) {
+    if (left == 0) return (long long)len;
+    const ssize_t r = pread(fd, out, left, (off_t)off);
+    if (r > 0) { out += r; off += (uint64_t)r; left -= (size_t)r; continue; }
+    if (r == 0) return (long long)(len - left);
+    if (errno != EINTR) return -1;
   }
-  return (long long)got;
 }
 
 // Sequential reader over a file descriptor with a refillable window (headers of real models run to tens of MB of
@@ -98,7 +99,7 @@ struct Reader {
     const size_t want = (size_t)std::min<uint64_t>(std::max<uint64_t>(need, 1u << 20), size - pos);
     buf.resize(want);
     buf_off = pos;
-    if (pread_full(fd, buf.data(), want, pos) != (long long)want) return ok = false;
+    if (read_at(fd, buf.data(), want, pos) != (long long)want) return ok = false;
     return true;
   }
   template <class T>
@@ -148,10 +149,10 @@ bool read_value(Reader& r, uint32_t t, Value& v, int depth) {
   for (uint64_t k = 0; k < n; k++) {
     Value e;
     if (!read_value(r, v.arr_type, e, depth + 1)) return false;
-    if (v.arr_type == ARR) v.aa.push_back(std::move(e));
-    else if (v.arr_type == STR) v.as.push_back(std::move(e.s));
-    else if (v.arr_type == F32 || v.arr_type == F64) v.af.push_back(e.f);
-    else v.ai.push_back(e.i);
+    if (v.arr_type == ARR) v.nested.push_back(std::move(e));
+    else if (v.arr_type == STR) v.strings.push_back(std::move(e.s));
+    else if (v.arr_type == F32 || v.arr_type == F64) v.floats.push_back(e.f);
+    else v.ints.push_back(e.i);
   }
   return true;
 }
@@ -218,7 +219,10 @@ struct MsqGguf {
       const uint32_t t = r.get<uint32_t>();
       Value v;
       if (!r.ok || !read_value(r, t, v, 0)) { err = f.path + ": bad metadata value for key '" + key + "'"; return false; }
-      if (key == "general.alignment" && v.i > 0) file_align = (uint32_t)v.i;
+      if (key == "general.alignment") {
+        if (v.i < 1 || v.i > (1 << 20) || (v.i & (v.i - 1))) { err = f.path + ": general.alignment is not a power of two between 1 and 2^20"; return false; }
+        file_align = (uint32_t)v.i;
+      }
       if (!kv.count(key)) {  // merged across splits: the first occurrence wins
         kv_order.push_back(key);
         kv.emplace(std::move(key), std::move(v));
@@ -237,7 +241,13 @@ struct MsqGguf {
       t.split = split;
       if (!r.ok) { err = f.path + ": truncated tensor table"; return false; }
       const TypeRow* row = type_row(t.type);
-      const uint64_t nel = (uint64_t)t.ne[0] * t.ne[1] * t.ne[2] * t.ne[3];
+      uint64_t nel = 1;
+      bool fits = true;
+      for (int d = 0; d < 4; d++) {
+        if (t.ne[d] < 0 || (t.ne[d] > 0 && nel > (UINT64_MAX / 512) / (uint64_t)t.ne[d])) fits = false;  // x 292 bytes per block below
+        else nel *= (uint64_t)t.ne[d];
+      }
+      if (!fits) { err = f.path + ": tensor '" + t.name + "' has dimensions whose product overflows"; return false; }
       if (!row || t.ne[0] % row->blck) { err = f.path + ": tensor '" + t.name + "' has an unknown type or a ragged row"; return false; }
       t.nbytes = nel / row->blck * row->bytes;
       tensors.push_back(std::move(t));
@@ -245,8 +255,9 @@ struct MsqGguf {
     f.data_off = (r.pos + file_align - 1) / file_align * file_align;
     for (size_t k = first; k < tensors.size(); k++) {
       Tensor& t = tensors[k];
+      if (t.offset > f.size) { err = f.path + ": tensor '" + t.name + "' runs past the end of the file"; return false; }
       t.offset += f.data_off;  // absolute in its split
-      if (t.offset + t.nbytes > f.size) { err = f.path + ": tensor '" + t.name + "' runs past the end of the file"; return false; }
+      if (t.offset > f.size || t.nbytes > f.size - t.offset) { err = f.path + ": tensor '" + t.name + "' runs past the end of the file"; return false; }
       tindex.emplace(t.name, k);
     }
     return true;
@@ -274,7 +285,7 @@ int copy_file_to_device(hipStream_t st, int fd, uint64_t off, uint64_t len, uint
   for (int k = 0; pos < len && rc == MSQ_OK; k ^= 1) {
     const size_t n = (size_t)std::min<uint64_t>(kChunk, len - pos);
     if (hipEventSynchronize(done[k]) != hipSuccess) rc = fail(MSQ_ERR_HIP, "macseek quant: gguf: hipEventSynchronize failed");
-    else if (pread_full(fd, stage[k], n, off + pos) != (long long)n) rc = fail(MSQ_ERR_ARGUMENT, "macseek quant: gguf: short read at offset %llu", (unsigned long long)(off + pos));
+    else if (read_at(fd, stage[k], n, off + pos) != (long long)n) rc = fail(MSQ_ERR_ARGUMENT, "macseek quant: gguf: short read at offset %llu", (unsigned long long)(off + pos));
     else if (hipMemcpyAsync(dst + pos, stage[k], n, hipMemcpyHostToDevice, st) != hipSuccess || hipEventRecord(done[k], st) != hipSuccess)
       rc = fail(MSQ_ERR_HIP, "macseek quant: gguf: host to device copy failed");
     pos += n;
@@ -390,30 +401,30 @@ int64_t msq_gguf_arr_i64(const MsqGguf* g, const char* key, int64_t* out, int64_
   const Value* v = g && key ? g->find_kv(key) : nullptr;
   if (!v || v->type != ARR) return -1;
   int64_t n = 0;
-  if (!v->ai.empty()) { for (; n < (int64_t)v->ai.size() && n < cap; n++) out[n] = v->ai[n]; }
-  else { for (; n < (int64_t)v->af.size() && n < cap; n++) out[n] = (int64_t)v->af[n]; }
+  if (!v->ints.empty()) { for (; n < (int64_t)v->ints.size() && n < cap; n++) out[n] = v->ints[n]; }
+  else { for (; n < (int64_t)v->floats.size() && n < cap; n++) out[n] = (int64_t)v->floats[n]; }
   return n;
 }
 int64_t msq_gguf_arr_f64(const MsqGguf* g, const char* key, double* out, int64_t cap) {
   const Value* v = g && key ? g->find_kv(key) : nullptr;
   if (!v || v->type != ARR) return -1;
   int64_t n = 0;
-  if (!v->af.empty()) { for (; n < (int64_t)v->af.size() && n < cap; n++) out[n] = v->af[n]; }
-  else { for (; n < (int64_t)v->ai.size() && n < cap; n++) out[n] = (double)v->ai[n]; }
+  if (!v->floats.empty()) { for (; n < (int64_t)v->floats.size() && n < cap; n++) out[n] = v->floats[n]; }
+  else { for (; n < (int64_t)v->ints.size() && n < cap; n++) out[n] = (double)v->ints[n]; }
   return n;
 }
 const char* msq_gguf_arr_str(const MsqGguf* g, const char* key, int64_t index) {
   const Value* v = g && key ? g->find_kv(key) : nullptr;
-  return v && v->type == ARR && index >= 0 && (size_t)index < v->as.size() ? v->as[(size_t)index].c_str() : nullptr;
+  return v && v->type == ARR && index >= 0 && (size_t)index < v->strings.size() ? v->strings[(size_t)index].c_str() : nullptr;
 }
 // element `index` of a nested array (an array of arrays of integers): its length, and up to cap values
 int64_t msq_gguf_arr_nested_i64(const MsqGguf* g, const char* key, int64_t index, int64_t* out, int64_t cap) {
   const Value* v = g && key ? g->find_kv(key) : nullptr;
-  if (!v || v->type != ARR || index < 0 || (size_t)index >= v->aa.size()) return -1;
-  const Value& e = v->aa[(size_t)index];
+  if (!v || v->type != ARR || index < 0 || (size_t)index >= v->nested.size()) return -1;
+  const Value& e = v->nested[(size_t)index];
   int64_t n = 0;
-  for (; n < (int64_t)e.ai.size() && n < cap; n++) out[n] = e.ai[n];
-  return (int64_t)e.ai.size();
+  for (; n < (int64_t)e.ints.size() && n < cap; n++) out[n] = e.ints[n];
+  return (int64_t)e.ints.size();
 }
 
 int64_t msq_gguf_read(const MsqGguf* g, int tensor, uint64_t byte_off, void* dst, uint64_t len) {
@@ -422,7 +433,7 @@ int64_t msq_gguf_read(const MsqGguf* g, int tensor, uint64_t byte_off, void* dst
     fail(MSQ_ERR_ARGUMENT, "macseek quant: gguf_read: bad tensor index or range");
     return -1;
   }
-  return pread_full(g->files[t->split].fd, dst, (size_t)len, t->offset + byte_off);
+  return read_at(g->files[t->split].fd, dst, (size_t)len, t->offset + byte_off);
 }
 
 int msq_gguf_load_tensor(void* stream, const MsqGguf* g, int tensor, uint64_t byte_off, uint64_t len, const MsqBuffer* dst) {

@@ -162,10 +162,15 @@ __global__ __launch_bounds__(256) void router_fused_kernel(const float* __restri
     double sc;
     float key;
     score_key(v, bias[e], sc, key);
-    // Results cross to the selecting workgroup through device-scope atomic stores and loads only, which go to the
-    // level of the memory system that all CUs share; waiting for the stores' completion orders them before the counter
-    // increment. A release fence would do it too, at the price of writing back the whole L2 of this workgroup's XCD
-    // (measured: the launch takes 19 us with plain stores and a fence, 15 us with atomic stores and a fence).
+    // Hand-over to the selecting workgroup. Writer side: the three results are device-scope atomic stores (they are
+    // written through to the level of the memory system that all XCDs share, never parked in this XCD's L2), the
+    // wave waits until the memory system has acknowledged them (vmcnt(0)), and only then, after the workgroup
+    // barrier, is the counter incremented: a store that is acknowledged is visible to every device-scope load, so no
+    // record can be observed older than the count that announces it. This is the effect of a release fence without its
+    // price: a device-scope release writes back the whole L2 of this workgroup's XCD (measured: the launch takes
+    // 19 us with plain stores and a fence, 15 us with atomic stores and a fence, less without the fence). Reader side:
+    // the workgroup that draws the last count passes an acquire fence (cheap: it drops cached lines, writes nothing)
+    // and reads the records with device-scope atomic loads.
     uint64_t* r = (uint64_t*)(recs + e);
     __hip_atomic_store(logits + e, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     __hip_atomic_store(r, __builtin_bit_cast(uint64_t, sc), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -180,6 +185,7 @@ __global__ __launch_bounds__(256) void router_fused_kernel(const float* __restri
   }
   __syncthreads();
   if (!last) return;
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
   if (wave == 0) {
     const uint32_t epl = n_exp >> 6;
     float key[kMaxEpl];

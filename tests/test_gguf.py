@@ -125,6 +125,13 @@ def test_bad_files_are_rejected(tmp_path):
     W.write_gguf(p, [], [("r", 14, [100, 2], np.zeros(10, np.uint8))])
     with pytest.raises(q.QuantError, match="ragged row"):
         gguf.Gguf(p)
+    # an alignment that is no power of two; dimensions whose product does not fit 64 bits
+    W.write_gguf(p, [], [("r", 0, [4], np.zeros(16, np.uint8))], alignment=24)
+    with pytest.raises(q.QuantError, match="general.alignment is not a power of two"):
+        gguf.Gguf(p)
+    W.write_gguf(p, [], [("r", 0, [1 << 40, 1 << 40], np.zeros(16, np.uint8))])
+    with pytest.raises(q.QuantError, match="product overflows"):
+        gguf.Gguf(p)
 
 
 def test_expert_layout(tmp_path):  # src/store/experts.mm:36-56
