@@ -682,11 +682,13 @@ def bench_matmul(torch, args):
     from macseek_amd import quant as q
     dev = torch.device("cuda:0")
     rows_out = []
-    # n = 2048: dequantize-then-GEMM; n = 256 and 512: the fused kernel (mm_fused_kernel)
-    for n, t, name, rows, cols in ((2048, q.QType.Q6_K, "Q6_K", 1536, 7168), (2048, q.QType.Q5_K, "Q5_K", 512, 7168),
-                                   (2048, q.QType.IQ4_NL, "IQ4_NL", 7168, 4096), (2048, q.QType.BF16, "BF16", 384, 7168),
-                                   (512, q.QType.Q6_K, "Q6_K", 1536, 7168), (256, q.QType.Q6_K, "Q6_K", 1536, 7168),
-                                   (512, q.QType.IQ4_NL, "IQ4_NL", 7168, 4096), (256, q.QType.IQ4_NL, "IQ4_NL", 7168, 4096)):
+    # n = 2048 and 512: dequantize-then-GEMM; n <= 128 (<= 256 on matrices of at most 2048 rows): the fused kernel
+    # (mm_fused_kernel); "route" names which one served the case
+    cases = [(2048, q.QType.Q6_K, "Q6_K", 1536, 7168), (2048, q.QType.Q5_K, "Q5_K", 512, 7168),
+             (2048, q.QType.IQ4_NL, "IQ4_NL", 7168, 4096), (2048, q.QType.BF16, "BF16", 384, 7168)]
+    for n in (512, 256, 128, 64, 16):
+        cases += [(n, q.QType.Q6_K, "Q6_K", 1536, 7168), (n, q.QType.IQ4_NL, "IQ4_NL", 7168, 4096)]
+    for n, t, name, rows, cols in cases:
         if int(t) == 30:
             W = (torch.randn(rows * cols, device=dev) * 0.02).to(torch.bfloat16).view(torch.uint8)
         else:
@@ -707,7 +709,9 @@ def bench_matmul(torch, args):
         torch.cuda.synchronize()
         ms = a.elapsed_time(b) / reps
         flops = 2.0 * n * rows * cols
-        rows_out.append({"type": name, "rows": rows, "cols": cols, "n": n, "us_per_call": ms * 1e3, "TFLOPs": flops / (ms * 1e-3) / 1e12})
+        fused = n <= 128 or (n <= 256 and rows <= 2048)
+        rows_out.append({"type": name, "rows": rows, "cols": cols, "n": n, "us_per_call": ms * 1e3, "TFLOPs": flops / (ms * 1e-3) / 1e12,
+                         "route": "mm_fused_kernel" if fused else "dequant + rocBLAS"})
     head = rows_out[0]
     n = 2048
     cpu = None
@@ -725,7 +729,7 @@ def bench_matmul(torch, args):
     return {"value": head["TFLOPs"], "ms_per_step": head["us_per_call"] * 1e-3, "dtype": "f16 x f16 MFMA (weights and activations rounded to fp16), f32 accumulate",
             "config": {"workload": "prefill matmul, 2048 tokens, BASELINE configs[4] shapes; one step = one msq_matmul call of the Q6_K 1536x7168 case", "cases": rows_out},
             "roofline": {"bound": "mfma", "achieved": head["TFLOPs"], "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": head["TFLOPs"] / MFMA_PEAK_TFLOPS,
-                         "traffic": None, "kernel": "f32_to_f16_kernel + dequant_kernel<Q6_K, fp16> + rocBLAS fp16 GEMM (whole call; up to 512 tokens: mm_fused_kernel, see cases)", "flops_per_launch": 2.0 * n * 1536 * 7168,
+                         "traffic": None, "kernel": "f32_to_f16_kernel + dequant_kernel<Q6_K, fp16> + rocBLAS fp16 GEMM (whole call; few tokens: mm_fused_kernel, see cases)", "flops_per_launch": 2.0 * n * 1536 * 7168,
                          "avg_launch_us": head["us_per_call"]},
             "cpu_baseline": cpu}
 

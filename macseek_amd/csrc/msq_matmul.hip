@@ -2,15 +2,18 @@
 // host code src/kernels/quant.mm:159-248, kernels src/kernels/quant_mm.metal:81-185).
 //
 // The reference multiplies fp16 activations by weight tiles dequantized to fp16 inside its GEMM kernel and, from
-// n >= 512, dequantizes the whole matrix to fp16 once and runs a dense GEMM (quant.mm:204-221). The same split is used
-// here. Up to 512 tokens: mm_fused_kernel (msq_mm.cuh) decodes each weight tile once per 128 tokens straight into
-// matrix-core fragments -- no fp16 copy of W or X, no scratch, the call only enqueues. Above: the bit-exact
-// dequantizer writes W as fp16 into library-owned scratch (22 MB for a 7168 x 1536 projection, a few microseconds at
-// 8 TB/s) and the product is a plain fp16 x fp16 -> fp32 GEMM left to rocBLAS. That scratch only grows: a larger
-// request allocates a new block and the old one stays alive until the process ends (work already enqueued may still
-// read it), so growing never waits for the stream; it does allocate, so the first call of a larger shape must not be
-// inside a stream capture, and like the reference's scratch (docs/modules/quant.md:265-268) it is shared by all calls:
-// calls above 512 tokens must be enqueued on one stream at a time.
+// n >= 512, dequantizes the whole matrix to fp16 once and runs a dense GEMM (quant.mm:204-221). The same two routes
+// exist here; the switch between them sits where they were measured to cross (use_fused below). Fused route:
+// mm_fused_kernel (msq_mm.cuh) decodes each weight tile straight into matrix-core fragments -- no fp16 copy of W or X,
+// no scratch, the call only enqueues; K is cut into slices that are summed into Y with fp32 atomic adds when the tiles
+// alone would not fill the device (then the last bits of Y depend on the order in which the slices finish; MSQ_MM_SPLITK=1
+// keeps one slice per tile and with it bit-reproducible sums). Materialising route: the bit-exact dequantizer writes
+// W as fp16 into library-owned scratch (22 MB for a 7168 x 1536 projection, a few microseconds at 8 TB/s) and the
+// product is a plain fp16 x fp16 -> fp32 GEMM left to rocBLAS. That scratch only grows: a larger request allocates a
+// new block and the old one stays alive until the process ends (work already enqueued may still read it), so growing
+// never waits for the stream; it does allocate, so the first call of a larger shape must not be inside a stream
+// capture, and like the reference's scratch (docs/modules/quant.md:265-268) it is shared by all calls: calls on this
+// route must be enqueued on one stream at a time.
 #include <rocblas/rocblas.h>
 
 #include <cstdlib>
@@ -39,11 +42,15 @@ std::mutex g_mu;
 Scratch g_x16, g_w16;
 std::vector<void*> g_retired;  // outgrown blocks: kept until the process ends
 rocblas_handle g_blas = nullptr;
-// tokens up to which the fused kernel serves the call (the reference's threshold is 512, quant.mm:204); MSQ_MM_FUSED_MAX
-// overrides it for experiments
-int fused_max_tokens() {
-  static const int v = [] { const char* e = getenv("MSQ_MM_FUSED_MAX"); return e && *e ? atoi(e) : 512; }();
-  return v;
+// Which calls the fused kernel serves. The reference switches to dequantize-then-GEMM at 512 tokens (quant.mm:204); here
+// the switch sits where the two routes were measured to cross on MI355X: the fused kernel wins up to 128 tokens on every
+// matrix tried (Q6_K 1536x7168 at 128 tokens: 25 us against 36 us; 16 tokens: 9.5 against 30) and up to 256 tokens on
+// matrices of at most 2048 rows; above, the materialising route is ahead (IQ4_NL 7168x4096 at 512 tokens: 63 us against
+// 124). MSQ_MM_FUSED_MAX = N makes the switch "up to N tokens" for every matrix (0: never fused).
+bool use_fused(int n, int rows) {
+  static const int forced = [] { const char* e = getenv("MSQ_MM_FUSED_MAX"); return e && *e ? atoi(e) : -1; }();
+  if (forced >= 0) return n <= forced;
+  return n <= 128 || (n <= 256 && rows <= 2048);
 }
 
 // at least `bytes` of device memory in s (>= 64 MiB like the reference's, quant.mm:176-183)
@@ -113,30 +120,53 @@ int gemm_f16(hipStream_t st, const uint16_t* W16, const uint16_t* X16, float* Y,
   return MSQ_OK;
 }
 
+__global__ __launch_bounds__(256) void zero_f32_kernel(float* __restrict__ y, size_t n) {
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) y[i] = 0.f;
+}
+
+// K slices per tile: MSQ_MM_SPLITK = 1 keeps every sum inside one workgroup (bit-reproducible results), 0 / unset lets
+// the launcher choose
+int splitk_limit() {
+  static const int v = [] { const char* e = getenv("MSQ_MM_SPLITK"); return e && *e ? atoi(e) : 0; }();
+  return v;
+}
+
 template <class F, bool X_F32>
-int launch_mm_t(hipStream_t st, const MmArgs& a) {
-  auto go = [&](auto wv_tag, auto tm_tag) {
+int launch_mm_t(hipStream_t st, MmArgs a) {
+  const long cus = device_info().cus;
+  const uint32_t nstages = a.cols / kMmKStage;
+  auto go = [&](auto wv_tag, auto tm_tag) -> int {
     constexpr int WV = decltype(wv_tag)::value, TM = decltype(tm_tag)::value;
     const size_t lds = (size_t)F::LDS_WORDS * 4 + 2 * (size_t)16 * TM * kMmPitch;
-    allow_large_lds(mm_fused_kernel<F, WV, TM, X_F32>, lds);
-    hipLaunchKernelGGL((mm_fused_kernel<F, WV, TM, X_F32>), dim3((a.rows + 16 * WV - 1) / (16 * WV), (a.n + 16 * TM - 1) / (16 * TM)),
-                       dim3(64 * WV), lds, st, a);
+    const int rc = allow_large_lds(mm_fused_kernel<F, WV, TM, X_F32>, lds);
+    if (rc != MSQ_OK) return rc;
+    const long gx = (a.rows + 16 * WV - 1) / (16 * WV), gy = (a.n + 16 * TM - 1) / (16 * TM);
+    // Few tiles: the K range is cut into slices (at least two stages each) until there are about two workgroups per CU;
+    // a workgroup's K loop is a chain of stage latencies, so a call is as slow as its longest chain. The slices of a tile
+    // meet in Y through fp32 atomic adds, in whatever order they finish.
+    long kz = std::min<long>((2 * cus + gx * gy - 1) / (gx * gy), std::max<long>(1, nstages / 2));
+    if (splitk_limit() > 0) kz = std::min<long>(kz, splitk_limit());
+    a.slice_stages = (uint32_t)((nstages + kz - 1) / kz);
+    kz = (nstages + a.slice_stages - 1) / a.slice_stages;
+    a.atomic_out = kz > 1 ? 1u : 0u;
+    if (a.atomic_out && !a.accumulate) {
+      const size_t cnt = (size_t)a.n * a.rows;
+      hipLaunchKernelGGL(zero_f32_kernel, dim3((unsigned)((cnt + 255) / 256)), dim3(256), 0, st, a.Y, cnt);
+    }
+    hipLaunchKernelGGL((mm_fused_kernel<F, WV, TM, X_F32>), dim3((unsigned)gx, (unsigned)gy, (unsigned)kz), dim3(64 * WV), lds, st, a);
+    MSQ_HIP(hipGetLastError());
+    return MSQ_OK;
   };
-  // the largest tile (a weight tile is decoded once per workgroup, an activation tile staged once) that still gives
-  // every CU a workgroup; with fewer, the call is bound by the latency of one workgroup's K loop
-  const long cus = device_info().cus;
+  // token tiles per workgroup: what the call's tokens need, at most eight; eight waves when that still leaves a
+  // workgroup per CU, four otherwise
   auto wgs = [&](long wv, long tm) { return ((a.rows + 16 * wv - 1) / (16 * wv)) * ((a.n + 16 * tm - 1) / (16 * tm)); };
   using I1 = std::integral_constant<int, 1>; using I2 = std::integral_constant<int, 2>;
   using I4 = std::integral_constant<int, 4>; using I8 = std::integral_constant<int, 8>;
-  const long want = cus;
-  if (a.n > 64 && wgs(8, 8) >= want) go(I8{}, I8{});
-  else if (a.n > 64 && wgs(4, 8) >= want) go(I4{}, I8{});
-  else if (a.n > 32 && wgs(4, 4) >= want) go(I4{}, I4{});
-  else if (a.n > 16 && wgs(4, 2) >= want) go(I4{}, I2{});
-  else if (a.n > 16 && wgs(4, 1) < want) go(I4{}, I2{});
-  else go(I4{}, I1{});
-  MSQ_HIP(hipGetLastError());
-  return MSQ_OK;
+  if (a.n > 64) return wgs(8, 8) >= cus ? go(I8{}, I8{}) : go(I4{}, I8{});
+  if (a.n > 32) return go(I4{}, I4{});
+  if (a.n > 16) return go(I4{}, I2{});
+  return go(I4{}, I1{});
 }
 template <bool X_F32>
 int launch_mm(hipStream_t st, int t, const MmArgs& a) {
@@ -192,7 +222,7 @@ int msq_matmul_h(void* stream, int t, const MsqBuffer* W, int rows, int cols, co
     return fail(MSQ_ERR_ARGUMENT, "macseek quant: matmul: buffer missing, too small or misaligned (type %s rows %d cols %d n %d)",
                 msq_type_name_of(t), rows, cols, n);
   hipStream_t st = (hipStream_t)stream;
-  if (n <= fused_max_tokens()) {
+  if (use_fused(n, rows)) {
     const MmArgs a{bptr(X16), bptr(W), (float*)bptr_mut(Y), (uint32_t)n, (uint32_t)rows, (uint32_t)cols, (uint32_t)xs,
                    (uint32_t)msq_type_row_bytes(t, cols), accumulate ? 1u : 0u};
     return launch_mm<false>(st, t, a);
@@ -209,7 +239,7 @@ int msq_matmul(void* stream, int t, const MsqBuffer* W, int rows, int cols, cons
     return fail(MSQ_ERR_ARGUMENT, "macseek quant: matmul: buffer missing, too small or misaligned (type %s rows %d cols %d n %d)",
                 msq_type_name_of(t), rows, cols, n);
   hipStream_t st = (hipStream_t)stream;
-  if (n <= fused_max_tokens()) {
+  if (use_fused(n, rows)) {
     const MmArgs a{bptr(X), bptr(W), (float*)bptr_mut(Y), (uint32_t)n, (uint32_t)rows, (uint32_t)cols, (uint32_t)cols,
                    (uint32_t)msq_type_row_bytes(t, cols), accumulate ? 1u : 0u};
     return launch_mm<true>(st, t, a);  // X is rounded to fp16 on its way into LDS

@@ -3,8 +3,9 @@
 // src/kernels/quant_mm.metal:87-115). Numerics are the reference's: activations and weights rounded to fp16, fp32
 // accumulation (quant.hpp:36-39).
 //
-// A workgroup of WV waves owns 16 WV weight rows x 16 TM tokens (the host picks the largest tile that still gives the
-// device a workgroup per CU: below that the call is bound by the latency of a workgroup's K loop). A wave owns one 16-row tile of W: per K step
+// A workgroup of WV waves owns 16 WV weight rows x 16 TM tokens of one K slice (blockIdx.z). A workgroup's K loop is a
+// chain of stage latencies and a small matrix has few tiles, so the host cuts K into slices until the device holds about
+// two workgroups per CU; the slices of a tile then meet in Y through fp32 atomic adds. A wave owns one 16-row tile of W: per K step
 // (32 columns) it decodes the lane's eight weights into exact fp16 payloads + fp32 scale (the fragment decoders of
 // msq_mfma.cuh), rounds scale * payload (+ add) to fp16 once (v_fma_mix: fp32 arithmetic, one rounding -- the value
 // the reference's dequantized tile holds) and feeds TM matrix instructions, one per token tile. The activation tile
@@ -20,6 +21,8 @@ struct MmArgs {
   const uint8_t* W;    // raw block rows
   float* Y;            // [n][rows]
   uint32_t n, rows, cols, x_stride, row_bytes, accumulate;
+  uint32_t slice_stages;  // 128-column stages per K slice (blockIdx.z picks the slice)
+  uint32_t atomic_out;    // several K slices: every slice adds its tile to Y with fp32 atomics (Y holds zeros or the sum to add to)
 };
 
 // F32 and BF16 weight rows as fp16 payloads (the matmul multiplies every type as fp16)
@@ -81,6 +84,7 @@ __global__ __launch_bounds__(64 * WV) void mm_fused_kernel(const MmArgs a) {
   const uint32_t m0 = blockIdx.y * TOK;
   const gptr_t wrow = as_global(a.W) + (size_t)min(row, a.rows - 1) * a.row_bytes;
   const uint32_t nstages = a.cols / kMmKStage;
+  const uint32_t st0 = blockIdx.z * a.slice_stages, st1 = min(st0 + a.slice_stages, nstages);  // this workgroup's K slice
 
   // activation stage loader: granule g = (token g / 16, columns 8 (g % 16) ..); tokens past n repeat the last one
   u32x4 pa[AG][X_F32 ? 2 : 1];
@@ -128,7 +132,7 @@ __global__ __launch_bounds__(64 * WV) void mm_fused_kernel(const MmArgs a) {
     }
   };
 
-  a_issue(0);
+  a_issue(st0);
   F::fill_lds(tbl, (int)tid, NT);
   a_store(0);
   __syncthreads();
@@ -138,8 +142,9 @@ __global__ __launch_bounds__(64 * WV) void mm_fused_kernel(const MmArgs a) {
   for (int t = 0; t < TM; t++) acc[t] = f4_t{0.f, 0.f, 0.f, 0.f};
   uint32_t touch = 0;
 
-  for (uint32_t st = 0; st < nstages; st++) {
-    const uint32_t sn = st + 1 < nstages ? st + 1 : st;  // the last stage fetches itself again: no branch around the loads
+  for (uint32_t st = st0; st < st1; st++) {
+    const uint32_t sn = st + 1 < st1 ? st + 1 : st;  // the last stage fetches itself again: no branch around the loads
+    const uint32_t buf = (st - st0) & 1u;
     a_issue(sn);
     // the next stage's weight bytes are touched now (a lane per 32 bytes of its row's stage), so that the fragment
     // loads of that stage, which sit right in front of their decode, find them in the nearest cache
@@ -149,7 +154,7 @@ __global__ __launch_bounds__(64 * WV) void mm_fused_kernel(const MmArgs a) {
       touch ^= *(const MSQ_GLOBAL uint32_t*)(wrow - ((uintptr_t)wrow & 3u) + off);
       if (stage_bytes > 128u) touch ^= *(const MSQ_GLOBAL uint32_t*)(wrow - ((uintptr_t)wrow & 3u) + (min(off + 128u, a.row_bytes - 4u) & ~3u));
     }
-    const uint8_t* arow = abuf + (st & 1u) * ABUF + n16 * kMmPitch + 16u * q;
+    const uint8_t* arow = abuf + buf * ABUF + n16 * kMmPitch + 16u * q;
     // the four steps' fragments first: their loads are then in flight together (one trip to memory per stage)
     constexpr int NS = kMmKStage / 32;
     uint32_t h[NS][4];
@@ -185,7 +190,7 @@ __global__ __launch_bounds__(64 * WV) void mm_fused_kernel(const MmArgs a) {
         acc[t] = mfma_f16(x, h[js], acc[t]);
       }
     }
-    a_store((st & 1u) ^ 1u);  // the other buffer was last read one stage ago, before the previous barrier
+    a_store(buf ^ 1u);  // the other buffer was last read one stage ago, before the previous barrier
     __syncthreads();
   }
 
@@ -199,7 +204,8 @@ __global__ __launch_bounds__(64 * WV) void mm_fused_kernel(const MmArgs a) {
         const uint32_t tok = m0 + 16u * t + 4u * q + i;
         if (tok < a.n) {
           float* y = a.Y + (size_t)tok * a.rows + row;
-          *y = a.accumulate ? *y + acc[t][i] : acc[t][i];
+          if (a.atomic_out) __hip_atomic_fetch_add(y, acc[t][i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          else *y = a.accumulate ? *y + acc[t][i] : acc[t][i];
         }
       }
     }

@@ -21,8 +21,12 @@ CASES = [  # (type, rows, cols, n, accumulate): tests/test_quant_matmul.mm:18-25
     (O.IQ2_XXS, 5120, 2304, 37, True), (O.IQ1_S, 300, 2304, 129, False), (O.BF16, 512, 5120, 48, False),
     (O.F16, 256, 1280, 70, False), (O.F32, 384, 5120, 36, False),
     (O.IQ4_NL, 1024, 4096, 32, False), (O.Q6_K, 48, 256, 1, True),
-    # both sides of the 512-token switch from the fused kernel to dequantize-then-GEMM (quant.mm:204)
-    (O.Q6_K, 384, 1024, 512, False), (O.Q5_K, 272, 1024, 513, True), (O.IQ4_NL, 96, 512, 700, False),
+    # both sides of the switches from the fused kernel to dequantize-then-GEMM (the reference's sits at 512 tokens,
+    # quant.mm:204): 128 tokens for matrices of more than 2048 rows, 256 tokens below
+    (O.IQ4_NL, 2304, 512, 128, False), (O.IQ4_NL, 2304, 512, 129, True), (O.Q6_K, 384, 1024, 256, False),
+    (O.Q5_K, 272, 1024, 257, True), (O.Q6_K, 384, 1024, 512, False), (O.IQ4_NL, 96, 512, 700, False),
+    # the fused kernel with one K slice per tile (two stages of K: nothing to cut) and with many (the cases above)
+    (O.Q8_0, 16384, 256, 100, True),
 ]
 
 
