@@ -148,14 +148,22 @@ struct DecIQ1SQ {
       // low byte of qh: bits 0..2 = h0, bits 3..5 = h1, bits 6..7 = low bits of h2
       lds[LUT_LO_AT + b] = ((b & 7u) << 3) | (((b >> 3) & 7u) << 11) | (((b >> 6) & 3u) << 19);
     }
-    for (uint32_t i0 = tid, j = 0; i0 < ITEMS; i0 += nt, j++) {
-      uint4 v = r.v[0];
-      if (j == 1) v = r.v[1];
-      if (j >= 2) v = ((const uint4*)g_tbl_iq1s8.w)[i0];  // workgroups of fewer than 1024 threads
-      // image byte o = 16 i0 = (b << 7) | (sign << 6) | (h << 3) goes to LDS byte (b << 8) | (c << 7) | (o & 127)
-      const uint32_t o = 16u * i0, at = (((o & ~127u) << 1) | (o & 127u)) >> 2;
+    // image byte o = 16 i = (b << 7) | (sign << 6) | (h << 3) goes to LDS byte (b << 8) | (c << 7) | (o & 127)
+    auto put = [&](uint32_t i, const uint4& v) {
+      const uint32_t o = 16u * i, at = (((o & ~127u) << 1) | (o & 127u)) >> 2;
       *(uint4*)(lds + GRID_AT + at) = v;
       *(uint4*)(lds + GRID_AT + at + 32u) = v;
+    };
+#pragma unroll
+    for (int j = 0; j < 2; j++)
+      if (tid + j * nt < ITEMS) put(tid + j * nt, r.v[j]);
+    if (2u * nt < ITEMS) {  // workgroups of fewer than 1024 threads fetch the rest here
+      // (the index is recomputed behind a barrier the compiler cannot look through: hoisted to the kernel's start, this
+      // loop's addresses cost every thread of the usual 1024-thread launch five spilled registers -- 4 MB of scratch
+      // writes per launch)
+      uint32_t t2 = tid;
+      asm volatile("" : "+v"(t2));
+      for (uint32_t i0 = t2 + 2u * nt; i0 < ITEMS; i0 += nt) put(i0, ((const uint4*)g_tbl_iq1s8.w)[i0]);
     }
   }
   __device__ static void fill_lds(uint32_t* lds, uint32_t tid, uint32_t nt) { finish_tables(lds, issue_tables(tid, nt), tid, nt); }
