@@ -31,9 +31,9 @@ HBM_PEAK_GBPS = 8000.0
 
 # HBM bytes per launch of the decode gate/up kernel, from the FETCH_SIZE / WRITE_SIZE counter runs of this workload
 # (KiB per dispatch, scaled by what the same counters read for a 1 GiB copy: x2.000 and x1.000): 42.91 MB + 0.06 MB
-GU_TRAFFIC_BYTES = 42970419
+GU_TRAFFIC_BYTES = 47006028
 # HBM bytes of the three launches of the prefill gate/up GEMM together (same counters, same scaling), configs[3]
-PF_GU_TRAFFIC_BYTES = None
+PF_GU_TRAFFIC_BYTES = 4288842222
 
 
 def cores():
@@ -510,10 +510,11 @@ def bench_issue_probe(torch, args):
     cus = torch.cuda.get_device_properties(0).multi_processor_count
     sink = torch.zeros(4 * cus * 4, dtype=torch.uint8, device=dev)
     sb = q.Buffer.of(sink).c()
-    VALU, MFMA16, MFMA4, MFMA8, LDS, VINT = 1, 2, 4, 8, 16, 32
+    VALU, MFMA16, MFMA4, MFMA8, LDS, VINT, VPK, VFMA = 1, 2, 4, 8, 16, 32, 64, 128
     mixes = [("valu32", VALU), ("mfma16_f16_x8", MFMA16), ("mfma_fp4_fp6_x8", MFMA4), ("mfma_fp8_x8", MFMA8), ("lds_b32_x16", LDS),
              ("valu32+mfma16_f16_x8", VALU | MFMA16), ("valu32+mfma_fp4_fp6_x8", VALU | MFMA4), ("valu32+lds_b32_x16", VALU | LDS),
-             ("valu32+lds_b32_x16+mfma_fp4_fp6_x8", VALU | LDS | MFMA4), ("vint32", VINT), ("vint32+mfma16_f16_x8", VINT | MFMA16)]
+             ("valu32+lds_b32_x16+mfma_fp4_fp6_x8", VALU | LDS | MFMA4), ("vint32", VINT), ("vint32+mfma16_f16_x8", VINT | MFMA16),
+             ("vpk32", VPK), ("vpk32+mfma16_f16_x8", VPK | MFMA16), ("vfma32", VFMA), ("vfma32+mfma16_f16_x8", VFMA | MFMA16)]
     iters = 4096
     rows = []
     for wps, grid, block in ((1, cus, 256), (2, cus, 512), (4, cus, 1024), (8, 2 * cus, 1024)):

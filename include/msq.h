@@ -7,8 +7,9 @@
  *     ordered by the stream, so the reference's explicit Enc::barrier() between them has no counterpart.
  *   - weights are raw GGUF block rows: an [in -> out] matrix is rows = out rows of cols = in elements
  *     (quant.hpp:4); weight bases need 4-byte alignment only, activations / outputs 16-byte alignment
- *     (docs/modules/quant.md:27-30). Activations must be finite and inside the fp16 range (they are staged as
- *     fp16 pairs for the block formats, as the reference does for its n > 1 paths).
+ *     (docs/modules/quant.md:27-30). Activations must be finite and inside the fp16 range, |x| <= 65504 (the block
+ *     formats stage them as fp16 pairs, as the reference does for its n > 1 paths; larger values turn into
+ *     infinities). MoE routing weights up to 5 keep the down projection's inputs inside that range.
  *   - all buffers are caller-owned device memory; MsqBuffer mirrors ms::Buffer {buf, off, size}
  *     (src/core/metal.hpp:11-18).
  *   - misuse is reported, not aborted: functions return 0 on success or a negative MSQ_ERR_* code and leave a
@@ -109,14 +110,18 @@ int msq_f32_to_f16(void* stream, const MsqBuffer* X, const MsqBuffer* X16, size_
 
 /* reference: ms::q::encode_matmul_h (quant.hpp:43-45, quant.mm:193-238). Prefill matmul
  * Y[n x rows] (+)= X16[n x x_stride] . W^T, X16 fp16 (x_stride = cols if 0), Y F32, any n >= 1, cols % 128 == 0.
- * Weights are rounded to fp16 and products accumulate in fp32, the reference's numerics (quant.hpp:36-39). The fp16
- * copy of W lives in scratch the library owns and grows on demand (reference: quant.mm:176-184): calls sharing it
- * must be enqueued on one stream at a time, and a call that grows it synchronises that stream and allocates. */
+ * Weights are rounded to fp16 and products accumulate in fp32, the reference's numerics (quant.hpp:36-39).
+ * Up to 128 tokens (256 on matrices of at most 2048 rows; MSQ_MM_FUSED_MAX=N in the environment: up to N) a fused
+ * kernel serves the call: nothing is allocated and the call only enqueues. When the matrix has few tiles it sums K
+ * slices into Y with fp32 atomic adds, so the last bits of Y can differ between runs (MSQ_MM_SPLITK=1: one slice,
+ * reproducible). Above, an fp16 copy of W goes to scratch that the library owns (reference: quant.mm:176-184): that
+ * scratch only grows (a larger shape allocates a new block, never waits for the stream; inside a stream capture a call
+ * that would have to grow it fails with MSQ_ERR_SCRATCH), and calls sharing it must be enqueued on one stream at a time. */
 int msq_matmul_h(void* stream, int qtype, const MsqBuffer* W, int rows, int cols, const MsqBuffer* X16, const MsqBuffer* Y,
                  int n, int accumulate, int x_stride);
 
 /* reference: ms::q::encode_matmul (quant.hpp:40-41, quant.mm:240-248): converts X (F32 [n x cols], 16-byte aligned)
- * into library-owned fp16 scratch, then msq_matmul_h. */
+ * into library-owned fp16 scratch, then msq_matmul_h; the fused kernel reads the F32 activations as they are. */
 int msq_matmul(void* stream, int qtype, const MsqBuffer* W, int rows, int cols, const MsqBuffer* X, const MsqBuffer* Y, int n,
                int accumulate);
 
@@ -134,8 +139,9 @@ int msq_bw_probe(void* stream, const MsqBuffer* src, size_t bytes, const MsqBuff
 /* Instruction-issue probe (no reference counterpart; the reference prices its kernels against a bandwidth probe only):
  * `grid` workgroups of `block` threads each run `iters` iterations of a fixed instruction group per wave. `mask` ORs
  * the groups: 1 = 32 vector ops, 2 = 8 fp16 16x16x32 matrix ops, 4 = 8 block-scaled fp4 x fp6 16x16x128 matrix ops,
- * 8 = 8 fp8 16x16x128 matrix ops, 16 = 16 random 32-bit LDS reads, 32 = 32 integer vector ops; supported mixes: 1, 2,
- * 4, 8, 16, 32, 1|2, 1|4, 1|16, 1|4|16, 32|2. `sink` holds >= 4 * grid bytes. The benchmark turns the timings into ns per issue slot. */
+ * 8 = 8 fp8 16x16x128 matrix ops, 16 = 16 random 32-bit LDS reads, 32 = 32 integer vector ops, 64 = 32 packed-fp16
+ * multiplies, 128 = 32 fp32 fused multiply-adds; supported mixes: 1, 2, 4, 8, 16, 32, 64, 128, 1|2, 1|4, 1|16, 1|4|16,
+ * 32|2, 64|2, 128|2. `sink` holds >= 4 * grid bytes. The benchmark turns the timings into ns per issue slot. */
 int msq_issue_probe(void* stream, int mask, int grid, int block, int iters, const MsqBuffer* sink);
 
 /* ---------------------------------------------------------------------------------------------- MoE, one token */
@@ -238,13 +244,15 @@ typedef struct MsqMoePrefillArgs {
 
 /* reference: ms::q::moe_prefill_scratch_bytes (quant.hpp:117, quant.mm:427-431). Layout (caller-owned device memory):
  * header (expert pointer table, offsets, token-tile table) | Xg fp16[(total+n) x dim] | H fp16[(total+n) x inter] |
- * Z f32[(total+n) x dim]. The header is filled by an asynchronous copy on the stream, so unlike the reference the
- * scratch may still be in use by earlier work on the same stream. */
+ * Z f32[(total+n) x dim]. The header is written by small kernels that carry it in their arguments, so unlike the
+ * reference the scratch may still be in use by earlier work on the same stream. */
 size_t msq_moe_prefill_scratch_bytes(int total_entries, int n_tokens, int n_exp, int dim, int inter);
 
 /* reference: ms::q::encode_moe_prefill (quant.hpp:118, quant.mm:433-612). Enqueues gather, grouped gate/up GEMM +
- * SwiGLU, grouped down GEMM and the ordered reduction into Y. Activations and H are staged as fp16 (as in the
- * reference), weights are used exactly. The result is bit-identical from run to run. n_tokens <= 0 returns MSQ_OK and
+ * SwiGLU, grouped down GEMM and the ordered reduction into Y. Activations and H are staged as fp16 and weights enter
+ * the matrix instructions as fp16 (the whole weight rounded once), as in the reference's tiles. The call only enqueues
+ * (no host copy, no wait, no allocation) and can be captured in a HIP graph; `offs` (host memory) is read at call time and
+ * travels to the device inside kernel arguments. The result is bit-identical from run to run. n_tokens <= 0 returns MSQ_OK and
  * does nothing (quant.mm:435). */
 int msq_moe_prefill(void* stream, const MsqMoePrefillArgs* a);
 

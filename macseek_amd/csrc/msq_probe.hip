@@ -11,7 +11,10 @@
 //   MFMA8  8 x the same instruction with fp8 A and B operands
 //   LDS    16 x ds_read_b32 at per-lane pseudo-random addresses inside a 8 KB table (+ one v_xor per value read)
 //   VINT   32 x v_and_or_b32 (integer only: nothing that could share hardware with the matrix cores)
-// and the mixes VALU+MFMA16, VALU+MFMA4, VALU+LDS, VALU+LDS+MFMA4, VINT+MFMA16 (groups interleaved 4 : 1 in program order).
+//   VPK    32 x v_pk_mul_f16 (packed fp16 arithmetic, four chains)
+//   VFMA   32 x v_fma_f32 (four chains)
+// and the mixes VALU+MFMA16, VALU+MFMA4, VALU+LDS, VALU+LDS+MFMA4, VINT+MFMA16, VPK+MFMA16, VFMA+MFMA16 (groups
+// interleaved 4 : 1 in program order).
 #include "msq_host.h"
 
 namespace msq {
@@ -21,7 +24,7 @@ typedef _Float16 ph2_t __attribute__((ext_vector_type(2)));
 typedef float pf4_t __attribute__((ext_vector_type(4)));
 typedef int pi8_t __attribute__((ext_vector_type(8)));
 
-enum { P_VALU = 1, P_MFMA16 = 2, P_MFMA4 = 4, P_MFMA8 = 8, P_LDS = 16, P_VINT = 32 };
+enum { P_VALU = 1, P_MFMA16 = 2, P_MFMA4 = 4, P_MFMA8 = 8, P_LDS = 16, P_VINT = 32, P_VPK = 64, P_VFMA = 128 };
 
 template <int MASK>
 __global__ __launch_bounds__(1024) void issue_probe_kernel(uint32_t* sink, uint32_t iters, uint32_t seed) {
@@ -62,6 +65,21 @@ __global__ __launch_bounds__(1024) void issue_probe_kernel(uint32_t* sink, uint3
         for (int j = 0; j < 4; j++) {
           u[(g + j) & 3] = (u[(g + j) & 3] & 0x00FFF0F0u) | u[(g + j + 1) & 3];
           asm volatile("" : "+v"(u[(g + j) & 3]));
+        }
+      }
+      if constexpr (MASK & P_VPK) {
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+          const ph2_t r = __builtin_bit_cast(ph2_t, u[(g + j) & 3]) * __builtin_bit_cast(ph2_t, w);  // one v_pk_mul_f16
+          u[(g + j) & 3] = __builtin_bit_cast(uint32_t, r);
+          asm volatile("" : "+v"(u[(g + j) & 3]));
+        }
+      }
+      if constexpr (MASK & P_VFMA) {
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+          f[(g + j) & 3] = __builtin_fmaf(f[(g + j) & 3], __builtin_bit_cast(float, xs), __builtin_bit_cast(float, w));
+          asm volatile("" : "+v"(f[(g + j) & 3]));
         }
       }
       if constexpr (MASK & P_LDS) {
@@ -110,6 +128,10 @@ extern "C" int msq_issue_probe(void* stream, int mask, int grid, int block, int 
     case P_VALU | P_LDS: launch_probe<P_VALU | P_LDS>(st, grid, block, s, iters); break;
     case P_VINT: launch_probe<P_VINT>(st, grid, block, s, iters); break;
     case P_VINT | P_MFMA16: launch_probe<P_VINT | P_MFMA16>(st, grid, block, s, iters); break;
+    case P_VPK: launch_probe<P_VPK>(st, grid, block, s, iters); break;
+    case P_VPK | P_MFMA16: launch_probe<P_VPK | P_MFMA16>(st, grid, block, s, iters); break;
+    case P_VFMA: launch_probe<P_VFMA>(st, grid, block, s, iters); break;
+    case P_VFMA | P_MFMA16: launch_probe<P_VFMA | P_MFMA16>(st, grid, block, s, iters); break;
     case P_VALU | P_LDS | P_MFMA4: launch_probe<P_VALU | P_LDS | P_MFMA4>(st, grid, block, s, iters); break;
     default: return fail(MSQ_ERR_ARGUMENT, "macseek quant: issue_probe: unknown instruction mix %d", mask);
   }
