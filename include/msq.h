@@ -271,7 +271,9 @@ int msq_router_topk(void* stream, const MsqBuffer* logits, const MsqBuffer* bias
  * logits = W[n_exp][dim] . x[dim] and the selection in one launch; W is F32 (the reference's ffn_gate_inp) or BF16.
  * scratch (>= msq_router_scratch_bytes(n_exp), the reference's Scratch::router_logits + counter) receives the logits in
  * its first n_exp floats; the caller zeroes it once before the first call and the call leaves its counter re-armed.
- * Calls sharing a scratch must not overlap. */
+ * A scratch belongs to one stream at a time: calls sharing it must not overlap. A launch that fails (MSQ_ERR_HIP) or is
+ * torn down part-way may leave the counter between zero and the workgroup count, after which calls would select
+ * nothing: zero the scratch again before it is reused. */
 size_t msq_router_scratch_bytes(int n_exp);
 int msq_router_fused(void* stream, int wtype, const MsqBuffer* x, const MsqBuffer* W, const MsqBuffer* bias,
                      const MsqBuffer* scratch, const MsqBuffer* ids, const MsqBuffer* w, int dim, int n_exp,
