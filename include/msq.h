@@ -44,7 +44,10 @@ typedef struct MsqBuffer { void* dev; size_t off; size_t size; } MsqBuffer;
 
 /* reference: ms::q::MvCfg (quant.hpp:12). Launch shape of the decode matvec, 0 = auto:
  * nr = rows one wave computes per tile, rsg = row-waves per workgroup, ks = waves splitting K inside a workgroup.
- * nr and rsg never change a row's summation order; ks does. */
+ * nr and rsg never change a row's summation order; ks does.
+ * The environment can impose the same three values on every call, on top of a passed shape (reference:
+ * MACSEEK_MV_NR / _RSG / _KS and MACSEEK_MVN_*, quant.mm:78-83,141): MSQ_MV_NR, MSQ_MV_RSG, MSQ_MV_KS for one token,
+ * MSQ_MVN_NR, MSQ_MVN_RSG, MSQ_MVN_KS for msq_matvec_n with several; read once per process. */
 typedef struct MsqMvCfg { int nr, rsg, ks; } MsqMvCfg;
 
 /* Library / device bring-up (no reference counterpart: Metal pipelines are created lazily by ms::Device). Optional:

@@ -256,6 +256,23 @@ bool mv_type_ok(int t) {
     default: return false;
   }
 }
+// Launch-shape overrides from the environment, on top of the caller's MsqMvCfg (reference: MACSEEK_MV_NR / _RSG / _KS,
+// quant.mm:78-83, and MACSEEK_MVN_NR / _SG for the small-N form, quant.mm:141): MSQ_MV_NR / MSQ_MV_RSG / MSQ_MV_KS for
+// one token, MSQ_MVN_NR / MSQ_MVN_RSG / MSQ_MVN_KS for several. Returns null when nothing is imposed.
+int env_knob(const char* name) {
+  const char* v = getenv(name);
+  return v && *v ? atoi(v) : 0;
+}
+const MsqMvCfg* effective_cfg(const MsqMvCfg* cfg, bool several, MsqMvCfg* store) {
+  static const int e1[3] = {env_knob("MSQ_MV_NR"), env_knob("MSQ_MV_RSG"), env_knob("MSQ_MV_KS")};
+  static const int en[3] = {env_knob("MSQ_MVN_NR"), env_knob("MSQ_MVN_RSG"), env_knob("MSQ_MVN_KS")};
+  const int* e = several ? en : e1;
+  *store = cfg ? *cfg : MsqMvCfg{0, 0, 0};
+  if (e[0] > 0) store->nr = e[0];
+  if (e[1] > 0) store->rsg = e[1];
+  if (e[2] > 0) store->ks = e[2];
+  return (store->nr > 0 || store->rsg > 0 || store->ks > 0) ? store : nullptr;
+}
 // column granularity the kernels need: dense types use a virtual 256 block like the reference (quant.mm:31-32)
 int mv_col_multiple(int t) { return msq_type_block_elems(t) == 1 ? 256 : msq_type_block_elems(t); }
 
@@ -268,6 +285,8 @@ namespace msq {
 // does not fit them (the caller then takes another path). Arguments are already validated.
 int matvec_tok(hipStream_t st, int t, const uint8_t* W, int rows, int cols, const float* X, float* Y, int n, int accumulate,
                int groups, const MsqMvCfg* cfg, const float* norm_w, float eps) {
+  MsqMvCfg several;
+  if (n > 1) cfg = effective_cfg(cfg, true, &several);
   // Q8_0 keeps fp32 activations (32 registers per token): four tokens per pass, the other formats eight
   const int T = n == 1 ? 1 : (t == MSQ_Q8_0 || n <= 4) ? 4 : 8;
   MvShape s;
@@ -311,8 +330,10 @@ int msq_matvec_cfg(int t, int rows, int cols, MsqMvCfg* out) {
   MvShape s;
   if (!out) return fail(MSQ_ERR_ARGUMENT, "macseek quant: matvec_cfg: null output");
   if (!mv_type_ok(t) || rows < 1 || cols < 1 || cols % mv_col_multiple(t)) return unsupported("matvec_cfg", t, rows, cols);
-  const bool tok = mv_tok_shape(t, rows, cols, 1, 1, nullptr, &s) && tok_serves_single(t, rows, cols, s, nullptr);  // as msq_matvec decides
-  if (!tok && !mv_shape(t, rows, cols, 1, nullptr, &s)) return unsupported("matvec_cfg", t, rows, cols);
+  MsqMvCfg env;
+  const MsqMvCfg* cfg = effective_cfg(nullptr, false, &env);
+  const bool tok = mv_tok_shape(t, rows, cols, 1, 1, cfg, &s) && tok_serves_single(t, rows, cols, s, cfg);  // as msq_matvec decides
+  if (!tok && !mv_shape(t, rows, cols, 1, cfg, &s)) return unsupported("matvec_cfg", t, rows, cols);
   out->nr = s.rpw; out->rsg = s.rw; out->ks = s.ks;
   return MSQ_OK;
 }
@@ -326,6 +347,8 @@ static int matvec_impl(void* stream, const char* what, int t, const MsqBuffer* W
     return fail(MSQ_ERR_ARGUMENT, "macseek quant: %s: buffer missing or too small (type %s rows %d cols %d)", what,
                 msq_type_name_of(t), rows, cols);
   hipStream_t st = (hipStream_t)stream;
+  MsqMvCfg imposed;
+  cfg = effective_cfg(cfg, false, &imposed);
   {  // shapes with several rows per wave (chosen for matrices of more than a row per wave and CU, or imposed by cfg) go
      // through the prefetching kernel; a shape names its kernel, so row chunks launched with the shape of the whole
      // matrix repeat its bits

@@ -157,6 +157,32 @@ def test_row_chunks_are_bit_identical(dev, t):
     assert torch.equal(full, parts) and torch.equal(full, other)
 
 
+def test_environment_imposes_the_launch_shape(dev, tmp_path):
+    # MSQ_MV_NR / _RSG / _KS (reference: MACSEEK_MV_*, quant.mm:78-83) are read once per process: a child process runs with
+    # them set; its matvec_cfg reports the imposed shape and its result has the bits of the same shape passed as MvCfg
+    import os, subprocess, sys
+    t, rows, cols = O.Q6_K, 1024, 2048
+    child = (
+        "import sys, numpy as np, torch\n"
+        "sys.path.insert(0, %r); sys.path.insert(0, %r)\n"
+        "import oracle as O\nfrom macseek_amd import quant as q\nfrom util import up\n"
+        "t, rows, cols = O.Q6_K, 1024, 2048\n"
+        "c = q.matvec_cfg(t, rows, cols)\nassert (c.nr, c.rsg, c.ks) == (3, 2, 1), (c.nr, c.rsg, c.ks)\n"
+        "Wd, xd = up(O.random_blocks(t, rows * cols, 5)), up(O.randn(cols, 6))\n"
+        "y = torch.empty(rows, dtype=torch.float32, device='cuda:0')\ne = q.Enc()\n"
+        "q.encode_matvec(e, t, q.Buffer.of(Wd), rows, cols, q.Buffer.of(xd), q.Buffer.of(y))\ne.wait()\n"
+        "np.save(%r, y.cpu().numpy())\n"
+    ) % (os.path.dirname(os.path.dirname(os.path.abspath(__file__))), os.path.dirname(os.path.abspath(__file__)), str(tmp_path / "y.npy"))
+    env = dict(os.environ, MSQ_MV_NR="3", MSQ_MV_RSG="2", MSQ_MV_KS="1")
+    subprocess.run([sys.executable, "-c", child], env=env, check=True, timeout=100)
+    Wd, xd = up(O.random_blocks(t, rows * cols, 5)), up(O.randn(cols, 6))
+    y = torch.empty(rows, dtype=torch.float32, device=dev)
+    e = q.Enc()
+    q.encode_matvec(e, t, q.Buffer.of(Wd), rows, cols, q.Buffer.of(xd), q.Buffer.of(y), False, 1, q.MvCfg(nr=3, rsg=2, ks=1))
+    e.wait()
+    assert np.array_equal(np.load(tmp_path / "y.npy").view(np.uint32), y.cpu().numpy().view(np.uint32))
+
+
 def test_repeat_is_bit_identical_and_unwritten_rows_untouched(dev):
     t, rows, cols = O.IQ2_XXS, 1000, 7168
     Wb = O.random_blocks(t, rows * cols, 1)
