@@ -205,7 +205,7 @@ constexpr int pf_blk_waves(int T) { return T > 3 ? 12 : 16; }
 // register count low enough for three or four waves per SIMD, which is what overlaps decode, matrix and LDS work
 constexpr int pf_blk_rt(bool gu, int) { return gu ? 1 : 2; }
 constexpr int pf_blk_rows(bool gu, int T) { return pf_blk_waves(T) * pf_blk_rt(gu, T) * 16; }  // weight rows per work item
-// activation staging: double-buffered for up to three token tiles, a single buffer (two barriers per block) for six
+// activation staging: double-buffered for up to three token tiles, a single buffer (two barriers per block) for seven
 template <class B>
 constexpr size_t pf_blk_lds(int T) { return (size_t)B::LDS_WORDS * 4 + (T > 3 ? 1 : 2) * (size_t)(T > 3 ? kPfBigTokens : kPfBlkTokens) * kPfBlkPitch; }
 
@@ -418,8 +418,8 @@ __device__ __forceinline__ void pf_block_body(const PfBlkArgs& a) {
 }
 
 // Kernel variants: T = 1 takes the items of one token tile; T = 3 those of two or three tiles, so that they share one
-// launch and its tail; T = 6 the blocks of 49 to 96 entries that the popular experts are cut into (their weights are
-// then decoded half as often; 12 waves, one activation buffer).
+// launch and its tail; T = 7 the blocks of 49 to 112 entries that the popular experts are cut into (their weights are
+// then decoded once per 112 entries; 12 waves, one activation buffer).
 template <class B, bool GU, int T>
 __global__ __launch_bounds__(64 * pf_blk_waves(T)) void moe_pf_block_kernel(const PfBlkArgs a) {
   if constexpr (T == 1 || T > 3) {
