@@ -52,38 +52,28 @@ def test_matvec_n_vs_oracle(dev, t, rows, cols, groups, n, acc):
     e.wait()
     got = Yd.cpu().numpy().astype(np.float64).reshape(n, rows)
     assert np.all(np.isfinite(got))
-    # the library's dispatch: rows of up to 16384 columns (dense types: 8192) go through the dot-product kernel, which
-    # stages activations like the decode matvec; the formats whose activation rows it stages in LDS also need room for
-    # the rows of a round there (160 KB less tables and partial sums: the latter are left out here). Wider rows go
-    # through the MFMA kernel, or as n decode matvecs when that is cheaper
-    dots = cols <= (8192 if t in (O.F32, O.F16, O.BF16) else 16384)
-    if t in (O.IQ1_S, O.IQ2_XXS, O.IQ4_NL, O.Q8_0):
-        T = 1 if n == 1 else 4 if (t == O.Q8_0 or n <= 4) else 8
-        G = min(T, 2 if t == O.IQ1_S else 4)
-        table = {O.IQ1_S: 32768, O.IQ2_XXS: 6144, O.IQ4_NL: 1024, O.Q8_0: 0}[t]
-        dots = dots and table + G * (cols + cols // 32 * 4) * 4 <= 160 * 1024
-    mb = q.row_bytes(q.QType(t), cols) * rows / 1e6
-    mfma_ok = n > 1 and t != O.F32 and not (groups > 1 and (rows // groups) % 16)
-    few = n * (3.0 + mb / 1.5) < 20.0 + mb
-    uses_mfma = mfma_ok and not dots and not few
-    Xh = half_round(X, t) if uses_mfma else X
-    if not uses_mfma and t not in (O.F32, O.F16, O.BF16, O.Q8_0):
-        Xh = X.astype(np.float16).astype(np.float32)  # the decode (n = 1) path stages fp16 pairs for the block formats
-    err_h = err_f = err_ns = 0.0
+    # Which kernel serves a shape is the library's business. Its kernels differ in how they stage activations: rounded
+    # to fp16 (block formats everywhere, every format in the MFMA kernel) or kept in fp32 (Q8_0 and dense types in the
+    # dot-product kernels). The result has to match the reference on ONE of these stagings to the tight bound, and the
+    # F32 reference to the loose one.
+    stagings = [X.astype(np.float16).astype(np.float32), X]
+    if t == O.BF16:
+        stagings.append(half_round(X, t))  # the MFMA kernel's two-term split for bf16 weights
+    err_f = err_ns = 0.0
+    err_hs = [0.0 for _ in stagings]
     for tok in range(n):
-        for hv, Xs in ((1, Xh), (0, X)):
+        y0 = Y0[tok * rows:(tok + 1) * rows].astype(np.float64)
+        for k, Xs in enumerate(stagings):
             ry, mag, wn2 = O.matvec(t, Wb, rows, cols, Xs[tok * xs:(tok + 1) * xs], groups)
-            y0 = Y0[tok * rows:(tok + 1) * rows].astype(np.float64)
             if acc:
                 ry, mag = ry + y0, mag + np.abs(y0)
             d = np.abs(got[tok] - ry)
-            ev = float(np.max(d / (mag + 1e-12)))
-            if hv:
-                err_h = max(err_h, ev)
-            else:
-                err_f = max(err_f, ev)
+            err_hs[k] = max(err_hs[k], float(np.max(d / (mag + 1e-12))))
+            if Xs is X:
+                err_f = max(err_f, float(np.max(d / (mag + 1e-12))))
                 xn = np.repeat(np.sqrt((Xs[tok * xs:(tok + 1) * xs].astype(np.float64) ** 2).reshape(groups, cols).sum(1)), rows // groups)
                 err_ns = max(err_ns, float(np.max(d / (np.sqrt(wn2 + (y0 ** 2 if acc else 0)) * xn + 1e-30))))
+    err_h = min(err_hs)
     print(f"  {O.TYPE_NAMES[t]:8s} [{cols:5d} -> {rows:5d}] g{groups} n={n:<2d} {'acc' if acc else '   '} "
           f"err(x staged) {err_h:.2e}  err(vs F32) {err_f:.2e}  north-star {err_ns:.2e}")
     # reference bounds: 2e-6 against the half-x reference for its F32-FMA kernel (n < 8), 1e-4 on its tile path,
