@@ -186,23 +186,83 @@ __global__ __launch_bounds__(256) void router_fused_kernel(const float* __restri
   __syncthreads();
   if (!last) return;
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
-  if (wave == 0) {
-    const uint32_t epl = n_exp >> 6;
-    float key[kMaxEpl];
-    double sc[kMaxEpl];
+  // Selection in two levels. Six rounds of "wave-wide best, then remove it" by one wave over all experts is a chain of
+  // twelve DPP reductions plus a six-way local maximum per round, run by a wave that has its SIMD to itself: 3 us.
+  // Here each of the four waves picks the six best of its quarter of the experts (two per lane at most: the local
+  // maximum is one comparison), leaves them in LDS, and wave 0 picks the six best of those 24 (one per lane). The six
+  // best overall are among the six best of their quarters, and "greater key, then lower expert id" is a total order, so
+  // the result is the one-level selection's.
+  __shared__ float c_key[4 * kTopK];
+  __shared__ int c_id[4 * kTopK];
+  __shared__ double c_sc[4 * kTopK];
+  const uint32_t quarter = n_exp >> 2;  // experts of this wave: quarter * wave + {lane, lane + 64}
+  {
+    float key[2];
+    double sc[2];
 #pragma unroll
-    for (uint32_t i = 0; i < kMaxEpl; i++) {
+    for (uint32_t i = 0; i < 2; i++) {
       key[i] = -INFINITY;
       sc[i] = 0.0;
-      if (i < epl) {  // device-scope loads: the records were written by other CUs during this launch
-        const uint64_t* r = (const uint64_t*)(recs + lane + 64u * i);
+      if (lane + 64u * i < quarter) {  // device-scope loads: the records were written by other CUs during this launch
+        const uint64_t* r = (const uint64_t*)(recs + quarter * wave + lane + 64u * i);
         const uint64_t s64 = __hip_atomic_load(r, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         const uint64_t k64 = __hip_atomic_load(r + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         sc[i] = __builtin_bit_cast(double, s64);
         key[i] = __builtin_bit_cast(float, (uint32_t)k64);
       }
     }
-    select6(key, sc, epl, route_scale, lane, ids, wts);
+#pragma unroll
+    for (int k = 0; k < kTopK; k++) {
+      // the lane's best: strict comparisons from -inf up, so NaN and -inf keys are never candidates and the lower id
+      // wins among equals
+      float bk = -INFINITY;
+      bool second = false, any = false;
+      if (key[0] > bk) { bk = key[0]; any = true; }
+      if (key[1] > bk) { bk = key[1]; second = true; any = true; }
+      const int be = any ? (int)(quarter * wave + lane + (second ? 64u : 0u)) : 0x7fffffff;
+      const float m = wave_max_f(bk);
+      const int win = wave_min_i(bk == m ? be : 0x7fffffff);
+      if (win != 0x7fffffff && be == win) {  // one lane
+        c_key[wave * kTopK + k] = bk;
+        c_id[wave * kTopK + k] = win;
+        c_sc[wave * kTopK + k] = second ? sc[1] : sc[0];
+        if (second) key[1] = -INFINITY; else key[0] = -INFINITY;
+      }
+      if (win == 0x7fffffff && lane == 0) { c_key[wave * kTopK + k] = -INFINITY; c_id[wave * kTopK + k] = 0x7fffffff; c_sc[wave * kTopK + k] = 0.0; }
+    }
+  }
+  __syncthreads();
+  if (wave == 0) {
+    float ck = lane < 4u * kTopK ? c_key[lane] : -INFINITY;
+    const int ce = lane < 4u * kTopK ? c_id[lane] : 0x7fffffff;
+    const double cs = lane < 4u * kTopK ? c_sc[lane] : 0.0;
+    int sel_e[kTopK];
+    double sel_s[kTopK];
+    double sum = 0.0;  // the six scores are added in selection order, as the reference adds them
+#pragma unroll
+    for (int k = 0; k < kTopK; k++) {
+      const float m = wave_max_f(ck);
+      const int win = wave_min_i((ck == m && ce != 0x7fffffff) ? ce : 0x7fffffff);
+      if (win == 0x7fffffff) {  // fewer than six comparable keys (NaN logits): expert 0 with weight 0
+        sel_e[k] = 0;
+        sel_s[k] = 0.0;
+        continue;
+      }
+      const uint64_t holder = __builtin_amdgcn_ballot_w64(ce == win);
+      const int src = (int)__builtin_ctzll(holder);
+      if (ce == win) ck = -INFINITY;
+      const uint64_t bits = __builtin_bit_cast(uint64_t, cs);
+      const uint32_t lo = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)bits, src);
+      const uint32_t hi = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)(bits >> 32), src);
+      sel_e[k] = win;
+      sel_s[k] = __builtin_bit_cast(double, ((uint64_t)hi << 32) | lo);
+      sum += sel_s[k];
+    }
+    if (lane < (uint32_t)kTopK) {
+#pragma unroll
+      for (int k = 0; k < kTopK; k++)
+        if (lane == (uint32_t)k) { ids[k] = sel_e[k]; wts[k] = (float)(sel_s[k] / (sum + 1e-20) * (double)route_scale); }
+    }
     if (lane == 0) __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
 }

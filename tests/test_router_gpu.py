@@ -147,6 +147,56 @@ def test_router_fused_vs_oracle(dev, wtype, dim):
     print(f"  router_fused {wtype.name} dim={dim}: near-ties against fp64 logits {ties}")
 
 
+@pytest.mark.parametrize("n_exp", [64, 128, 384, 512])
+def test_router_fused_ties_expert_counts_and_nan(dev, n_exp):
+    """The fused router selects in two levels (each wave of the last workgroup from its quarter of the experts, then one
+    wave from the 24 survivors): exact ties inside a lane's pair of experts, across lanes and across quarters must go to
+    the lower expert id, fewer than six comparable keys give expert 0 with weight 0, for every supported expert count."""
+    dim = 256
+    rng = np.random.default_rng(n_exp)
+    W = (rng.standard_normal((n_exp, dim)) * 0.05).astype(np.float32)
+    q4 = n_exp // 4
+    # identical rows: same logit, same bias -> same key. Pairs (e, e + 64) share a lane when the quarter has 128
+    # experts; (e, e + q4) sit in different quarters; runs of equal rows sit in neighbouring lanes
+    W[3 + q4] = W[3]
+    W[7 + 2 * q4] = W[7]
+    W[10:14] = W[10]
+    if q4 > 64:
+        W[5 + 64] = W[5]
+    big = np.array([3, 7, 10, 5], dtype=np.int64)
+    W[big] *= 6.0  # make the tied rows the likely winners
+    W[3 + q4], W[7 + 2 * q4], W[10:14] = W[3], W[7], W[10]
+    if q4 > 64:
+        W[5 + 64] = W[5]
+    bias = np.zeros(n_exp, dtype=np.float32)
+    Wd, bd = up(W.reshape(-1)), up(bias)
+    s = arch.Scratch.create(n_exp)
+    ids = torch.zeros(6, dtype=torch.int32, device=dev)
+    w = torch.zeros(6, dtype=torch.float32, device=dev)
+    e = q.Enc()
+    for it in range(6):
+        x = O.randn(dim, 300 + it)
+        x = np.abs(x) * np.sign(W[10] + 1e-9) if it % 2 else x  # odd rounds: row 10 (and its copies) gets a large logit
+        arch.encode_router_fused(e, q.Buffer.of(up(x.astype(np.float32))), q.Buffer.of(Wd), q.Buffer.of(bd), q.Buffer.of(ids), q.Buffer.of(w), s, dim)
+        e.wait()
+        got_logits = s.mem[: n_exp * 4].view(torch.float32).cpu().numpy()
+        assert np.array_equal(got_logits[3], got_logits[3 + q4]) and np.array_equal(got_logits[10], got_logits[13])
+        rid, rw = O.router(got_logits[None], bias)
+        assert np.array_equal(ids.cpu().numpy()[None], rid), (it, ids.cpu().numpy(), rid)
+        assert np.array_equal(w.cpu().numpy()[None].view(np.uint32), rw.view(np.uint32))
+    # NaN activations: every logit is NaN, nothing is comparable
+    x = np.full(dim, np.nan, dtype=np.float32)
+    arch.encode_router_fused(e, q.Buffer.of(up(x)), q.Buffer.of(Wd), q.Buffer.of(bd), q.Buffer.of(ids), q.Buffer.of(w), s, dim)
+    e.wait()
+    assert not ids.any() and not w.any()
+    # and the scratch is left re-armed: the next call works
+    x = O.randn(dim, 999)
+    arch.encode_router_fused(e, q.Buffer.of(up(x)), q.Buffer.of(Wd), q.Buffer.of(bd), q.Buffer.of(ids), q.Buffer.of(w), s, dim)
+    e.wait()
+    rid, rw = O.router(s.mem[: n_exp * 4].view(torch.float32).cpu().numpy()[None], bias)
+    assert np.array_equal(ids.cpu().numpy()[None], rid)
+
+
 def test_router_fused_repeats_bit_identically_and_checks_arguments(dev):
     n_exp, dim, R = 384, 7168, 300
     Wd, bd, xd = up(O.randn(n_exp * dim, 1, 0.02)), up(O.randn(n_exp, 2, 0.1)), up(O.randn(dim, 3))
