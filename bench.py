@@ -32,7 +32,7 @@ HBM_PEAK_GBPS = 8000.0
 # HBM bytes per launch of the decode gate/up kernel, from the FETCH_SIZE / WRITE_SIZE counter runs of this workload
 # (KiB per dispatch, scaled by what the same counters read for a 1 GiB copy: x2.000 and x1.000): 42.92 MB + 0.06 MB
 GU_TRAFFIC_BYTES = 42983346
-# HBM bytes of the three launches of the prefill gate/up GEMM together (same counters, same scaling), configs[3]
+# HBM bytes of the launches of the prefill gate/up GEMM together (same counters, same scaling), configs[3]
 PF_GU_TRAFFIC_BYTES = 4288940933
 
 
@@ -389,7 +389,8 @@ def bench_moe_prefill(torch, steps, warmup, with_cpu=True):
     gu_mean, gu_med, gu_min = event_ms_per_launch(torch, lambda i: call(), max(3, min(steps, 10)))
     os.environ["MSQ_MOEP_SKIP"] = str(1 | 2 | 4 | 16 | 32)
     dn_mean, _, _ = event_ms_per_launch(torch, lambda i: call(), max(3, min(steps, 10)))
-    # the three launches of the gate/up GEMM on their own: one-tile items, two- and three-tile items, popular experts' blocks
+    # the item classes of the gate/up GEMM on their own: one-tile items, two- and three-tile items (one launch together
+    # otherwise), popular experts' blocks
     split = {}
     for name, keep in (("one_tile_items", 64), ("two_three_tile_items", 128), ("blocks_of_popular_experts", 256)):
         os.environ["MSQ_MOEP_SKIP"] = str((1 | 4 | 8 | 16 | 32) | ((64 | 128 | 256) & ~keep))
@@ -412,12 +413,12 @@ def bench_moe_prefill(torch, steps, warmup, with_cpu=True):
                    "weight_bytes_touched": int(len(used)) * per_exp},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": achieved / MFMA_PEAK_TFLOPS,
                      "traffic": PF_GU_TRAFFIC_BYTES, "traffic_source": "profiles/moe_prefill_hbm_traffic_fetch_write.txt",
-                     "kernel": "moe_pf_block_kernel<BlkIQ2XXS, gate/up> (three launches: blocks of 49..112 entries of the popular experts, two- and three-tile items, one-tile items)",
+                     "kernel": "moe_pf_block_kernel<BlkIQ2XXS, gate/up> (two launches: blocks of 49..112 entries of the popular experts; items of one to three token tiles)",
                      "gate_up_time_split": split,
                      "flops_per_launch": gu_flops,
                      "avg_launch_us": gu_mean * 1e3, "min_launch_us": gu_min * 1e3,
                      "weight_GBps": int(len(used)) * 2 * gu_b / (gu_mean * 1e-3) / 1e9,
-                     "second_kernel": {"kernel": "moe_pf_block_kernel<BlkIQ2XXS, down> (three launches)", "avg_launch_us": dn_mean * 1e3,
+                     "second_kernel": {"kernel": "moe_pf_block_kernel<BlkIQ2XXS, down> (two launches)", "avg_launch_us": dn_mean * 1e3,
                                        "achieved": 2.0 * DIM * INTER * total / (dn_mean * 1e-3) / 1e12}},
         "pct_of_mfma_peak": 100 * value / MFMA_PEAK_TFLOPS,
     }

@@ -417,18 +417,20 @@ __device__ __forceinline__ void pf_block_body(const PfBlkArgs& a) {
   }
 }
 
-// Kernel variants: T = 1 takes the items of one token tile; T = 3 those of two or three tiles, so that they share one
-// launch and its tail; T = 7 the blocks of 49 to 112 entries that the popular experts are cut into (their weights are
-// then decoded once per 112 entries; 12 waves, one activation buffer).
+// Kernel variants: T = 3 takes the items of up to three token tiles in one launch, largest first (each runs the body
+// built for its tile count; one launch has one tail of half-idle CUs); T = 7 the blocks of 49 to 112 entries that the
+// popular experts are cut into (their weights are then decoded once per 112 entries; 12 waves, one activation buffer).
 template <class B, bool GU, int T>
 __global__ __launch_bounds__(64 * pf_blk_waves(T)) void moe_pf_block_kernel(const PfBlkArgs a) {
-  if constexpr (T == 1 || T > 3) {
+  if constexpr (T > 3) {
     pf_block_body<B, GU, T>(a);
   } else {
     const uint32_t item = ((blockIdx.x >> 3) / a.row_chunks) * 8u + (blockIdx.x & 7u);
     if (item >= a.nitems) return;
-    if (a.items[3 * item + 2] > 32) pf_block_body<B, GU, 3>(a);
-    else pf_block_body<B, GU, 2>(a);
+    const uint32_t cnt = a.items[3 * item + 2];
+    if (cnt > 32) pf_block_body<B, GU, 3>(a);
+    else if (cnt > 16) pf_block_body<B, GU, 2>(a);
+    else pf_block_body<B, GU, 1>(a);
   }
 }
 

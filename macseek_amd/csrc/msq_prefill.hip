@@ -69,11 +69,11 @@ int launch_block_t(hipStream_t st, PfBlkArgs a, uint32_t n6, uint32_t n3, uint32
   int rc;
   a.items = items; a.nitems = n6;
   if (!(skip & 256) && (rc = launch_block_tt<B, GU, kPfBigTiles>(st, a))) return rc;
-  a.items = items + 3 * (size_t)n6; a.nitems = n3 + n2;
-  if (!(skip & 128) && (rc = launch_block_tt<B, GU, 3>(st, a))) return rc;
-  a.items = items + 3 * (size_t)(n6 + n3 + n2); a.nitems = n - n6 - n3 - n2;
-  if (skip & 64) return MSQ_OK;
-  return launch_block_tt<B, GU, 1>(st, a);
+  // one launch for everything up to three tiles, largest first: one tail of half-idle CUs instead of two (the profiling
+  // mask can leave either part out)
+  const uint32_t lo = (skip & 128) ? n6 + n3 + n2 : n6, hi = (skip & 64) ? n6 + n3 + n2 : n;
+  a.items = items + 3 * (size_t)lo; a.nitems = hi > lo ? hi - lo : 0u;
+  return launch_block_tt<B, GU, 3>(st, a);
 }
 bool block_path(int t) { return t == MSQ_IQ1_S || t == MSQ_IQ2_XXS; }
 template <bool GU>
@@ -143,7 +143,7 @@ int msq_moe_prefill(void* stream, const MsqMoePrefillArgs* p) {
   hipStream_t st = (hipStream_t)stream;
   const int cus = device_info().cus;
   // PROFILING ONLY (wrong output): MSQ_MOEP_SKIP bit mask 1 gather, 2 routed gate/up, 4 shared gate/up, 8 routed down,
-  // 16 shared down, 32 reduce; of the block GEMMs' three launches 64 the one-tile items, 128 the two- and three-tile
+  // 16 shared down, 32 reduce; of the block GEMMs' work 64 the one-tile items, 128 the two- and three-tile
   // items, 256 the blocks of the popular experts -- read on every call (reference: MACSEEK_MOEP_SKIP,
   // src/kernels/quant.mm:520-522)
   const char* skip_env = getenv("MSQ_MOEP_SKIP");
