@@ -254,7 +254,10 @@ size_t msq_moe_prefill_scratch_bytes(int total_entries, int n_tokens, int n_exp,
 /* reference: ms::q::encode_moe_prefill (quant.hpp:118, quant.mm:433-612). Enqueues gather, grouped gate/up GEMM +
  * SwiGLU, grouped down GEMM and the ordered reduction into Y. Activations and H are staged as fp16 and weights enter
  * the matrix instructions as fp16 (the whole weight rounded once), as in the reference's tiles. The call only enqueues
- * (no host copy, no wait, no allocation) and can be captured in a HIP graph; `offs` (host memory) is read at call time and
+ * (no host copy, no wait, no allocation) and can be captured in a HIP graph. Two of its launches are independent and
+ * run side by side: one is forked onto a stream that the library owns (one per device, created by msq_init() or by the
+ * first call outside a capture) and joined back before the call's later launches, all through events, so the caller
+ * sees the ordering of a single stream (MSQ_MOEP_ONE_STREAM=1 in the environment turns the fork off); `offs` (host memory) is read at call time and
  * travels to the device inside kernel arguments. The result is bit-identical from run to run. n_tokens <= 0 returns MSQ_OK and
  * does nothing (quant.mm:435). */
 int msq_moe_prefill(void* stream, const MsqMoePrefillArgs* a);

@@ -5,6 +5,8 @@
 #include <cstring>
 #include <vector>
 
+#include <mutex>
+
 #include "msq_host.h"
 #include "msq_prefill.cuh"
 
@@ -60,6 +62,33 @@ int launch_block_tt(hipStream_t st, PfBlkArgs a) {
   MSQ_HIP(hipGetLastError());
   return MSQ_OK;
 }
+// A second stream of the library's own, per device, and the two events that fork work onto it and join it back: the
+// popular experts' blocks and the small items are independent launches of one workgroup per CU each, and the first
+// ends in a round that fills less than half of the CUs. Forked, the small items start on the CUs that round leaves
+// idle. Fork and join are event dependencies, so a stream capture records them like any other (the objects are created
+// outside of captures: by msq_init() or by the first call that is not being captured; until then calls stay on one stream).
+struct SideStream { hipStream_t stream = nullptr; hipEvent_t fork = nullptr, join = nullptr; bool ok = false; };
+std::mutex g_side_mu;
+SideStream g_side[16];
+SideStream* side_stream(hipStream_t st) {
+  static const bool off = [] { const char* e = getenv("MSQ_MOEP_ONE_STREAM"); return e && *e && atoi(e) != 0; }();
+  int dev = 0;
+  if (off || hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 16) return nullptr;
+  SideStream& s = g_side[dev];
+  if (!s.ok) {
+    hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(st, &cs) != hipSuccess || cs != hipStreamCaptureStatusNone) return nullptr;
+    if (hipStreamCreateWithFlags(&s.stream, hipStreamNonBlocking) != hipSuccess ||
+        hipEventCreateWithFlags(&s.fork, hipEventDisableTiming) != hipSuccess ||
+        hipEventCreateWithFlags(&s.join, hipEventDisableTiming) != hipSuccess) {
+      (void)hipGetLastError();
+      return nullptr;
+    }
+    s.ok = true;
+  }
+  return &s;
+}
+
 // items are sorted by size, largest first: n6 blocks of more than 48 entries, n3 items of three token tiles, n2 of two,
 // then the one-tile items; skip: profiling mask (see msq_moe_prefill)
 template <class B, bool GU>
@@ -68,6 +97,21 @@ int launch_block_t(hipStream_t st, PfBlkArgs a, uint32_t n6, uint32_t n3, uint32
   const uint32_t n = a.nitems;
   int rc;
   a.items = items; a.nitems = n6;
+  const bool small_items = n > n6 && (skip & (64 | 128)) != (64 | 128);
+  if (n6 && !(skip & 256) && small_items) {
+    std::lock_guard<std::mutex> lock(g_side_mu);
+    if (SideStream* s = side_stream(st)) {
+      MSQ_HIP(hipEventRecord(s->fork, st));
+      MSQ_HIP(hipStreamWaitEvent(s->stream, s->fork, 0));
+      if ((rc = launch_block_tt<B, GU, kPfBigTiles>(s->stream, a))) return rc;
+      MSQ_HIP(hipEventRecord(s->join, s->stream));
+      const uint32_t lo = (skip & 128) ? n6 + n3 + n2 : n6, hi = (skip & 64) ? n6 + n3 + n2 : n;
+      a.items = items + 3 * (size_t)lo; a.nitems = hi > lo ? hi - lo : 0u;
+      rc = launch_block_tt<B, GU, 3>(st, a);
+      MSQ_HIP(hipStreamWaitEvent(st, s->join, 0));
+      return rc;
+    }
+  }
   if (!(skip & 256) && (rc = launch_block_tt<B, GU, kPfBigTiles>(st, a))) return rc;
   // one launch for everything up to three tiles, largest first: one tail of half-idle CUs instead of two (the profiling
   // mask can leave either part out)
@@ -91,6 +135,12 @@ int launch_gemm(int t, hipStream_t st, const PfArgs& a, int cus) {
 }
 
 }  // namespace
+
+void prefill_side_stream_setup() {
+  std::lock_guard<std::mutex> lock(g_side_mu);
+  (void)side_stream(nullptr);
+}
+
 }  // namespace msq
 
 using namespace msq;
