@@ -62,10 +62,12 @@ int launch_block_tt(hipStream_t st, PfBlkArgs a) {
   MSQ_HIP(hipGetLastError());
   return MSQ_OK;
 }
-// A second stream of the library's own, per device, and the two events that fork work onto it and join it back: the
-// popular experts' blocks and the small items are independent launches of one workgroup per CU each, and the first
-// ends in a round that fills less than half of the CUs. Forked, the small items start on the CUs that round leaves
-// idle. Fork and join are event dependencies, so a stream capture records them like any other (the objects are created
+// A second stream of the library's own, per device, and the two events that fork work onto it and join it back. The
+// routed experts' work falls into two classes that never meet before the final reduction: the popular experts' blocks
+// (gate/up, then down of the same entries) and the small items (likewise). Each launch has one workgroup per CU and
+// ends in a round that leaves CUs idle (the blocks' last round fills less than half of them); as two pipelines on two
+// streams, each class starts on the CUs the other leaves idle, and no class waits for the other's gate/up before its
+// own down. Fork and join are event dependencies, so a stream capture records them like any other (the objects are created
 // outside of captures: by msq_init() or by the first call that is not being captured; until then calls stay on one stream).
 struct SideStream { hipStream_t stream = nullptr; hipEvent_t fork = nullptr, join = nullptr; bool ok = false; };
 std::mutex g_side_mu;
@@ -90,39 +92,26 @@ SideStream* side_stream(hipStream_t st) {
 }
 
 // items are sorted by size, largest first: n6 blocks of more than 48 entries, n3 items of three token tiles, n2 of two,
-// then the one-tile items; skip: profiling mask (see msq_moe_prefill)
+// then the one-tile items; which: kBig (the blocks), kSmall (everything up to three tiles, one launch: one tail of
+// half-idle CUs instead of two) or both; skip: profiling mask (see msq_moe_prefill)
+enum { kBig = 1, kSmall = 2 };
 template <class B, bool GU>
-int launch_block_t(hipStream_t st, PfBlkArgs a, uint32_t n6, uint32_t n3, uint32_t n2, int skip) {
+int launch_block_t(hipStream_t st, PfBlkArgs a, uint32_t n6, uint32_t n3, uint32_t n2, int skip, int which) {
   const uint32_t* items = a.items;
   const uint32_t n = a.nitems;
   int rc;
   a.items = items; a.nitems = n6;
-  const bool small_items = n > n6 && (skip & (64 | 128)) != (64 | 128);
-  if (n6 && !(skip & 256) && small_items) {
-    std::lock_guard<std::mutex> lock(g_side_mu);
-    if (SideStream* s = side_stream(st)) {
-      MSQ_HIP(hipEventRecord(s->fork, st));
-      MSQ_HIP(hipStreamWaitEvent(s->stream, s->fork, 0));
-      if ((rc = launch_block_tt<B, GU, kPfBigTiles>(s->stream, a))) return rc;
-      MSQ_HIP(hipEventRecord(s->join, s->stream));
-      const uint32_t lo = (skip & 128) ? n6 + n3 + n2 : n6, hi = (skip & 64) ? n6 + n3 + n2 : n;
-      a.items = items + 3 * (size_t)lo; a.nitems = hi > lo ? hi - lo : 0u;
-      rc = launch_block_tt<B, GU, 3>(st, a);
-      MSQ_HIP(hipStreamWaitEvent(st, s->join, 0));
-      return rc;
-    }
-  }
-  if (!(skip & 256) && (rc = launch_block_tt<B, GU, kPfBigTiles>(st, a))) return rc;
-  // one launch for everything up to three tiles, largest first: one tail of half-idle CUs instead of two (the profiling
-  // mask can leave either part out)
+  if ((which & kBig) && !(skip & 256) && (rc = launch_block_tt<B, GU, kPfBigTiles>(st, a))) return rc;
+  if (!(which & kSmall)) return MSQ_OK;
   const uint32_t lo = (skip & 128) ? n6 + n3 + n2 : n6, hi = (skip & 64) ? n6 + n3 + n2 : n;
   a.items = items + 3 * (size_t)lo; a.nitems = hi > lo ? hi - lo : 0u;
   return launch_block_tt<B, GU, 3>(st, a);
 }
 bool block_path(int t) { return t == MSQ_IQ1_S || t == MSQ_IQ2_XXS; }
 template <bool GU>
-int launch_block(int t, hipStream_t st, const PfBlkArgs& a, uint32_t n6, uint32_t n3, uint32_t n2, int skip) {
-  return t == MSQ_IQ1_S ? launch_block_t<BlkIQ1S, GU>(st, a, n6, n3, n2, skip) : launch_block_t<BlkIQ2XXS, GU>(st, a, n6, n3, n2, skip);
+int launch_block(int t, hipStream_t st, const PfBlkArgs& a, uint32_t n6, uint32_t n3, uint32_t n2, int skip, int which) {
+  return t == MSQ_IQ1_S ? launch_block_t<BlkIQ1S, GU>(st, a, n6, n3, n2, skip, which)
+                        : launch_block_t<BlkIQ2XXS, GU>(st, a, n6, n3, n2, skip, which);
 }
 
 template <bool GU>
@@ -252,8 +241,10 @@ int msq_moe_prefill(void* stream, const MsqMoePrefillArgs* p) {
   }
   uint8_t* sc = bptr_mut(&p->scratch);
   // The header travels in kernel arguments, a few KB per launch: nothing is read from host memory after this call
-  // returns, the call never waits for the stream, and a stream capture records the values themselves.
-  {
+  // returns, the call never waits for the stream, and a stream capture records the values themselves. The gather does
+  // not read the header: the header's launches (a dozen, each a few microseconds of launch latency) go to the side
+  // stream when there is one and are joined behind the gather.
+  auto write_header = [&](hipStream_t hs) {
     const size_t used = 24 * (size_t)(ne + 1) + 4 * (size_t)(ne + 2) + 8 * (size_t)(nt_routed + nt_shared) +
                         12 * (size_t)(ni_routed + ni_shared);
     const size_t words = (used + 3) / 4;
@@ -261,10 +252,9 @@ int msq_moe_prefill(void* stream, const MsqMoePrefillArgs* p) {
       HdrChunk c;
       const uint32_t n = (uint32_t)std::min<size_t>(kHdrChunkWords, words - w0);
       memcpy(c.w, hdr.data() + 4 * w0, 4 * (size_t)n);  // hdr is padded to a multiple of 256 bytes
-      hipLaunchKernelGGL(moe_pf_header_kernel, dim3(1), dim3(256), 0, st, (uint32_t*)sc + w0, c, n);
+      hipLaunchKernelGGL(moe_pf_header_kernel, dim3(1), dim3(256), 0, hs, (uint32_t*)sc + w0, c, n);
     }
-    MSQ_HIP(hipGetLastError());
-  }
+  };
   const size_t rows = (size_t)total + n;
   uint16_t* Xg = (uint16_t*)(sc + hbytes);
   uint16_t* H = (uint16_t*)((uint8_t*)Xg + align256(rows * dim * 2));
@@ -276,11 +266,28 @@ int msq_moe_prefill(void* stream, const MsqMoePrefillArgs* p) {
 
   // 1) gather + convert
   const uint32_t grows = (uint32_t)(total + (p->has_shared ? n : 0));
-  if (grows > 0 && !(skip & 1)) {
-    const dim3 grid((dim / 4 + 255) / 256, grows), block(256);
-    const int* tok = total > 0 ? (const int*)bptr(&p->tok) : nullptr;
-    if (p->x_is_bf16) hipLaunchKernelGGL((moe_pf_gather_kernel<true>), grid, block, 0, st, (const void*)bptr(&p->X), Xg, tok, (uint32_t)total, grows, (uint32_t)dim);
-    else hipLaunchKernelGGL((moe_pf_gather_kernel<false>), grid, block, 0, st, (const void*)bptr(&p->X), Xg, tok, (uint32_t)total, grows, (uint32_t)dim);
+  auto gather = [&]() {
+    if (grows > 0 && !(skip & 1)) {
+      const dim3 grid((dim / 4 + 255) / 256, grows), block(256);
+      const int* tok = total > 0 ? (const int*)bptr(&p->tok) : nullptr;
+      if (p->x_is_bf16) hipLaunchKernelGGL((moe_pf_gather_kernel<true>), grid, block, 0, st, (const void*)bptr(&p->X), Xg, tok, (uint32_t)total, grows, (uint32_t)dim);
+      else hipLaunchKernelGGL((moe_pf_gather_kernel<false>), grid, block, 0, st, (const void*)bptr(&p->X), Xg, tok, (uint32_t)total, grows, (uint32_t)dim);
+    }
+  };
+  {
+    std::lock_guard<std::mutex> lock(g_side_mu);
+    SideStream* s = (grows > 0 && !(skip & 1)) ? side_stream(st) : nullptr;
+    if (s) {
+      MSQ_HIP(hipEventRecord(s->fork, st));
+      MSQ_HIP(hipStreamWaitEvent(s->stream, s->fork, 0));
+      write_header(s->stream);
+      MSQ_HIP(hipEventRecord(s->join, s->stream));
+      gather();
+      MSQ_HIP(hipStreamWaitEvent(st, s->join, 0));
+    } else {
+      write_header(st);
+      gather();
+    }
     MSQ_HIP(hipGetLastError());
   }
   PfArgs a{};
@@ -295,25 +302,50 @@ int msq_moe_prefill(void* stream, const MsqMoePrefillArgs* p) {
   b.H = H; b.Z = Z; b.wt = a.wt; b.ptrs = d_ptrs; b.offs = d_offs; b.total = (uint32_t)total;
   // one GEMM over the routed experts or over the shared expert: block kernel for the codebook formats, else the
   // token-tile kernel
-  auto gemm = [&](auto gu_tag, int type, bool shared, const uint16_t* A, uint32_t K, uint32_t N, size_t row_bytes) -> int {
+  auto gemm = [&](auto gu_tag, int type, bool shared, const uint16_t* A, uint32_t K, uint32_t N, size_t row_bytes,
+                  hipStream_t gs, int which) -> int {
     constexpr bool GU = decltype(gu_tag)::value;
     if (block_path(type)) {
       b.A = A; b.K = K; b.N = N; b.nblocks = K / 256; b.row_bytes = (uint32_t)row_bytes;
       b.items = d_items + (shared ? 3 * (size_t)ni_routed : 0); b.nitems = shared ? ni_shared : ni_routed;
       const uint32_t* nc = shared ? nc_shared : nc_routed;
-      return launch_block<GU>(type, st, b, nc[0], nc[1], nc[2], skip);
+      return launch_block<GU>(type, gs, b, nc[0], nc[1], nc[2], skip, which);
     }
     a.A = A; a.N = N; steps(K); a.row_bytes = (uint32_t)row_bytes;
     a.tiles = d_tiles + (shared ? 2 * (size_t)nt_routed : 0); a.ntiles = shared ? nt_shared : nt_routed;
-    return launch_gemm<GU>(type, st, a, cus);
+    return launch_gemm<GU>(type, gs, a, cus);
   };
   int rc;
-  // 2) gate + up + SwiGLU -> H
-  if (nt_routed && !(skip & 2) && (rc = gemm(std::true_type{}, p->t_gate_up, false, Xg, (uint32_t)dim, (uint32_t)inter, rb_gu))) return rc;
-  if (nt_shared && !(skip & 4) && (rc = gemm(std::true_type{}, p->t_shared, true, Xg, (uint32_t)dim, (uint32_t)inter, rb_sgu))) return rc;
-  // 3) down -> Z
-  if (nt_routed && !(skip & 8) && (rc = gemm(std::false_type{}, p->t_down, false, H, (uint32_t)inter, (uint32_t)dim, rb_d))) return rc;
-  if (nt_shared && !(skip & 16) && (rc = gemm(std::false_type{}, p->t_shared, true, H, (uint32_t)inter, (uint32_t)dim, rb_sd))) return rc;
+  const bool routed_gu = nt_routed && !(skip & 2), routed_dn = nt_routed && !(skip & 8);
+  const int both = kBig | kSmall;
+  // The routed experts' two item classes as two pipelines (see SideStream) when both exist and a side stream does
+  bool forked = false;
+  if ((routed_gu || routed_dn) && block_path(p->t_gate_up) && block_path(p->t_down) && nc_routed[0] > 0 &&
+      ni_routed > nc_routed[0] && !(skip & 256) && (skip & (64 | 128)) != (64 | 128)) {
+    std::lock_guard<std::mutex> lock(g_side_mu);
+    if (SideStream* s = side_stream(st)) {
+      forked = true;
+      MSQ_HIP(hipEventRecord(s->fork, st));
+      MSQ_HIP(hipStreamWaitEvent(s->stream, s->fork, 0));
+      rc = routed_gu ? gemm(std::true_type{}, p->t_gate_up, false, Xg, (uint32_t)dim, (uint32_t)inter, rb_gu, s->stream, kBig) : MSQ_OK;
+      if (rc == MSQ_OK && routed_dn) rc = gemm(std::false_type{}, p->t_down, false, H, (uint32_t)inter, (uint32_t)dim, rb_d, s->stream, kBig);
+      MSQ_HIP(hipEventRecord(s->join, s->stream));
+      if (rc == MSQ_OK && routed_gu) rc = gemm(std::true_type{}, p->t_gate_up, false, Xg, (uint32_t)dim, (uint32_t)inter, rb_gu, st, kSmall);
+      if (rc == MSQ_OK && nt_shared && !(skip & 4)) rc = gemm(std::true_type{}, p->t_shared, true, Xg, (uint32_t)dim, (uint32_t)inter, rb_sgu, st, both);
+      if (rc == MSQ_OK && routed_dn) rc = gemm(std::false_type{}, p->t_down, false, H, (uint32_t)inter, (uint32_t)dim, rb_d, st, kSmall);
+      if (rc == MSQ_OK && nt_shared && !(skip & 16)) rc = gemm(std::false_type{}, p->t_shared, true, H, (uint32_t)inter, (uint32_t)dim, rb_sd, st, both);
+      MSQ_HIP(hipStreamWaitEvent(st, s->join, 0));  // the side stream is joined whatever happened above
+      if (rc != MSQ_OK) return rc;
+    }
+  }
+  if (!forked) {
+    // 2) gate + up + SwiGLU -> H
+    if (routed_gu && (rc = gemm(std::true_type{}, p->t_gate_up, false, Xg, (uint32_t)dim, (uint32_t)inter, rb_gu, st, both))) return rc;
+    if (nt_shared && !(skip & 4) && (rc = gemm(std::true_type{}, p->t_shared, true, Xg, (uint32_t)dim, (uint32_t)inter, rb_sgu, st, both))) return rc;
+    // 3) down -> Z
+    if (routed_dn && (rc = gemm(std::false_type{}, p->t_down, false, H, (uint32_t)inter, (uint32_t)dim, rb_d, st, both))) return rc;
+    if (nt_shared && !(skip & 16) && (rc = gemm(std::false_type{}, p->t_shared, true, H, (uint32_t)inter, (uint32_t)dim, rb_sd, st, both))) return rc;
+  }
   // 4) ordered reduction into Y
   if ((nt_routed || nt_shared) && !(skip & 32)) {
     const dim3 grid((dim / 4 + 255) / 256, (unsigned)n), block(256);
