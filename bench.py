@@ -31,9 +31,9 @@ HBM_PEAK_GBPS = 8000.0
 
 # HBM bytes per launch of the decode gate/up kernel, from the FETCH_SIZE / WRITE_SIZE counter runs of this workload
 # (KiB per dispatch, scaled by what the same counters read for a 1 GiB copy: x2.000 and x1.000): 42.92 MB + 0.06 MB
-GU_TRAFFIC_BYTES = 42983346
+GU_TRAFFIC_BYTES = 42983355
 # HBM bytes of the launches of the prefill gate/up GEMM together (same counters, same scaling), configs[3]
-PF_GU_TRAFFIC_BYTES = 4288940933
+PF_GU_TRAFFIC_BYTES = 4325703722
 
 
 def cores():
@@ -743,9 +743,14 @@ def main():
     ap.add_argument("--warmup", type=int, default=100)
     ap.add_argument("--workload", default="moe_decode",
                     choices=["moe_decode", "moe_prefill", "matvec_iq1s", "matvec_iq2xxs", "q8_0", "matvec_n", "router", "matmul", "stream", "copy_calibration", "issue_probe"])
+    ap.add_argument("--one-stream", action="store_true",
+                    help="profiling runs: msq_moe_prefill keeps its launches on one stream (MSQ_MOEP_ONE_STREAM=1), so that "
+                         "per-kernel durations and counters are not those of two kernels sharing the device")
     ap.add_argument("--gpu-only", action="store_true",
                     help="profiling runs: skip the CPU baseline leg and the prefill appendix of the default workload")
     args = ap.parse_args()
+    if args.one_stream:
+        os.environ["MSQ_MOEP_ONE_STREAM"] = "1"
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU (one MI355X per box); --gpus %d is not supported" % args.gpus, file=sys.stderr)
         sys.exit(2)
