@@ -441,27 +441,28 @@ __global__ __launch_bounds__(256) void moe_pf_header_kernel(uint32_t* dst, const
   for (uint32_t i = threadIdx.x; i < n; i += blockDim.x) dst[i] = c.w[i];
 }
 
-// Xg[i] = fp16(X[src(i)]): i < total gathers token tok[i]; rows total .. total + n - 1 are the tokens themselves
+// Xg[i] = fp16(X[src(i)]): i < total gathers token tok[i]; rows total .. total + n - 1 are the tokens themselves. One
+// workgroup per row, eight elements (one 16-byte store) per thread and pass.
 template <bool X_BF16>
 __global__ __launch_bounds__(256) void moe_pf_gather_kernel(const void* __restrict__ X, uint16_t* __restrict__ Xg,
                                                             const int* __restrict__ tok, uint32_t total, uint32_t nrows,
                                                             uint32_t dim) {
-  const uint32_t i = blockIdx.y;
+  const uint32_t i = blockIdx.x;
   if (i >= nrows) return;
   const uint32_t src = i < total ? (uint32_t)tok[i] : i - total;
-  for (uint32_t c4 = blockIdx.x * blockDim.x + threadIdx.x; c4 < dim / 4; c4 += gridDim.x * blockDim.x) {
-    float4 v;
+  auto f = [](uint32_t w) { return __builtin_bit_cast(float, w); };
+  for (uint32_t c8 = threadIdx.x; c8 < dim / 8; c8 += blockDim.x) {
+    u32x4 o;
     if constexpr (X_BF16) {
-      const uint2 b = ((const uint2*)((const uint16_t*)X + (size_t)src * dim))[c4];
-      v = make_float4(__builtin_bit_cast(float, b.x << 16), __builtin_bit_cast(float, b.x & 0xFFFF0000u),
-                      __builtin_bit_cast(float, b.y << 16), __builtin_bit_cast(float, b.y & 0xFFFF0000u));
+      const u32x4 b = ((const u32x4*)((const uint16_t*)X + (size_t)src * dim))[c8];
+      o = u32x4{pack_h2(f(b.x << 16), f(b.x & 0xFFFF0000u)), pack_h2(f(b.y << 16), f(b.y & 0xFFFF0000u)),
+                pack_h2(f(b.z << 16), f(b.z & 0xFFFF0000u)), pack_h2(f(b.w << 16), f(b.w & 0xFFFF0000u))};
     } else {
-      v = ((const float4*)((const float*)X + (size_t)src * dim))[c4];
+      const u32x4* p = (const u32x4*)((const float*)X + (size_t)src * dim) + 2 * (size_t)c8;
+      const u32x4 lo = p[0], hi = p[1];
+      o = u32x4{pack_h2(f(lo.x), f(lo.y)), pack_h2(f(lo.z), f(lo.w)), pack_h2(f(hi.x), f(hi.y)), pack_h2(f(hi.z), f(hi.w))};
     }
-    uint2 o;
-    o.x = pack_h2(v.x, v.y);
-    o.y = pack_h2(v.z, v.w);
-    ((uint2*)(Xg + (size_t)i * dim))[c4] = o;
+    ((u32x4*)(Xg + (size_t)i * dim))[c8] = o;
   }
 }
 

@@ -164,6 +164,8 @@ int msq_moe_prefill(void* stream, const MsqMoePrefillArgs* p) {
   const size_t xbytes = (size_t)n * dim * (p->x_is_bf16 ? 2 : 4);
   if (!buf_ok(&p->X, xbytes) || !buf_ok(&p->Y, (size_t)n * dim * 4))
     return fail(MSQ_ERR_ARGUMENT, "macseek quant: moe_prefill: X / Y missing or too small");
+  if (((uintptr_t)bptr(&p->X) & 15) || ((uintptr_t)bptr(&p->Y) & 15) || ((uintptr_t)bptr(&p->scratch) & 255))
+    return fail(MSQ_ERR_ARGUMENT, "macseek quant: moe_prefill: X / Y not 16-byte aligned or scratch not 256-byte aligned");
   if (total > 0 && (!buf_ok(&p->tok, (size_t)total * 4) || !buf_ok(&p->wt, (size_t)total * 4)))
     return fail(MSQ_ERR_ARGUMENT, "macseek quant: moe_prefill: tok / wt missing or too small");
   if (p->k_per_token > 0 && !buf_ok(&p->slot_of, (size_t)n * p->k_per_token * 4))
@@ -268,7 +270,7 @@ int msq_moe_prefill(void* stream, const MsqMoePrefillArgs* p) {
   const uint32_t grows = (uint32_t)(total + (p->has_shared ? n : 0));
   auto gather = [&]() {
     if (grows > 0 && !(skip & 1)) {
-      const dim3 grid((dim / 4 + 255) / 256, grows), block(256);
+      const dim3 grid(grows), block(256);
       const int* tok = total > 0 ? (const int*)bptr(&p->tok) : nullptr;
       if (p->x_is_bf16) hipLaunchKernelGGL((moe_pf_gather_kernel<true>), grid, block, 0, st, (const void*)bptr(&p->X), Xg, tok, (uint32_t)total, grows, (uint32_t)dim);
       else hipLaunchKernelGGL((moe_pf_gather_kernel<false>), grid, block, 0, st, (const void*)bptr(&p->X), Xg, tok, (uint32_t)total, grows, (uint32_t)dim);
