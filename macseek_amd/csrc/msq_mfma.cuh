@@ -253,13 +253,16 @@ __device__ __forceinline__ uint32_t blk_col_of(uint32_t q, uint32_t j) { return 
 // entries are, so the random lookups run at the conflict-free rate.
 struct BlkIQ2XXS {
   static constexpr int LDS_WORDS = (MSQ_IQ2XXS_GRID_N + 128) * 16 * 4, BLOCK_BYTES = 66;
+  // the sign table comes first: both table bases then fit the 16-bit offset field of the LDS instructions (signs at 0,
+  // grid at 32 KB), and a lookup address is one v_and_or of the entry index and the lane's column
+  static constexpr uint32_t GRID_AT = 128u * 256u;
   __device__ static void fill_lds(uint32_t* lds, int tid, int nt) {
     const uint4* grid = (const uint4*)g_tbl_iq2xxs.w;
     const uint4* sign = (const uint4*)g_tbl_sign.w;
     uint4* dst = (uint4*)lds;
     for (int i = tid; i < (MSQ_IQ2XXS_GRID_N + 128) * 16; i += nt) {
       const int e = i >> 4;
-      dst[i] = e < MSQ_IQ2XXS_GRID_N ? grid[e] : sign[e - MSQ_IQ2XXS_GRID_N];
+      dst[i] = e < 128 ? sign[e] : grid[e - 128];
     }
   }
   struct Raw { uint32_t w[4]; uint32_t d; };  // {a0, a1} of sub-block 2 q, then of 2 q + 1; fp16 bits of d
@@ -274,11 +277,11 @@ struct BlkIQ2XXS {
   __device__ static Look lookup(const Raw& r, int j, const uint32_t* tbl, uint32_t col) {
     const uint32_t a0 = r.w[2 * (j >> 2)], a1 = r.w[2 * (j >> 2) + 1];
     const int l = j & 3;
-    const uint32_t cg = col << 4, cs = cg | (MSQ_IQ2XXS_GRID_N * 256u);
+    const uint32_t cg = col << 4;
     const uint32_t g8 = l == 0 ? a0 << 8 : l == 1 ? a0 : a0 >> (8 * l - 8);    // grid index byte at bits 8..15
     const uint32_t s8 = 7 * l < 8 ? a1 << (8 - 7 * l) : a1 >> (7 * l - 8);     // sign index at bits 8..14
     const uint8_t* t8 = (const uint8_t*)tbl;
-    return {*(const uint4*)(t8 + ((g8 & 0xFF00u) | cg)), *(const uint4*)(t8 + ((s8 & 0x7F00u) | cs))};
+    return {*(const uint4*)(t8 + GRID_AT + ((g8 & 0xFF00u) | cg)), *(const uint4*)(t8 + ((s8 & 0x7F00u) | cg))};
   }
   // weight = fp16(d (2 s + 1) / 8) * (+-grid), rounded to fp16 like the reference's dequantized tiles
   // (src/kernels/quant_moe_prefill.metal:153-167): the whole scale rides in the payload
