@@ -115,9 +115,9 @@ int msq_f32_to_f16(void* stream, const MsqBuffer* X, const MsqBuffer* X16, size_
  * Y[n x rows] (+)= X16[n x x_stride] . W^T, X16 fp16 (x_stride = cols if 0), Y F32, any n >= 1, cols % 128 == 0.
  * Weights are rounded to fp16 and products accumulate in fp32, the reference's numerics (quant.hpp:36-39).
  * Up to 128 tokens (256 on matrices of at most 2048 rows; MSQ_MM_FUSED_MAX=N in the environment: up to N) a fused
- * kernel serves the call: nothing is allocated and the call only enqueues. When the matrix has few tiles it sums K
- * slices into Y with fp32 atomic adds, so the last bits of Y can differ between runs (MSQ_MM_SPLITK=1: one slice,
- * reproducible). Above, an fp16 copy of W goes to scratch that the library owns (reference: quant.mm:176-184): that
+ * kernel serves the call: nothing is allocated and the call only enqueues. When the matrix has few tiles K is cut into
+ * slices whose partial sums pass through a 32 MB buffer inside the library and are added in order (results repeat bit for
+ * bit; calls on this route share the buffer: one stream at a time). Above, an fp16 copy of W goes to scratch that the library owns (reference: quant.mm:176-184): that
  * scratch only grows (a larger shape allocates a new block, never waits for the stream; inside a stream capture a call
  * that would have to grow it fails with MSQ_ERR_SCRATCH), and calls sharing it must be enqueued on one stream at a time. */
 int msq_matmul_h(void* stream, int qtype, const MsqBuffer* W, int rows, int cols, const MsqBuffer* X16, const MsqBuffer* Y,

@@ -50,6 +50,7 @@ const DeviceInfo& device_info();  // cached facts of the current device (CU coun
 
 // looks up this device's copy of the static MoE scratch (msq_moe.hip); called by msq_init() and by the entry point
 int static_scratch_setup(float** out);
+void matmul_partials_setup();     // msq_matmul.hip: looks up the current device's partial-sum buffer
 void prefill_side_stream_setup();  // msq_prefill.hip: creates the current device's side stream and its two events
 
 // small-N matvec through the dot-product kernels (msq_matvec.hip); MSQ_ERR_UNSUPPORTED, without a message, when the

@@ -5,9 +5,10 @@
 // n >= 512, dequantizes the whole matrix to fp16 once and runs a dense GEMM (quant.mm:204-221). The same two routes
 // exist here; the switch between them sits where they were measured to cross (use_fused below). Fused route:
 // mm_fused_kernel (msq_mm.cuh) decodes each weight tile straight into matrix-core fragments -- no fp16 copy of W or X,
-// no scratch, the call only enqueues; K is cut into slices that are summed into Y with fp32 atomic adds when the tiles
-// alone would not fill the device (then the last bits of Y depend on the order in which the slices finish; MSQ_MM_SPLITK=1
-// keeps one slice per tile and with it bit-reproducible sums). Materialising route: the bit-exact dequantizer writes
+// nothing allocated, the call only enqueues; when the tiles alone would not fill the device K is cut into slices whose
+// partial sums go to a file-scope device buffer and are added in order by a second launch (no floating-point atomics:
+// results repeat bit for bit; calls on this route share the buffer and must be enqueued on one stream at a time).
+// Materialising route: the bit-exact dequantizer writes
 // W as fp16 into library-owned scratch (22 MB for a 7168 x 1536 projection, a few microseconds at 8 TB/s) and the
 // product is a plain fp16 x fp16 -> fp32 GEMM left to rocBLAS. That scratch only grows: a larger request allocates a
 // new block and the old one stays alive until the process ends (work already enqueued may still read it), so growing
@@ -120,13 +121,27 @@ int gemm_f16(hipStream_t st, const uint16_t* W16, const uint16_t* X16, float* Y,
   return MSQ_OK;
 }
 
-__global__ __launch_bounds__(256) void zero_f32_kernel(float* __restrict__ y, size_t n) {
-  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (i < n) y[i] = 0.f;
+// Partial sums of the fused kernel's K slices: a file-scope device array, so the fused route allocates nothing and can
+// be captured. Every GPU holds its own copy; its address is looked up once per device (hipGetSymbolAddress) by
+// msq_init() or the first call. Calls of the fused route share it: like the reference's module scratch
+// (docs/modules/quant.md:265-268) they must be enqueued on one stream at a time.
+constexpr size_t kMmPartialBytes = (size_t)32 << 20;
+__device__ __align__(256) float g_mm_partials[kMmPartialBytes / 4];
+float* g_mm_partials_ptr[16] = {};
+float* mm_partials() {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 16) return nullptr;
+  std::lock_guard<std::mutex> lock(g_mu);
+  if (!g_mm_partials_ptr[dev]) {
+    void* p = nullptr;
+    if (hipGetSymbolAddress(&p, HIP_SYMBOL(g_mm_partials)) != hipSuccess) { (void)hipGetLastError(); return nullptr; }
+    g_mm_partials_ptr[dev] = (float*)p;
+  }
+  return g_mm_partials_ptr[dev];
 }
 
-// K slices per tile: MSQ_MM_SPLITK = 1 keeps every sum inside one workgroup (bit-reproducible results), 0 / unset lets
-// the launcher choose
+// K slices per tile at most: MSQ_MM_SPLITK (experiments; 1 keeps every sum inside one workgroup), 0 / unset lets the
+// launcher choose
 int splitk_limit() {
   static const int v = [] { const char* e = getenv("MSQ_MM_SPLITK"); return e && *e ? atoi(e) : 0; }();
   return v;
@@ -144,17 +159,20 @@ int launch_mm_t(hipStream_t st, MmArgs a) {
     const long gx = (a.rows + 16 * WV - 1) / (16 * WV), gy = (a.n + 16 * TM - 1) / (16 * TM);
     // Few tiles: the K range is cut into slices (at least two stages each) until there are about two workgroups per CU;
     // a workgroup's K loop is a chain of stage latencies, so a call is as slow as its longest chain. The slices of a tile
-    // meet in Y through fp32 atomic adds, in whatever order they finish.
+    // leave their sums in the partial buffer (as many slices as it holds) and a second launch adds them in order.
+    const size_t cnt = (size_t)a.n * a.rows;
     long kz = std::min<long>((2 * cus + gx * gy - 1) / (gx * gy), std::max<long>(1, nstages / 2));
+    kz = std::min<long>(kz, (long)(kMmPartialBytes / (cnt * 4)));
     if (splitk_limit() > 0) kz = std::min<long>(kz, splitk_limit());
+    float* partials = kz > 1 ? mm_partials() : nullptr;
+    if (!partials) kz = 1;
     a.slice_stages = (uint32_t)((nstages + kz - 1) / kz);
     kz = (nstages + a.slice_stages - 1) / a.slice_stages;
-    a.atomic_out = kz > 1 ? 1u : 0u;
-    if (a.atomic_out && !a.accumulate) {
-      const size_t cnt = (size_t)a.n * a.rows;
-      hipLaunchKernelGGL(zero_f32_kernel, dim3((unsigned)((cnt + 255) / 256)), dim3(256), 0, st, a.Y, cnt);
-    }
+    a.partials = kz > 1 ? partials : nullptr;
     hipLaunchKernelGGL((mm_fused_kernel<F, WV, TM, X_F32>), dim3((unsigned)gx, (unsigned)gy, (unsigned)kz), dim3(64 * WV), lds, st, a);
+    if (a.partials)
+      hipLaunchKernelGGL(mm_reduce_kernel, dim3((unsigned)((cnt + 255) / 256)), dim3(256), 0, st, (const float*)a.partials, a.Y, cnt,
+                         (uint32_t)kz, a.accumulate);
     MSQ_HIP(hipGetLastError());
     return MSQ_OK;
   };
@@ -199,6 +217,9 @@ int matmul_big(hipStream_t st, int t, const MsqBuffer* W, int rows, int cols, co
 }
 
 }  // namespace
+
+void matmul_partials_setup() { (void)mm_partials(); }
+
 }  // namespace msq
 
 using namespace msq;

@@ -315,6 +315,7 @@ int msq_init(void) {
   const DeviceInfo& d = device_info();
   if (!d.ok) return fail(MSQ_ERR_HIP, "macseek quant: no gfx950 device is current");
   prefill_side_stream_setup();
+  matmul_partials_setup();
   return static_scratch_setup(nullptr);
 }
 const char* msq_last_error(void) { return g_err; }

@@ -5,7 +5,8 @@
 //
 // A workgroup of WV waves owns 16 WV weight rows x 16 TM tokens of one K slice (blockIdx.z). A workgroup's K loop is a
 // chain of stage latencies and a small matrix has few tiles, so the host cuts K into slices until the device holds about
-// two workgroups per CU; the slices of a tile then meet in Y through fp32 atomic adds. A wave owns one 16-row tile of W: per K step
+// two workgroups per CU; every slice leaves its tile in a partial-sum buffer and mm_reduce_kernel adds the slices in
+// their order (no floating-point atomics: the result does not depend on which slice finishes first). A wave owns one 16-row tile of W: per K step
 // (32 columns) it decodes the lane's eight weights into exact fp16 payloads + fp32 scale (the fragment decoders of
 // msq_mfma.cuh), rounds scale * payload (+ add) to fp16 once (v_fma_mix: fp32 arithmetic, one rounding -- the value
 // the reference's dequantized tile holds) and feeds TM matrix instructions, one per token tile. The activation tile
@@ -22,7 +23,8 @@ struct MmArgs {
   float* Y;            // [n][rows]
   uint32_t n, rows, cols, x_stride, row_bytes, accumulate;
   uint32_t slice_stages;  // 128-column stages per K slice (blockIdx.z picks the slice)
-  uint32_t atomic_out;    // several K slices: every slice adds its tile to Y with fp32 atomics (Y holds zeros or the sum to add to)
+  float* partials;        // several K slices: slice z leaves its tile in partials[z][n][rows] and a second kernel adds the
+                          // slices in order (null: one slice, written to Y directly)
 };
 
 // F32 and BF16 weight rows as fp16 payloads (the matmul multiplies every type as fp16)
@@ -204,12 +206,29 @@ __global__ __launch_bounds__(64 * WV) void mm_fused_kernel(const MmArgs a) {
         const uint32_t tok = m0 + 16u * t + 4u * q + i;
         if (tok < a.n) {
           float* y = a.Y + (size_t)tok * a.rows + row;
-          if (a.atomic_out) __hip_atomic_fetch_add(y, acc[t][i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          if (a.partials) a.partials[((size_t)blockIdx.z * a.n + tok) * a.rows + row] = acc[t][i];
           else *y = a.accumulate ? *y + acc[t][i] : acc[t][i];
         }
       }
     }
   }
+}
+
+// Y (+)= partials[0] + partials[1] + ... in that order, element by element
+__global__ __launch_bounds__(256) void mm_reduce_kernel(const float* __restrict__ partials, float* __restrict__ Y, size_t count,
+                                                        uint32_t slices, uint32_t accumulate) {
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= count) return;
+  float s = 0.f;
+  for (uint32_t z0 = 0; z0 < slices; z0 += 8u) {  // eight slices requested before the first is added
+    float t[8];
+#pragma unroll
+    for (uint32_t k = 0; k < 8u; k++) t[k] = partials[(size_t)min(z0 + k, slices - 1u) * count + i];
+#pragma unroll
+    for (uint32_t k = 0; k < 8u; k++)
+      if (z0 + k < slices) s += t[k];
+  }
+  Y[i] = accumulate ? Y[i] + s : s;
 }
 
 }  // namespace msq

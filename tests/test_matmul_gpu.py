@@ -82,9 +82,9 @@ def test_f32_to_f16_and_strided_matmul_h(dev):
 
 
 def test_fused_matmul_in_a_captured_graph(dev):
-    """Up to 128 tokens the call allocates nothing and only enqueues: captured into a HIP graph (the zero fill of Y and
-    the K-sliced kernel), every replay meets the bound of the eager call, with eager work between the replays. (The
-    slices meet in Y through atomic adds, so replays agree to rounding, not bit for bit.)"""
+    """Up to 128 tokens the call allocates nothing and only enqueues: captured into a HIP graph (the K-sliced kernel and
+    the ordered sum of its slices), every replay repeats the eager result bit for bit, with eager work between the
+    replays."""
     t, rows, cols, n = O.Q6_K, 640, 2048, 40
     Wb = O.random_blocks(t, rows * cols, 21)
     X = O.randn(n * cols, 22)
@@ -97,16 +97,18 @@ def test_fused_matmul_in_a_captured_graph(dev):
         q.encode_matmul(q.Enc(side), t, q.Buffer.of(Wd), rows, cols, q.Buffer.of(Xd), q.Buffer.of(Yd), n)  # warm-up
     torch.cuda.current_stream().wait_stream(side)
     torch.cuda.synchronize()
+    eager = Yd.clone()
+    got = eager.cpu().numpy().astype(np.float64).reshape(n, rows)
+    assert float(np.max(np.abs(got - sh) / (mag + 1e-12))) <= 1e-5
     g = torch.cuda.CUDAGraph()
     with torch.cuda.graph(g):
         q.encode_matmul(q.Enc(torch.cuda.current_stream()), t, q.Buffer.of(Wd), rows, cols, q.Buffer.of(Xd), q.Buffer.of(Yd), n)
     for rep in range(4):
-        Yd.fill_(7.0)  # the replay itself must clear Y
+        Yd.fill_(7.0)  # the replay itself must overwrite Y
         torch.cuda.synchronize()
         g.replay()
         torch.cuda.synchronize()
-        got = Yd.cpu().numpy().astype(np.float64).reshape(n, rows)
-        assert float(np.max(np.abs(got - sh) / (mag + 1e-12))) <= 1e-5, f"replay {rep}"
+        assert torch.equal(Yd, eager), f"replay {rep} differs from the eager result"
         _ = (Xd * 2).sum().item()  # eager work between the replays
 
 
