@@ -45,7 +45,7 @@ std::vector<void*> g_retired;  // outgrown blocks: kept until the process ends
 rocblas_handle g_blas = nullptr;
 // Which calls the fused kernel serves. The reference switches to dequantize-then-GEMM at 512 tokens (quant.mm:204); here
 // the switch sits where the two routes were measured to cross on MI355X: the fused kernel wins up to 128 tokens on every
-// matrix tried (Q6_K 1536x7168 at 128 tokens: 25 us against 36 us; 16 tokens: 9.5 against 30) and up to 256 tokens on
+// matrix tried (Q6_K 1536x7168 at 128 tokens: 22.5 us against 36 us; 16 tokens: 11 against 30) and up to 256 tokens on
 // matrices of at most 2048 rows; above, the materialising route is ahead (IQ4_NL 7168x4096 at 512 tokens: 63 us against
 // 124). MSQ_MM_FUSED_MAX = N makes the switch "up to N tokens" for every matrix (0: never fused).
 bool use_fused(int n, int rows) {
