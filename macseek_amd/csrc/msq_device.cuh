@@ -22,7 +22,8 @@ constexpr int kWave = 64;
 
 // ------------------------------------------------------------------------------------------------ constant tables
 // fp16 images of the codebooks, expanded at compile time from the base-3 packed form.
-struct TblIQ1S { uint32_t w[MSQ_IQ1S_GRID_N * 4]; };      // 8 halves (-1, 0, +1) per entry
+// 8 halves (-1, 0, +1) per entry, then sixteen {2 s + 1, -+ (2 s + 1) / 8} float pairs indexed by the top four bits of qh
+struct TblIQ1S { uint32_t w[MSQ_IQ1S_GRID_N * 4 + 32]; };
 struct TblIQ2XXS { uint32_t w[MSQ_IQ2XXS_GRID_N * 4]; };  // 8 halves (8, 25, 43) per entry
 struct TblSign { uint32_t w[128 * 4]; };                  // 8 fp16 sign-bit masks per 7-bit sign index
 struct TblIQ4NL { uint32_t w[256]; };                     // byte -> {half(kv[lo nibble]), half(kv[hi nibble])}
@@ -46,6 +47,16 @@ constexpr TblIQ1S make_iq1s() {
       const uint32_t hi = hv[c % 3]; c /= 3;
       t.w[4 * i + j] = lo | (hi << 16);
     }
+  }
+  // the sub-block factors of a unit, ready made: entry k = qh >> 12 (bit 3: sign of delta, bits 0..2: s) holds the
+  // floats 2 s + 1 and (k & 8 ? -0.125 : +0.125) * (2 s + 1), both exact
+  for (int k = 0; k < 16; k++) {
+    const int f = 2 * (k & 7) + 1;  // 1, 3, .. 15
+    int e = 0;
+    while ((f >> (e + 1)) != 0) e++;
+    const uint32_t fb = ((uint32_t)(e + 127) << 23) | (((uint32_t)f << (23 - e)) & 0x7FFFFFu);  // float bits of f
+    t.w[MSQ_IQ1S_GRID_N * 4 + 2 * k] = fb;
+    t.w[MSQ_IQ1S_GRID_N * 4 + 2 * k + 1] = (fb - (3u << 23)) | ((k & 8) ? 0x80000000u : 0u);  // f / 8 with delta's sign
   }
   return t;
 }
@@ -368,10 +379,19 @@ __device__ __forceinline__ float sum_h2(const uint32_t* v, int n) {
 
 // ---- IQ1_S: {fp16 d; u8 qs[32]; u16 qh[8]}, 50 bytes / 256 weights; unit = one 32-weight sub-block
 struct DecIQ1S {
-  static constexpr int UNIT = 32, LDS_WORDS = MSQ_IQ1S_GRID_N * 4;
+  static constexpr int UNIT = 32, GRID_WORDS = MSQ_IQ1S_GRID_N * 4, LDS_WORDS = GRID_WORDS + 32;
   static constexpr bool STAGE_X = true;
   typedef X32 X;
   struct Raw { uint32_t qs, qh, d; };
+  // The two sub-block factors of a unit, {2 s + 1, delta (2 s + 1)}, come from the table behind the grid: one 8-byte read
+  // (sixteen entries in distinct banks: conflict-free) instead of six vector instructions.
+  __device__ static float2 factors(const Raw& r, const uint32_t* lds) {
+    return *(const float2*)((const uint8_t*)lds + GRID_WORDS * 4 + ((r.qh >> 9) & 0x78u));
+  }
+  // d (2 s + 1) (acc + delta sx)
+  __device__ static float scaled(const Raw& r, float2 f, float acc, float sx) {
+    return half_bits_to_float(r.d) * __builtin_fmaf(f.x, acc, f.y * sx);
+  }
   __device__ static void fill_lds(uint32_t* lds, int tid, int nt) { copy_words16(lds, g_tbl_iq1s.w, LDS_WORDS, tid, nt); }
   static constexpr int NTBL = 1;
   __device__ static CopyJob tbl_job(int, uint32_t at) { return {(const uint4*)g_tbl_iq1s.w, at, LDS_WORDS / 4, false}; }
@@ -409,17 +429,16 @@ struct DecIQ1S {
       acc = dot2(g.z, x.v[4 * l + 2], acc);
       acc = dot2(g.w, x.v[4 * l + 3], acc);
     }
-    const float dl = half_bits_to_float(r.d) * (float)(2u * ((r.qh >> 12) & 7u) + 1u);
-    const float delta = (r.qh & 0x8000u) ? -0.125f : 0.125f;
-    return dl * (acc + delta * x.sx);
+    return scaled(r, factors(r, lds), acc, x.sx);
   }
   // the same dot split for software pipelining: lookup() only issues the table reads of a stage, partial() consumes
   // them (the last stage applies the scale), so a caller can keep the next stage's reads in flight during the math
   static constexpr int STAGES = 1;
-  struct Look { uint4 g[4]; };
+  struct Look { uint4 g[4]; float2 f; };
   __device__ static Look lookup(const Raw& r, int, const uint32_t* lds) {
     const uint8_t* grid = (const uint8_t*)lds;
     Look k;
+    k.f = factors(r, lds);
 #pragma unroll
     for (int l = 0; l < 4; l++) {
       const uint32_t off = (((r.qs >> (8 * l)) & 0xFFu) << 4) | (((r.qh >> (3 * l)) & 7u) << 12);
@@ -442,9 +461,7 @@ struct DecIQ1S {
       acc1 = dot2(k.g[l + 1].w, x.v[4 * l + 7], acc1);
     }
     acc += acc1;
-    const float dl = half_bits_to_float(r.d) * (float)(2u * ((r.qh >> 12) & 7u) + 1u);
-    const float delta = (r.qh & 0x8000u) ? -0.125f : 0.125f;
-    return dl * (acc + delta * x.sx);
+    return scaled(r, k.f, acc, x.sx);
   }
 };
 
