@@ -535,10 +535,6 @@ __global__ __launch_bounds__(MAXT) void moe_down_kernel(const MoeArgs a) {
 #pragma unroll
       for (int j = 0; j < RPW; j++) cur[j] = DR::load(Dr + (size_t)min(w0 + j, w1 - 1) * a.rb_d_r, unit_r);
     }
-    if constexpr (RING_S) {
-#pragma unroll
-      for (int s = 0; s < NSH; s++) fetch_s(s);
-    }
     if (first) {
       // h rows this launch reads: the routed ones [0, NE), then the shared one at n_routed (NE is 0 or n_routed)
       const uint32_t lo = NE ? 0u : a.n_routed * a.inter;
@@ -560,6 +556,12 @@ __global__ __launch_bounds__(MAXT) void moe_down_kernel(const MoeArgs a) {
       if (!valid_r) xr = typename DR::X{};
       if (!valid_s) xs = typename DS::X{};
       first = false;
+    }
+    // the shared expert's first rows are requested only now: they are not needed before the routed rows are done, and
+    // requested with the routed ones they lengthen the queue that the prologue's copy waits behind
+    if constexpr (RING_S) {
+#pragma unroll
+      for (int s = 0; s < NSH; s++) fetch_s(s);
     }
     // ---- routed expert e, rows w0 .. w1
     if (NE) {
