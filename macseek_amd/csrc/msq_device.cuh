@@ -355,13 +355,12 @@ __device__ __forceinline__ void load_x32_consecutive(const float* x, uint32_t* v
     v[2 * i + 1] = pack_h2(f.z * s, f.w * s);
   }
 }
+// sum of 2 n fp16 values in fp32: one dot product with (1, 1) per pair instead of two conversions and two additions
 __device__ __forceinline__ float sum_h2(const uint32_t* v, int n) {
+  const h2_t one = {(_Float16)1, (_Float16)1};
   float s = 0.f;
 #pragma unroll
-  for (int i = 0; i < n; i++) {
-    const h2_t h = as_h2(v[i]);
-    s += (float)h.x + (float)h.y;
-  }
+  for (int i = 0; i < n; i++) s = __builtin_amdgcn_fdot2(as_h2(v[i]), one, s, false);
   return s;
 }
 

@@ -96,6 +96,12 @@ __device__ __forceinline__ const void* table_entry(const uint64_t* table, uint32
   return (const void*)((cptr_t)(uintptr_t)table)[i];
 }
 
+// floor(a / b) for a < 4096 and 0 < b <= 64 in four instructions instead of the forty of an integer division (wave
+// counts and rows of a chunk): (a + 0.5) / b lies at least 1 / 128 away from every integer, and the float product is
+// within 1 / 1024 of it.
+__device__ __forceinline__ uint32_t small_div(uint32_t a, uint32_t b) {
+  return (uint32_t)(((float)a + 0.5f) * __builtin_amdgcn_rcpf((float)b));
+}
 __device__ __forceinline__ uint32_t uniform(uint32_t v) { return (uint32_t)__builtin_amdgcn_readfirstlane((int)v); }
 __device__ __forceinline__ const void* uniform(const void* p) {
   const uint64_t v = (uint64_t)p;
@@ -491,8 +497,8 @@ __global__ __launch_bounds__(MAXT) void moe_down_kernel(const MoeArgs a) {
   const uint32_t NE = a.run_routed ? a.n_routed : 0u;       // routed experts computed here
   const uint32_t E = max(NE, 1u);
   const uint32_t wpg = E * KS;                              // waves per row-group
-  const uint32_t RW = nwaves / wpg, rg = uniform(wave / wpg), wl = uniform(wave % wpg);
-  const uint32_t e = uniform(wl / KS), ks = uniform(wl % KS);
+  const uint32_t RW = uniform(small_div(nwaves, wpg)), rg = uniform(small_div(wave, wpg)), wl = wave - rg * wpg;
+  const uint32_t e = uniform(small_div(wl, KS)), ks = wl - e * KS;
   const uint32_t slots = 4 * (NE * KS + (a.run_shared ? KS : 0u));  // partial sums per row: 4 per contributing wave
   const uint32_t PSTRIDE = slots + 1;
 
@@ -513,9 +519,12 @@ __global__ __launch_bounds__(MAXT) void moe_down_kernel(const MoeArgs a) {
   bool first = true;
   for (uint32_t c0 = wg_begin; c0 < wg_end; c0 += kMoeChunkRows) {
     const uint32_t c1 = min(wg_end, c0 + kMoeChunkRows), n = c1 - c0;
-    const uint32_t run = uniform((n + RW - 1) / RW);
+    const uint32_t run = uniform(small_div(n + RW - 1, RW));
     const uint32_t w0 = uniform(min(c0 + rg * run, c1)), w1 = uniform(min(w0 + run, c1));
 
+    // the value of y that this thread adds to in the epilogue, requested ahead of the rows (14.3 -> 14.15 us)
+    float yq = 0.f;
+    if (tid < n) yq = a.y[c0 + tid];
     // ---- request the first rows of both matrices
     typename DR::Raw cur[RING_R ? 1 : RPW], nxt[RING_R ? 1 : RPW];
     uint32_t pv = w0;  // routed ring cursor
@@ -617,7 +626,7 @@ __global__ __launch_bounds__(MAXT) void moe_down_kernel(const MoeArgs a) {
     __syncthreads();
     for (uint32_t t = tid; t < n; t += blockDim.x) {
       const float s = sum_in_order(part + t * PSTRIDE, slots);
-      a.y[c0 + t] += s * (1.f / kHScale);
+      a.y[c0 + t] = (t == tid ? yq : a.y[c0 + t]) + s * (1.f / kHScale);
     }
     __syncthreads();
   }
