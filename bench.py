@@ -188,8 +188,9 @@ def bench_moe_decode(torch, args):
     # eager event pairs also bracket the host's launch latency whenever the queue runs dry; the graph figure does not
     gu_graph = graph_ms_per_launch(torch, lambda i: run_part(i, q.MoePart.Gu), n_ev)
     dn_graph = graph_ms_per_launch(torch, lambda i: run_part(i, q.MoePart.Down), n_ev)
-    gu_bytes = TOPK * 2 * gu_b + 2 * sgu_b + DIM * 4 + h_bytes
-    dn_bytes = TOPK * dn_b + sdn_b + h_bytes + 2 * DIM * 4
+    # h leaves gate/up as fp32 and as fp16 (6 bytes a value); down reads the fp16 copy (2 bytes a value)
+    gu_bytes = TOPK * 2 * gu_b + 2 * sgu_b + DIM * 4 + h_bytes * 3 // 2
+    dn_bytes = TOPK * dn_b + sdn_b + h_bytes // 2 + 2 * DIM * 4
     achieved = gu_bytes / (gu_graph * 1e-3) / 1e9
 
     # parity spot check of the last state against the oracle is the tests' job; here only the CPU baseline leg

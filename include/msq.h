@@ -172,7 +172,8 @@ typedef struct MsqMoeDecodeArgs {
   MsqExpertSlot shared;
   MsqBuffer x;     /* F32[dim] */
   MsqBuffer y;     /* F32[dim], the result is ACCUMULATED into y */
-  MsqBuffer scratch; /* >= msq_moe_decode_scratch_bytes(inter): F32 h[(MSQ_MAX_ROUTED + 1)][inter] */
+  MsqBuffer scratch; /* >= msq_moe_decode_scratch_bytes(inter): F32 h[(MSQ_MAX_ROUTED + 1)][inter], then the same values
+                      * as F16 (x 128, the form the down kernel multiplies; written for IQ1_S / IQ2_XXS down + shared) */
   /* launch shape overrides, 0 = default: rows per wave (nr) and row-waves per workgroup (rsg) of the gate/up and
    * down kernels. They never change a row's summation order (reference: quant.hpp:67-69). */
   int gu_nr, gu_rsg, d_nr, d_rsg;
@@ -209,7 +210,7 @@ int msq_moe_decode_table_part(void* stream, const MsqMoeDecodeArgs* a, const Msq
 
 /* No counterpart in the reference. msq_moe_decode for callers that cannot allocate device memory (code under HIP
  * graph capture, tight serving loops, harnesses that forbid hipMalloc): `a->scratch` is ignored, the h rows live in a
- * device array inside the library (7 x 4096 floats = 112 KiB per GPU, held until the process ends), and the call
+ * device array inside the library (7 x 4096 x 6 bytes = 168 KiB per GPU, held until the process ends), and the call
  * allocates nothing. inter above msq_moe_decode_static_max_inter() (4096) is refused with MSQ_ERR_SCRATCH. Every call
  * on a GPU uses that GPU's one array: calls that overlap on one GPU (two streams) race; calls on one stream do not.
  * Results are bit-identical to msq_moe_decode with caller scratch. */

@@ -255,11 +255,12 @@ __device__ __forceinline__ void copy_words16(uint32_t* dst, const uint32_t* src,
 typedef uint32_t __attribute__((ext_vector_type(4))) u32x4;
 
 // One piece of a workgroup's prologue copy into LDS: n16 16-byte items from device memory to the LDS word offset dst;
-// padded: the items are activations and go to the padded rows of XLds (below).
+// pad_shift: 0, or four words of padding follow every 1 << pad_shift items (3: fp32 activations for the padded rows of
+// XLds below, 2: fp16 activations in the same arrangement, see XHalf).
 struct CopyJob {
   const uint4* src;
   uint32_t dst, n16;
-  bool padded;
+  uint32_t pad_shift;
 };
 // All pieces as one pass over their concatenation, K items per thread in flight: every load of a batch is requested
 // before the first LDS store waits for one (piece by piece, each copy would cost its own round trip to memory).
@@ -278,14 +279,14 @@ __device__ __forceinline__ void copy_jobs(uint32_t* smem, const CopyJob (&jobs)[
       const uint32_t i = min(base + k * nt, total - 1u);
       // the piece item i falls in: the last one that starts at or before i (pieces of no items are passed over)
       const uint4* src = jobs[0].src;
-      uint32_t dst = jobs[0].dst, pad = jobs[0].padded ? 4u : 0u, loc = i, first = 0;
+      uint32_t dst = jobs[0].dst, ps = jobs[0].pad_shift, loc = i, first = 0;
 #pragma unroll
       for (int j = 1; j < NJ; j++) {
         first += jobs[j - 1].n16;
-        if (i >= first) { src = jobs[j].src; dst = jobs[j].dst; pad = jobs[j].padded ? 4u : 0u; loc = i - first; }
+        if (i >= first) { src = jobs[j].src; dst = jobs[j].dst; ps = jobs[j].pad_shift; loc = i - first; }
       }
       v[k] = src[loc];
-      dw[k] = dst + 4u * loc + (loc >> 3) * pad;
+      dw[k] = dst + 4u * loc + (ps ? (loc >> ps) * 4u : 0u);
     }
 #pragma unroll
     for (int k = 0; k < K; k++)
@@ -299,7 +300,7 @@ __device__ __forceinline__ CopyJob tbl_job_of(int k, uint32_t at, bool live) {
   if constexpr (requires { D::NTBL; }) {
     if (live && k < D::NTBL) return D::tbl_job(k, at);
   }
-  return {nullptr, 0u, 0u, false};
+  return {nullptr, 0u, 0u, 0u};
 }
 
 // ------------------------------------------------------------------------------------------------ x slices
@@ -364,6 +365,21 @@ __device__ __forceinline__ float sum_h2(const uint32_t* v, int n) {
   return s;
 }
 
+// Activations that are already fp16 pairs (the h of the MoE layer, scaled and rounded by the kernel that wrote it): a
+// 32-value slice is 16 words, read as it is. Staged in LDS, four words of padding follow every slice (20 words apart:
+// 16 consecutive lanes hit 16 different bank quads, as with XLds).
+__host__ __device__ constexpr uint32_t xhalf_words(uint32_t cols) { return (cols >> 5) * 20u; }
+__device__ __forceinline__ X32 load_x32_half(const uint32_t* p) {
+  X32 r;
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    const u32x4 q = ((const u32x4*)p)[i];
+    r.v[4 * i] = q.x; r.v[4 * i + 1] = q.y; r.v[4 * i + 2] = q.z; r.v[4 * i + 3] = q.w;
+  }
+  r.sx = sum_h2(r.v, 16);
+  return r;
+}
+
 // ================================================================================================ decoders (n = 1)
 // Interface of a decoder D:
 //   UNIT            columns one lane owns per unit
@@ -393,7 +409,7 @@ struct DecIQ1S {
   }
   __device__ static void fill_lds(uint32_t* lds, int tid, int nt) { copy_words16(lds, g_tbl_iq1s.w, LDS_WORDS, tid, nt); }
   static constexpr int NTBL = 1;
-  __device__ static CopyJob tbl_job(int, uint32_t at) { return {(const uint4*)g_tbl_iq1s.w, at, LDS_WORDS / 4, false}; }
+  __device__ static CopyJob tbl_job(int, uint32_t at) { return {(const uint4*)g_tbl_iq1s.w, at, LDS_WORDS / 4, 0u}; }
   template <class S>
   __device__ static X load_x(S x, uint32_t u, float s = 1.f) {
     X r;
@@ -476,8 +492,8 @@ struct DecIQ2XXS {
   }
   static constexpr int NTBL = 2;
   __device__ static CopyJob tbl_job(int k, uint32_t at) {
-    if (k == 0) return {(const uint4*)g_tbl_iq2xxs.w, at, MSQ_IQ2XXS_GRID_N, false};
-    return {(const uint4*)g_tbl_sign.w, at + MSQ_IQ2XXS_GRID_N * 4, 128, false};
+    if (k == 0) return {(const uint4*)g_tbl_iq2xxs.w, at, MSQ_IQ2XXS_GRID_N, 0u};
+    return {(const uint4*)g_tbl_sign.w, at + MSQ_IQ2XXS_GRID_N * 4, 128, 0u};
   }
   template <class S>
   __device__ static X load_x(S x, uint32_t u, float s = 1.f) {

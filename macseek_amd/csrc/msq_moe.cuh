@@ -61,7 +61,32 @@ struct MoeArgs {
   // activations staged through LDS (padded rows of XLds): word offset in dynamic LDS, or read straight from device
   // memory when stage_x is 0 (rows too long for LDS)
   uint32_t xs_off, stage_x;
+  // Second copy of h as fp16, scaled by kHScale and rounded by the gate/up kernel: the form in which the down kernel's
+  // X32 decoders multiply it (half the bytes for every workgroup of the down kernel to stage, and no conversion there).
+  // Null when the down kernel's decoder pair does not read it (kHalfH).
+  _Float16* h16;
 };
+
+// h value i of the layer: fp32 for the caller's eyes, and the fp16 form that the down kernel would otherwise make of it
+__device__ __forceinline__ void store_h(const MoeArgs& a, size_t i, float v) {
+  a.h[i] = v;
+  if (a.h16) a.h16[i] = (_Float16)(v * kHScale);
+}
+// Whether the down kernel with decoders DR / DS reads h in the fp16 form (a property of the decoder pair, so that the
+// kernel holds one form only; the host passes MoeArgs::h16 by the same rule).
+template <class DR, class DS>
+constexpr bool kHalfH = std::is_same_v<typename DR::X, X32> && std::is_same_v<typename DS::X, X32>;
+// the lane's slice (unit u) of the h row that starts at column col0 of the staged rows hs / of the rows in device memory
+template <class D, bool HALF>
+__device__ __forceinline__ typename D::X load_h_staged(const uint32_t* hs, uint32_t col0, uint32_t u) {
+  if constexpr (HALF) return load_x32_half(hs + xhalf_words(col0) + 20u * u);
+  else return D::load_x(XLds{(const float*)hs + xlds_words(col0)}, u, kHScale);
+}
+template <class D, bool HALF>
+__device__ __forceinline__ typename D::X load_h_direct(const MoeArgs& a, uint32_t col0, uint32_t u) {
+  if constexpr (HALF) return load_x32_half((const uint32_t*)a.h16 + (col0 >> 1) + 16u * u);
+  else return D::load_x(a.h + col0, u, kHScale);
+}
 
 __device__ __forceinline__ float swiglu(float g, float u, float w) {  // quant_moe.metal:23-27
   g = fminf(g, 10.f);
@@ -154,7 +179,7 @@ __device__ __forceinline__ void moe_gu_run_direct(const MoeArgs& a, uint32_t* tb
     }
     if (first) {  // tables and activations arrive while the first weight rows are in flight
       const CopyJob jobs[3] = {tbl_job_of<D>(0, 0u, true), tbl_job_of<D>(1, 0u, true),
-                               {(const uint4*)a.x, (uint32_t)(smem - tbl) + a.xs_off, a.stage_x ? a.dim / 4u : 0u, true}};
+                               {(const uint4*)a.x, (uint32_t)(smem - tbl) + a.xs_off, a.stage_x ? a.dim / 4u : 0u, 3u}};
       copy_jobs<4>(tbl, jobs, tid, blockDim.x);
       if (a.stage_x) {
         __syncthreads();
@@ -204,7 +229,7 @@ __device__ __forceinline__ void moe_gu_run_direct(const MoeArgs& a, uint32_t* tb
         const uint32_t v = c0 + (q >> 1);
         const uint32_t e = shared ? 0u : v / a.inter, r = v - e * a.inter;
         const uint32_t he = shared ? a.n_routed : e;
-        a.h[(size_t)he * a.inter + r] = swiglu(sum, other, shared ? 1.f : a.wts[e]);
+        store_h(a, (size_t)he * a.inter + r, swiglu(sum, other, shared ? 1.f : a.wts[e]));
       }
     }
     __syncthreads();
@@ -299,7 +324,7 @@ __device__ __forceinline__ void moe_gu_run_ring(const MoeArgs& a, uint32_t* tbl,
         }
       } else {
         const CopyJob jobs[3] = {tbl_job_of<D>(0, 0u, true), tbl_job_of<D>(1, 0u, true),
-                                 {(const uint4*)a.x, (uint32_t)(smem - tbl) + a.xs_off, a.stage_x ? a.dim / 4u : 0u, true}};
+                                 {(const uint4*)a.x, (uint32_t)(smem - tbl) + a.xs_off, a.stage_x ? a.dim / 4u : 0u, 3u}};
         copy_jobs<4>(tbl, jobs, tid, blockDim.x);
         if (a.stage_x) {
           __syncthreads();
@@ -405,7 +430,7 @@ __device__ __forceinline__ void moe_gu_run_ring(const MoeArgs& a, uint32_t* tbl,
         const uint32_t v = c0 + (q >> 1);
         const uint32_t e = shared ? 0u : v / a.inter, r = v - e * a.inter;
         const uint32_t he = shared ? a.n_routed : e;
-        a.h[(size_t)he * a.inter + r] = swiglu(sum, other, shared ? 1.f : a.wts[e]);
+        store_h(a, (size_t)he * a.inter + r, swiglu(sum, other, shared ? 1.f : a.wts[e]));
       }
     }
     __syncthreads();
@@ -482,6 +507,7 @@ __device__ __forceinline__ void down_rows_ring(const uint32_t* tbl, const typena
 template <class DR, class DS, int MAXT>
 __global__ __launch_bounds__(MAXT) void moe_down_kernel(const MoeArgs a) {
   constexpr bool RING_R = requires { DR::STAGES; }, RING_S = requires { DS::STAGES; };
+  constexpr bool HALF = kHalfH<DR, DS>;
   constexpr int RPW = rows_in_flight<DR>(1);
   constexpr int NR = 4, NSH = 4;  // ring depth: routed rows, shared rows
   constexpr int TBL = DR::LDS_WORDS + DS::LDS_WORDS;
@@ -556,16 +582,19 @@ __global__ __launch_bounds__(MAXT) void moe_down_kernel(const MoeArgs a) {
       const uint32_t hi = (a.run_shared ? a.n_routed + 1u : a.n_routed) * a.inter;
       const CopyJob jobs[5] = {tbl_job_of<DR>(0, 0u, NE), tbl_job_of<DR>(1, 0u, NE),
                                tbl_job_of<DS>(0, DR::LDS_WORDS, a.run_shared), tbl_job_of<DS>(1, DR::LDS_WORDS, a.run_shared),
-                               {(const uint4*)(a.h + lo), (uint32_t)(smem - tbl) + a.xs_off, a.stage_x ? (hi - lo) / 4u : 0u, true}};
+                               HALF ? CopyJob{(const uint4*)(a.h16 + lo), (uint32_t)(smem - tbl) + a.xs_off,
+                                              a.stage_x ? (hi - lo) / 8u : 0u, 2u}
+                                    : CopyJob{(const uint4*)(a.h + lo), (uint32_t)(smem - tbl) + a.xs_off,
+                                              a.stage_x ? (hi - lo) / 4u : 0u, 3u}};
       copy_jobs<(MAXT <= 768 ? 8 : 4)>(tbl, jobs, tid, blockDim.x);
       if (a.stage_x) {
-        const float* hs = (const float*)(smem + a.xs_off);
+        const uint32_t* hs = smem + a.xs_off;
         __syncthreads();
-        if (NE) xr = DR::load_x(XLds{hs + xlds_words(e * a.inter)}, unit_r, kHScale);
-        if (a.run_shared) xs = DS::load_x(XLds{hs + xlds_words(a.n_routed * a.inter - lo)}, unit_s, kHScale);
+        if (NE) xr = load_h_staged<DR, HALF>(hs, e * a.inter, unit_r);
+        if (a.run_shared) xs = load_h_staged<DS, HALF>(hs, a.n_routed * a.inter - lo, unit_s);
       } else {
-        if (NE) xr = DR::load_x(a.h + (size_t)e * a.inter, unit_r, kHScale);
-        if (a.run_shared) xs = DS::load_x(a.h + (size_t)a.n_routed * a.inter, unit_s, kHScale);
+        if (NE) xr = load_h_direct<DR, HALF>(a, e * a.inter, unit_r);
+        if (a.run_shared) xs = load_h_direct<DS, HALF>(a, a.n_routed * a.inter, unit_s);
         __syncthreads();
       }
       if (!valid_r) xr = typename DR::X{};

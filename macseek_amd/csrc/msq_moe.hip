@@ -14,7 +14,7 @@ namespace msq {
 // uses the array's name as an address (it is only a handle for hipGetSymbolAddress), but the per-device pointer that
 // static_scratch_setup() looks up once, with that device current.
 constexpr int kStaticMaxInter = 4096;  // largest expert intermediate size the static scratch serves
-static __device__ __align__(256) float g_moe_static_scratch[(kMaxRouted + 1) * kStaticMaxInter];
+static __device__ __align__(256) float g_moe_static_scratch[(kMaxRouted + 1) * kStaticMaxInter * 3 / 2];  // fp32 h + fp16 h
 constexpr int kStaticMaxDevices = 64;
 static float* g_static_ptr[kStaticMaxDevices];
 static std::mutex g_static_mu;
@@ -163,6 +163,10 @@ int moe_decode_impl(hipStream_t st, const MsqMoeDecodeArgs* p, const MsqBuffer* 
       return fail(MSQ_ERR_ARGUMENT, "macseek quant: moe_decode: shared expert missing or too small");
     a.sgate = bptr(&s.gate); a.sup = bptr(&s.up); a.sdown = bptr(&s.down);
   }
+  // h also as scaled fp16, behind the fp32 rows, when the down kernel's decoder pair takes its activations in that form
+  // (kHalfH in msq_moe.cuh: both decoders of the instantiation, the placeholder of a layer without shared expert included)
+  auto x32_type = [](int t) { return t == MSQ_IQ1_S || t == MSQ_IQ2_XXS; };
+  if (x32_type(p->t_down) && x32_type(ts)) a.h16 = (_Float16*)(a.h + (size_t)(kMaxRouted + 1) * inter);
   const int cus = device_info().cus;
 
   // 1) gate + up + SwiGLU -> h
@@ -236,7 +240,8 @@ extern "C" int msq_exp_timeline(void* host_out) {
 extern "C" {
 
 size_t msq_moe_decode_scratch_bytes(int inter) {
-  return sizeof(float) * (size_t)(kMaxRouted + 1) * (size_t)(inter > 0 ? inter : MSQ_EXPERT_INTER);
+  // h of the routed experts and the shared one as fp32, then the same values as fp16 (MoeArgs::h16)
+  return (sizeof(float) + sizeof(_Float16)) * (size_t)(kMaxRouted + 1) * (size_t)(inter > 0 ? inter : MSQ_EXPERT_INTER);
 }
 int msq_moe_decode(void* stream, const MsqMoeDecodeArgs* a) {
   return moe_decode_impl((hipStream_t)stream, a, nullptr, MSQ_PART_ALL, false);
@@ -259,7 +264,7 @@ int msq_moe_decode_static(void* stream, const MsqMoeDecodeArgs* a) {
   MsqMoeDecodeArgs b = *a;
   b.scratch.dev = h;
   b.scratch.off = 0;
-  b.scratch.size = sizeof(float) * (size_t)(kMaxRouted + 1) * kStaticMaxInter;
+  b.scratch.size = sizeof(float) * (size_t)(kMaxRouted + 1) * kStaticMaxInter * 3 / 2;
   return moe_decode_impl((hipStream_t)stream, &b, nullptr, MSQ_PART_ALL, false);
 }
 
