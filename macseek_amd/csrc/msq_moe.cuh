@@ -135,7 +135,7 @@ __device__ __forceinline__ const void* uniform(const void* p) {
 
 // gate + up + SwiGLU over the virtual rows [wg * per, ...) of one kind of expert (routed: e * inter + r; shared: r).
 template <class D, int RPW>
-__device__ __forceinline__ void moe_gu_run_direct(const MoeArgs& a, uint32_t* tbl, uint32_t* smem, const bool shared, const uint32_t wg) {
+__device__ __forceinline__ void moe_gu_run_direct(const MoeArgs& a, const uint64_t* table, uint32_t* tbl, uint32_t* smem, const bool shared, const uint32_t wg) {
   float* part = (float*)smem;
   const uint32_t tid = threadIdx.x, lane = tid & 63u;
   const uint32_t wave = uniform(tid >> 6), nwaves = blockDim.x >> 6;
@@ -156,7 +156,7 @@ __device__ __forceinline__ void moe_gu_run_direct(const MoeArgs& a, uint32_t* tb
     const uint32_t e = shared ? 0u : v / a.inter, r = v - e * a.inter;
     const uint8_t* base;
     if (shared) base = which ? a.sup : a.sgate;
-    else if (a.table) base = (const uint8_t*)a.table[3 * e + which];
+    else if (table) base = (const uint8_t*)table[3 * e + which];
     else base = which ? a.up[e] : a.gate[e];
     return as_global(base) + (size_t)r * row_bytes;
   };
@@ -244,7 +244,7 @@ __device__ __forceinline__ void moe_gu_run_direct(const MoeArgs& a, uint32_t* tb
 // names an exact number of loads that may stay in flight. Table lookups run one decoder stage ahead of the dot
 // products (two alternating lookup buffers), so LDS latency overlaps the math as well.
 template <class D>
-__device__ __forceinline__ void moe_gu_run_ring(const MoeArgs& a, uint32_t* tbl, uint32_t* smem, const bool shared, const uint32_t wg) {
+__device__ __forceinline__ void moe_gu_run_ring(const MoeArgs& a, const uint64_t* table, uint32_t* tbl, uint32_t* smem, const bool shared, const uint32_t wg) {
   constexpr int NR = 4;  // row pairs in flight per wave
   constexpr int NS = D::STAGES;
   float* part = (float*)smem;
@@ -284,7 +284,7 @@ __device__ __forceinline__ void moe_gu_run_ring(const MoeArgs& a, uint32_t* tbl,
     const void *pg = nullptr, *pu = nullptr;
     auto set_expert = [&]() {
       if (shared) { pg = a.sgate; pu = a.sup; }
-      else if (a.table) { pg = table_entry(a.table, 3 * pe); pu = table_entry(a.table, 3 * pe + 1); }
+      else if (table) { pg = table_entry(table, 3 * pe); pu = table_entry(table, 3 * pe + 1); }
       else { pg = a.gate[pe]; pu = a.up[pe]; }
       pg = uniform(pg); pu = uniform(pu);  // buffer descriptors live in scalar registers
     };
@@ -439,13 +439,15 @@ __device__ __forceinline__ void moe_gu_run_ring(const MoeArgs& a, uint32_t* tbl,
 }
 
 template <class D>
-__device__ __forceinline__ void moe_gu_run(const MoeArgs& a, uint32_t* tbl, uint32_t* smem, const bool shared, const uint32_t wg) {
-  if constexpr (requires { D::STAGES; }) moe_gu_run_ring<D>(a, tbl, smem, shared, wg);
-  else moe_gu_run_direct<D, rows_in_flight<D>(2)>(a, tbl, smem, shared, wg);
+__device__ __forceinline__ void moe_gu_run(const MoeArgs& a, const uint64_t* table, uint32_t* tbl, uint32_t* smem, const bool shared, const uint32_t wg) {
+  if constexpr (requires { D::STAGES; }) moe_gu_run_ring<D>(a, table, tbl, smem, shared, wg);
+  else moe_gu_run_direct<D, rows_in_flight<D>(2)>(a, table, tbl, smem, shared, wg);
 }
 
+// table: MoeArgs::table once more, as an argument of its own in first place: built with kernel-argument preload it is
+// in scalar registers when the wave starts, and the expert addresses are requested one memory trip earlier.
 template <class DR, class DS>
-__global__ __launch_bounds__(1024) void moe_gu_kernel(const MoeArgs a) {
+__global__ __launch_bounds__(1024) void moe_gu_kernel(const uint64_t* table, const MoeArgs a) {
   // The codebook table is a static array: its LDS address is a compile-time constant that goes into the offset field
   // of the lookups (with a table in dynamic LDS every lookup address ends in an addition of the base). Partial sums and
   // the staged activations follow in dynamic LDS.
@@ -453,8 +455,8 @@ __global__ __launch_bounds__(1024) void moe_gu_kernel(const MoeArgs a) {
   __shared__ __attribute__((aligned(16))) uint32_t tbl[TBL > 0 ? TBL : 4];
   extern __shared__ __attribute__((aligned(16))) uint32_t smem[];
   MSQ_TL(0);
-  if (blockIdx.x < a.grid_routed) moe_gu_run<DR>(a, tbl, smem, false, blockIdx.x);
-  else moe_gu_run<DS>(a, tbl, smem, true, blockIdx.x - a.grid_routed);
+  if (blockIdx.x < a.grid_routed) moe_gu_run<DR>(a, table, tbl, smem, false, blockIdx.x);
+  else moe_gu_run<DS>(a, table, tbl, smem, true, blockIdx.x - a.grid_routed);
 }
 
 // down: workgroup = RW row-groups x (NE expert-waves x KS K-split waves). In a row-group, wave (e, ks) owns routed
@@ -505,7 +507,7 @@ __device__ __forceinline__ void down_rows_ring(const uint32_t* tbl, const typena
 
 // MAXT: largest workgroup the instantiation is launched with (768 threads leave 170 registers per lane, 1024 only 128)
 template <class DR, class DS, int MAXT>
-__global__ __launch_bounds__(MAXT) void moe_down_kernel(const MoeArgs a) {
+__global__ __launch_bounds__(MAXT) void moe_down_kernel(const uint64_t* table, const MoeArgs a) {
   constexpr bool RING_R = requires { DR::STAGES; }, RING_S = requires { DS::STAGES; };
   constexpr bool HALF = kHalfH<DR, DS>;
   constexpr int RPW = rows_in_flight<DR>(1);
@@ -533,7 +535,7 @@ __global__ __launch_bounds__(MAXT) void moe_down_kernel(const MoeArgs a) {
   const bool valid_r = NE && u0 < units_r, valid_s = a.run_shared && u0 < units_s;
   const uint32_t unit_r = u0 < units_r ? u0 : units_r - 1, unit_s = u0 < units_s ? u0 : units_s - 1;
   const void* Dr_ = nullptr;
-  if (NE) Dr_ = uniform(a.table ? table_entry(a.table, 3 * e + 2) : (const void*)a.down[e]);
+  if (NE) Dr_ = uniform(table ? table_entry(table, 3 * e + 2) : (const void*)a.down[e]);
   const gptr_t Dr = as_global(Dr_), Dsh = as_global(a.sdown);
 
   const auto off_r = [&] { if constexpr (RING_R) return DR::offsets(unit_r); else return 0; }();

@@ -42,16 +42,16 @@ bool shared_type_ok(int t) { return t == MSQ_Q6_K || t == MSQ_Q8_0 || t == MSQ_I
 template <class DR, class DS>
 void launch_gu_t(dim3 g, dim3 b, size_t lds, hipStream_t st, const MoeArgs& a) {
   allow_large_lds(moe_gu_kernel<DR, DS>, lds);
-  hipLaunchKernelGGL((moe_gu_kernel<DR, DS>), g, b, lds, st, a);
+  hipLaunchKernelGGL((moe_gu_kernel<DR, DS>), g, b, lds, st, a.table, a);
 }
 template <class DR, class DS>
 void launch_down_t(dim3 g, dim3 b, size_t lds, hipStream_t st, const MoeArgs& a) {
   if (b.x <= 768) {
     allow_large_lds(moe_down_kernel<DR, DS, 768>, lds);
-    hipLaunchKernelGGL((moe_down_kernel<DR, DS, 768>), g, b, lds, st, a);
+    hipLaunchKernelGGL((moe_down_kernel<DR, DS, 768>), g, b, lds, st, a.table, a);
   } else {
     allow_large_lds(moe_down_kernel<DR, DS, 1024>, lds);
-    hipLaunchKernelGGL((moe_down_kernel<DR, DS, 1024>), g, b, lds, st, a);
+    hipLaunchKernelGGL((moe_down_kernel<DR, DS, 1024>), g, b, lds, st, a.table, a);
   }
 }
 // launch-shape knobs for experiments (the reference exposes MACSEEK_MOE_* the same way, quant.mm:274-276)
