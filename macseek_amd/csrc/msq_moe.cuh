@@ -121,12 +121,6 @@ __device__ __forceinline__ const void* table_entry(const uint64_t* table, uint32
   return (const void*)((cptr_t)(uintptr_t)table)[i];
 }
 
-// floor(a / b) for a < 4096 and 0 < b <= 64 in four instructions instead of the forty of an integer division (wave
-// counts and rows of a chunk): (a + 0.5) / b lies at least 1 / 128 away from every integer, and the float product is
-// within 1 / 1024 of it.
-__device__ __forceinline__ uint32_t small_div(uint32_t a, uint32_t b) {
-  return (uint32_t)(((float)a + 0.5f) * __builtin_amdgcn_rcpf((float)b));
-}
 __device__ __forceinline__ uint32_t uniform(uint32_t v) { return (uint32_t)__builtin_amdgcn_readfirstlane((int)v); }
 __device__ __forceinline__ const void* uniform(const void* p) {
   const uint64_t v = (uint64_t)p;

@@ -160,7 +160,8 @@ __global__ __launch_bounds__(1024) void mv_kernel(const MvArgs a) {
 
   for (uint32_t tile = blockIdx.x; tile < a.ntiles; tile += gridDim.x) {
     const uint32_t tile_row0 = tile * tile_rows;
-    const uint32_t group = tile_row0 / a.rows_per_group;  // a tile never straddles two groups (host guarantees)
+    // a tile never straddles two groups (host guarantees)
+    const uint32_t group = a.rows_per_group >= a.rows ? 0u : tile_row0 / a.rows_per_group;
     if (group != cur_group) {
       if constexpr (NORM) {
 #pragma unroll
@@ -249,7 +250,8 @@ __global__ __launch_bounds__(1024) void mv_ring_kernel(const MvArgs a) {
       first = false;
       if (D::LDS_WORDS) __syncthreads();
     }
-    const uint32_t group = tile_row0 / a.rows_per_group;  // a tile never straddles two groups (host guarantees)
+    // a tile never straddles two groups (host guarantees)
+    const uint32_t group = a.rows_per_group >= a.rows ? 0u : tile_row0 / a.rows_per_group;
     if (group != cur_group) {
       const uint32_t units1[1] = {unit};
       typename D::X x1[1];
@@ -326,9 +328,14 @@ constexpr int tok_round() {
 // Decoders with STAGE_X take the activations through LDS (contiguous loads, tok_round() tokens per round); with the
 // others every lane reads its slices from device memory, all T tokens' loads in flight at once.
 template <class D, int ITERS, int T, bool NORM = false>
-__global__ __launch_bounds__(512) void mv_tok_kernel(const MvTokArgs ta) {
+__global__ __launch_bounds__(512) void mv_tok_kernel(const uint8_t* W_, uint32_t rows_, uint32_t row_bytes_, uint32_t units_, uint32_t ks_,
+                                                     uint32_t rpw_, uint32_t ntiles_, uint32_t rows_per_group_, const MvTokArgs ta) {
   constexpr bool STAGE = D::STAGE_X;
-  const MvArgs& a = ta.m;
+  // what the first weight loads need comes as leading arguments (delivered in scalar registers with the wave when the
+  // file is built with kernel-argument preload); the rest is read from the argument block
+  MvArgs a = ta.m;
+  a.W = W_; a.rows = rows_; a.row_bytes = row_bytes_; a.units = units_; a.ks = ks_; a.rpw = rpw_; a.ntiles = ntiles_;
+  a.rows_per_group = rows_per_group_;
   extern __shared__ __attribute__((aligned(16))) uint32_t smem[];
   // the codebook table is a static array: its LDS address is a compile-time constant, which saves the addition of a base
   // in every lookup address; partial sums (and staged activations) follow in dynamic LDS
@@ -337,7 +344,7 @@ __global__ __launch_bounds__(512) void mv_tok_kernel(const MvTokArgs ta) {
 
   const uint32_t tid = threadIdx.x, lane = tid & 63u, nwaves = blockDim.x >> 6;
   const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
-  const uint32_t KS = a.ks, ks = wave % KS, rw = wave / KS, RW = nwaves / KS;
+  const uint32_t KS = a.ks, rw = small_div(wave, KS), ks = wave - rw * KS, RW = small_div(nwaves, KS);
   const uint32_t tile_rows = RW * a.rpw;
   const uint32_t t0 = blockIdx.y * T;
 
@@ -360,7 +367,8 @@ __global__ __launch_bounds__(512) void mv_tok_kernel(const MvTokArgs ta) {
 
   for (uint32_t tile = blockIdx.x; tile < a.ntiles; tile += gridDim.x) {
     const uint32_t tile_row0 = tile * tile_rows;
-    const uint32_t group = tile_row0 / a.rows_per_group;  // a tile never straddles two groups (host guarantees)
+    // a tile never straddles two groups (host guarantees)
+    const uint32_t group = a.rows_per_group >= a.rows ? 0u : tile_row0 / a.rows_per_group;
     const uint32_t row0 = tile_row0 + rw * a.rpw;
     const uint32_t last = min(min(row0 + a.rpw, a.rows) - 1u, a.rows - 1u);  // last row of this wave's run
     // The wave's first NR rows are on their way while the activations are staged; a slot is refilled with the row NR
