@@ -20,10 +20,10 @@ def sources():
 # Per-file additions. The one-token MoE kernels take the expert address table as their first argument and have it
 # delivered in scalar registers with the wave (kernel-argument preload): the table can be read while the rest of the
 # arguments is still on its way from memory.
-# The token matvec kernel takes what its first weight loads need as nine leading words in the same way (Q8_0 4096 x 4096:
-# 8.25 -> 8.0 us; the codebook formats, whose table is staged first, do not move).
+# The token matvec kernel takes what its first loads need (activations, then weight rows) as twelve leading words in the
+# same way.
 EXTRA = {"msq_moe.hip": ["-mllvm", "-amdgpu-kernarg-preload-count=2"],
-         "msq_matvec.hip": ["-mllvm", "-amdgpu-kernarg-preload-count=9"]}
+         "msq_matvec.hip": ["-mllvm", "-amdgpu-kernarg-preload-count=12"]}
 
 
 def _compile(src):

@@ -211,7 +211,7 @@ int launch_mv_tok(hipStream_t st, const MvShape& s, MvTokArgs& ta) {
   }
   auto launch = [&](auto kernel, dim3 grid) {
     allow_large_lds(kernel, lds);
-    hipLaunchKernelGGL(kernel, grid, dim3(threads), lds, st, a.W, a.rows, a.row_bytes, a.units, a.ks, a.rpw, a.ntiles, a.rows_per_group, ta);
+    hipLaunchKernelGGL(kernel, grid, dim3(threads), lds, st, a.W, a.rows, a.row_bytes, a.units, a.ks, a.rpw, a.ntiles, a.rows_per_group, a.x, a.cols, ta);
   };
   if (a.norm_w) {  // fused input norm (single token)
     if constexpr (T != 1 || requires { D::STAGES; }) return MSQ_ERR_UNSUPPORTED;

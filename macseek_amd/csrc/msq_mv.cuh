@@ -329,13 +329,14 @@ constexpr int tok_round() {
 // others every lane reads its slices from device memory, all T tokens' loads in flight at once.
 template <class D, int ITERS, int T, bool NORM = false>
 __global__ __launch_bounds__(512) void mv_tok_kernel(const uint8_t* W_, uint32_t rows_, uint32_t row_bytes_, uint32_t units_, uint32_t ks_,
-                                                     uint32_t rpw_, uint32_t ntiles_, uint32_t rows_per_group_, const MvTokArgs ta) {
+                                                     uint32_t rpw_, uint32_t ntiles_, uint32_t rows_per_group_, const float* x_,
+                                                     uint32_t cols_, const MvTokArgs ta) {
   constexpr bool STAGE = D::STAGE_X;
   // what the first weight loads need comes as leading arguments (delivered in scalar registers with the wave when the
   // file is built with kernel-argument preload); the rest is read from the argument block
   MvArgs a = ta.m;
   a.W = W_; a.rows = rows_; a.row_bytes = row_bytes_; a.units = units_; a.ks = ks_; a.rpw = rpw_; a.ntiles = ntiles_;
-  a.rows_per_group = rows_per_group_;
+  a.rows_per_group = rows_per_group_; a.x = x_; a.cols = cols_;
   extern __shared__ __attribute__((aligned(16))) uint32_t smem[];
   // the codebook table is a static array: its LDS address is a compile-time constant, which saves the addition of a base
   // in every lookup address; partial sums (and staged activations) follow in dynamic LDS
@@ -348,6 +349,20 @@ __global__ __launch_bounds__(512) void mv_tok_kernel(const uint8_t* W_, uint32_t
   const uint32_t tile_rows = RW * a.rpw;
   const uint32_t t0 = blockIdx.y * T;
 
+  // One token of one group: its activations are requested before anything else, so that they come back ahead of the
+  // table and the weight rows (loads return in order) and are in LDS, converted, when the first rows arrive.
+  constexpr bool EARLY_X = T == 1 && STAGE && !NORM;
+  constexpr int XK = 4;
+  [[maybe_unused]] u32x4 xe[XK];
+  [[maybe_unused]] bool early = false;
+  if constexpr (EARLY_X) {
+    const uint32_t n4 = a.cols >> 2;
+    early = blockIdx.y == 0 && a.rows_per_group >= a.rows && n4 <= XK * blockDim.x;
+    if (early) {
+#pragma unroll
+      for (int k = 0; k < XK; k++) xe[k] = ((const u32x4*)a.x)[min(tid + k * blockDim.x, n4 - 1u)];
+    }
+  }
   D::fill_lds(tbl, (int)tid, (int)blockDim.x);
 
   uint32_t unit[ITERS];
@@ -388,8 +403,22 @@ __global__ __launch_bounds__(512) void mv_tok_kernel(const uint8_t* W_, uint32_t
       // tokens past the last repeat it; their results are never stored
       auto x_of = [&](int t) { return a.x + (size_t)min(t0 + t, ta.n - 1) * ta.x_stride + (size_t)group * a.x_group_stride; };
       constexpr int G = tok_round<D, T>();  // tokens staged per round (the host has made room for G padded rows)
+      bool staged = false;
+      if constexpr (EARLY_X) {
+        if (early && cur_group == 0xFFFFFFFFu) {  // (group 0, token 0: the row requested at the top)
 #pragma unroll
-      for (int t = 0; t < T; t++) {
+          for (int k = 0; k < XK; k++) {
+            const uint32_t i = tid + k * blockDim.x;
+            if (i < (a.cols >> 2)) *(u32x4*)(xs + 4u * i + (i >> 3) * 4u) = xe[k];
+          }
+          __syncthreads();
+#pragma unroll
+          for (int i = 0; i < ITERS; i++) xr[0][i] = D::load_x(XLds{xs}, unit[i]);
+          staged = true;
+        }
+      }
+#pragma unroll
+      for (int t = 0; t < T && !staged; t++) {
         if constexpr (NORM) {
 #pragma unroll
           for (int i = 0; i < ITERS; i++) xr[t][i] = D::load_x(XLds{xs}, unit[i]);
