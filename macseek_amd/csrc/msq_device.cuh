@@ -334,11 +334,11 @@ __device__ __forceinline__ void stage_x_rows(float* dst, const float* const (&sr
                                              uint32_t tid, uint32_t nt) {
   const uint32_t n4 = n >> 2;
   for (uint32_t base = tid; base < n4; base += K * nt) {
-    float4 v[GMAX][K];
+    u32x4 v[GMAX][K];  // (a plain vector type: arrays of the HIP struct types can end up in scratch memory)
 #pragma unroll
     for (int g = 0; g < GMAX; g++) {  // every src[g] is readable (rows past G are loaded and dropped)
 #pragma unroll
-      for (int k = 0; k < K; k++) v[g][k] = ((const float4*)src[g])[min(base + k * nt, n4 - 1u)];
+      for (int k = 0; k < K; k++) v[g][k] = ((const u32x4*)src[g])[min(base + k * nt, n4 - 1u)];
     }
 #pragma unroll
     for (int g = 0; g < GMAX; g++) {
@@ -346,7 +346,7 @@ __device__ __forceinline__ void stage_x_rows(float* dst, const float* const (&sr
 #pragma unroll
         for (int k = 0; k < K; k++) {
           const uint32_t i = base + k * nt;
-          if (i < n4) *(float4*)(dst + g * roww + 4u * i + (i >> 3) * 4u) = v[g][k];
+          if (i < n4) *(u32x4*)(dst + g * roww + 4u * i + (i >> 3) * 4u) = v[g][k];
         }
       }
     }

@@ -332,11 +332,10 @@ __global__ __launch_bounds__(512) void mv_tok_kernel(const uint8_t* W_, uint32_t
                                                      uint32_t rpw_, uint32_t ntiles_, uint32_t rows_per_group_, const float* x_,
                                                      uint32_t cols_, const MvTokArgs ta) {
   constexpr bool STAGE = D::STAGE_X;
-  // what the first weight loads need comes as leading arguments (delivered in scalar registers with the wave when the
-  // file is built with kernel-argument preload); the rest is read from the argument block
-  MvArgs a = ta.m;
-  a.W = W_; a.rows = rows_; a.row_bytes = row_bytes_; a.units = units_; a.ks = ks_; a.rpw = rpw_; a.ntiles = ntiles_;
-  a.rows_per_group = rows_per_group_; a.x = x_; a.cols = cols_;
+  // What the first loads need comes as leading arguments (W_ .. cols_: the fields of the same names in ta.m, delivered
+  // in scalar registers with the wave when the file is built with kernel-argument preload) and is used under those
+  // names below; the rest is read from the argument block.
+  const MvArgs& a = ta.m;
   extern __shared__ __attribute__((aligned(16))) uint32_t smem[];
   // the codebook table is a static array: its LDS address is a compile-time constant, which saves the addition of a base
   // in every lookup address; partial sums (and staged activations) follow in dynamic LDS
@@ -345,8 +344,8 @@ __global__ __launch_bounds__(512) void mv_tok_kernel(const uint8_t* W_, uint32_t
 
   const uint32_t tid = threadIdx.x, lane = tid & 63u, nwaves = blockDim.x >> 6;
   const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
-  const uint32_t KS = a.ks, rw = small_div(wave, KS), ks = wave - rw * KS, RW = small_div(nwaves, KS);
-  const uint32_t tile_rows = RW * a.rpw;
+  const uint32_t KS = ks_, rw = small_div(wave, KS), ks = wave - rw * KS, RW = small_div(nwaves, KS);
+  const uint32_t tile_rows = RW * rpw_;
   const uint32_t t0 = blockIdx.y * T;
 
   // One token of one group: its activations are requested before anything else, so that they come back ahead of the
@@ -356,11 +355,11 @@ __global__ __launch_bounds__(512) void mv_tok_kernel(const uint8_t* W_, uint32_t
   [[maybe_unused]] u32x4 xe[XK];
   [[maybe_unused]] bool early = false;
   if constexpr (EARLY_X) {
-    const uint32_t n4 = a.cols >> 2;
-    early = blockIdx.y == 0 && a.rows_per_group >= a.rows && n4 <= XK * blockDim.x;
+    const uint32_t n4 = cols_ >> 2;
+    early = blockIdx.y == 0 && rows_per_group_ >= rows_ && n4 <= XK * blockDim.x;
     if (early) {
 #pragma unroll
-      for (int k = 0; k < XK; k++) xe[k] = ((const u32x4*)a.x)[min(tid + k * blockDim.x, n4 - 1u)];
+      for (int k = 0; k < XK; k++) xe[k] = ((const u32x4*)x_)[min(tid + k * blockDim.x, n4 - 1u)];
     }
   }
   D::fill_lds(tbl, (int)tid, (int)blockDim.x);
@@ -370,22 +369,22 @@ __global__ __launch_bounds__(512) void mv_tok_kernel(const uint8_t* W_, uint32_t
 #pragma unroll
   for (int i = 0; i < ITERS; i++) {
     const uint32_t u = (ks * ITERS + i) * 64u + lane;
-    valid[i] = u < a.units;
-    unit[i] = valid[i] ? u : a.units - 1;  // idle lanes shadow the last unit; their result is dropped
+    valid[i] = u < units_;
+    unit[i] = valid[i] ? u : units_ - 1;  // idle lanes shadow the last unit; their result is dropped
   }
   typename D::X xr[T][ITERS];
   uint32_t cur_group = 0xFFFFFFFFu;
   float* xs = (float*)(smem + a.xs_off);
   if constexpr (NORM) stage_normed_x(a, smem, xs, tid, lane, wave, nwaves);  // synchronises (one token, one group)
   else if (D::LDS_WORDS) __syncthreads();
-  const uint32_t roww = xlds_words(a.cols);
+  const uint32_t roww = xlds_words(cols_);
 
-  for (uint32_t tile = blockIdx.x; tile < a.ntiles; tile += gridDim.x) {
+  for (uint32_t tile = blockIdx.x; tile < ntiles_; tile += gridDim.x) {
     const uint32_t tile_row0 = tile * tile_rows;
     // a tile never straddles two groups (host guarantees)
-    const uint32_t group = a.rows_per_group >= a.rows ? 0u : tile_row0 / a.rows_per_group;
-    const uint32_t row0 = tile_row0 + rw * a.rpw;
-    const uint32_t last = min(min(row0 + a.rpw, a.rows) - 1u, a.rows - 1u);  // last row of this wave's run
+    const uint32_t group = rows_per_group_ >= rows_ ? 0u : tile_row0 / rows_per_group_;
+    const uint32_t row0 = tile_row0 + rw * rpw_;
+    const uint32_t last = min(min(row0 + rpw_, rows_) - 1u, rows_ - 1u);  // last row of this wave's run
     // The wave's first NR rows are on their way while the activations are staged; a slot is refilled with the row NR
     // places ahead before its own bytes are used (rows past the run's last repeat it: no branch around a load).
     // Four rows in flight pay for the codebook formats at one token (a row slice is 8 bytes per lane: IQ1_S 4096x7168
@@ -395,13 +394,13 @@ __global__ __launch_bounds__(512) void mv_tok_kernel(const uint8_t* W_, uint32_t
     typename D::Raw ring[NR][ITERS];
 #pragma unroll
     for (int s = 0; s < NR; s++) {
-      const gptr_t wr = as_global(a.W) + (size_t)min(row0 + s, last) * a.row_bytes;
+      const gptr_t wr = as_global(W_) + (size_t)min(row0 + s, last) * row_bytes_;
 #pragma unroll
       for (int i = 0; i < ITERS; i++) ring[s][i] = D::load(wr, unit[i]);
     }
     if (group != cur_group) {
       // tokens past the last repeat it; their results are never stored
-      auto x_of = [&](int t) { return a.x + (size_t)min(t0 + t, ta.n - 1) * ta.x_stride + (size_t)group * a.x_group_stride; };
+      auto x_of = [&](int t) { return x_ + (size_t)min(t0 + t, ta.n - 1) * ta.x_stride + (size_t)group * a.x_group_stride; };
       constexpr int G = tok_round<D, T>();  // tokens staged per round (the host has made room for G padded rows)
       bool staged = false;
       if constexpr (EARLY_X) {
@@ -409,7 +408,7 @@ __global__ __launch_bounds__(512) void mv_tok_kernel(const uint8_t* W_, uint32_t
 #pragma unroll
           for (int k = 0; k < XK; k++) {
             const uint32_t i = tid + k * blockDim.x;
-            if (i < (a.cols >> 2)) *(u32x4*)(xs + 4u * i + (i >> 3) * 4u) = xe[k];
+            if (i < (cols_ >> 2)) *(u32x4*)(xs + 4u * i + (i >> 3) * 4u) = xe[k];
           }
           __syncthreads();
 #pragma unroll
@@ -417,8 +416,9 @@ __global__ __launch_bounds__(512) void mv_tok_kernel(const uint8_t* W_, uint32_t
           staged = true;
         }
       }
+      if (!staged) {
 #pragma unroll
-      for (int t = 0; t < T && !staged; t++) {
+      for (int t = 0; t < T; t++) {
         if constexpr (NORM) {
 #pragma unroll
           for (int i = 0; i < ITERS; i++) xr[t][i] = D::load_x(XLds{xs}, unit[i]);
@@ -431,12 +431,13 @@ __global__ __launch_bounds__(512) void mv_tok_kernel(const uint8_t* W_, uint32_t
             const float* src[G];
 #pragma unroll
             for (int k = 0; k < G; k++) src[k] = x_of(t + k);
-            stage_x_rows<G>(xs, src, G, roww, a.cols, tid, blockDim.x);
+            stage_x_rows<G>(xs, src, G, roww, cols_, tid, blockDim.x);
             __syncthreads();
           }
 #pragma unroll
           for (int i = 0; i < ITERS; i++) xr[t][i] = D::load_x(XLds{xs + (t % G) * roww}, unit[i]);
         }
+      }
       }
       cur_group = group;
     }
@@ -453,22 +454,22 @@ __global__ __launch_bounds__(512) void mv_tok_kernel(const uint8_t* W_, uint32_t
       }
       // transposed fold: afterwards acc[0] of lane l is token group8_sel<T>(l) summed over l's 16-lane row
       row16_fold<T>(acc, lane);
-      if (!(lane & 8u)) part[(((rw * a.rpw + j) * KS + ks) * 4 + (lane >> 4)) * T + group8_sel<T>(lane)] = acc[0];
+      if (!(lane & 8u)) part[(((rw * rpw_ + j) * KS + ks) * 4 + (lane >> 4)) * T + group8_sel<T>(lane)] = acc[0];
     };
-    for (uint32_t j0 = 0; j0 < a.rpw; j0 += NR) {
+    for (uint32_t j0 = 0; j0 < rpw_; j0 += NR) {
 #pragma unroll
       for (int s = 0; s < NR; s++) {
         typename D::Raw cur[ITERS];
-        const gptr_t wr = as_global(a.W) + (size_t)min(row0 + j0 + s + NR, last) * a.row_bytes;
+        const gptr_t wr = as_global(W_) + (size_t)min(row0 + j0 + s + NR, last) * row_bytes_;
 #pragma unroll
         for (int i = 0; i < ITERS; i++) { cur[i] = ring[s][i]; ring[s][i] = D::load(wr, unit[i]); }
-        if (NR == 1 || j0 + s < a.rpw) row_dot(cur, j0 + s);  // wave-uniform; no load inside
+        if (NR == 1 || j0 + s < rpw_) row_dot(cur, j0 + s);  // wave-uniform; no load inside
       }
     }
     __syncthreads();
     for (uint32_t idx = tid; idx < tile_rows * T; idx += blockDim.x) {
       const uint32_t r = idx % tile_rows, t = idx / tile_rows, row = tile_row0 + r;  // consecutive lanes: consecutive rows
-      if (row < a.rows && t0 + t < ta.n) {
+      if (row < rows_ && t0 + t < ta.n) {
         const float s = sum_in_order(part + r * 4 * KS * T + t, 4 * KS, T);
         float* y = a.y + (size_t)(t0 + t) * ta.y_stride + row;
         *y = a.accumulate ? *y + s : s;
