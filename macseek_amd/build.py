@@ -1,5 +1,7 @@
 """Build libmsq.so (hipcc, gfx950 only) in-tree. `python -m macseek_amd.build` or `build()`."""
+import json
 import os
+import re
 import subprocess
 import sys
 from concurrent.futures import ThreadPoolExecutor
@@ -26,26 +28,54 @@ EXTRA = {"msq_moe.hip": ["-mllvm", "-amdgpu-kernarg-preload-count=2"],
          "msq_matvec.hip": ["-mllvm", "-amdgpu-kernarg-preload-count=12"]}
 
 
+# What the compiler reports per kernel (-Rpass-analysis=kernel-resource-usage) is kept beside the library: registers, LDS
+# and, above all, scratch bytes per lane -- a kernel that starts to keep an array or spilled registers in scratch memory
+# still computes the right thing, several times slower, and tests/test_kernel_resources.py reads this file to notice.
+REPORT = os.path.join(HERE, "libmsq.kernels.json")
+_FIELDS = {"VGPRs": "vgprs", "AGPRs": "agprs", "TotalSGPRs": "sgprs", "ScratchSize [bytes/lane]": "scratch",
+           "VGPRs Spill": "vgpr_spill", "LDS Size [bytes/block]": "lds", "Occupancy [waves/SIMD]": "occupancy"}
+
+
+def _resources(text):
+    kernels, cur = {}, None
+    for l in text.splitlines():
+        m = re.search(r"remark:\s+Function Name: (\S+)", l)
+        if m:
+            cur = kernels.setdefault(m.group(1), {})
+            continue
+        m = re.search(r"remark:\s+([A-Za-z][A-Za-z \[\]/]*?): (\d+)", l)
+        if m and cur is not None and m.group(1) in _FIELDS:
+            cur[_FIELDS[m.group(1)]] = int(m.group(2))
+    return kernels
+
+
 def _compile(src):
     obj = os.path.join(OBJDIR, os.path.basename(src)[:-4] + ".o")
-    r = subprocess.run([HIPCC] + FLAGS + EXTRA.get(os.path.basename(src), []) + ["-c", src, "-o", obj],
+    r = subprocess.run([HIPCC] + FLAGS + EXTRA.get(os.path.basename(src), []) +
+                       ["-Rpass-analysis=kernel-resource-usage", "-c", src, "-o", obj],
                        stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
-    out = "\n".join(l for l in r.stdout.splitlines() if "packed-fp32-ops" not in l)
     if r.returncode != 0:
+        out = "\n".join(l for l in r.stdout.splitlines() if "packed-fp32-ops" not in l and "remark:" not in l)
         raise RuntimeError("hipcc failed for %s:\n%s" % (src, out))
-    return obj
+    return obj, _resources(r.stdout)
 
 
 def build(verbose=True):
     os.makedirs(OBJDIR, exist_ok=True)
     srcs = sources()
     with ThreadPoolExecutor(max_workers=min(8, len(srcs))) as ex:
-        objs = list(ex.map(_compile, srcs))
+        done = list(ex.map(_compile, srcs))
+    objs = [o for o, _ in done]
+    report = {}
+    for (_, k), src in zip(done, srcs):
+        report[os.path.basename(src)] = k
     r = subprocess.run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", OUT] + objs +
                        ["-L/opt/rocm/lib", "-lrocblas", "-Wl,-rpath,/opt/rocm/lib"],  # rocBLAS: the dense fp16 GEMM of msq_matmul for many tokens
                        stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     if r.returncode != 0:
         raise RuntimeError("link failed:\n" + r.stdout)
+    with open(REPORT, "w") as f:
+        json.dump(report, f, indent=1, sort_keys=True)
     if verbose:
         print("built", OUT, "from", [os.path.basename(s) for s in srcs])
     return OUT
