@@ -287,8 +287,8 @@ int matvec_tok(hipStream_t st, int t, const uint8_t* W, int rows, int cols, cons
                int groups, const MsqMvCfg* cfg, const float* norm_w, float eps) {
   MsqMvCfg several;
   if (n > 1) cfg = effective_cfg(cfg, true, &several);
-  // Q8_0 keeps fp32 activations (32 registers per token): four tokens per pass, the other formats eight
-  const int T = n == 1 ? 1 : (t == MSQ_Q8_0 || n <= 4) ? 4 : 8;
+  // tokens per pass over the weights: one, two, four or eight (Q8_0 keeps fp32 activations, 32 registers per token: four at most)
+  const int T = n <= 2 ? n : (t == MSQ_Q8_0 || n <= 4) ? 4 : 8;
   MvShape s;
   if (!mv_tok_shape(t, rows, cols, groups, (n + T - 1) / T, cfg, &s)) return MSQ_ERR_UNSUPPORTED;
   if (n == 1 && !tok_serves_single(t, rows, cols, s, cfg)) return MSQ_ERR_UNSUPPORTED;
@@ -300,8 +300,8 @@ int matvec_tok(hipStream_t st, int t, const uint8_t* W, int rows, int cols, cons
   ta.n = (uint32_t)n; ta.x_stride = (uint32_t)((size_t)cols * groups); ta.y_stride = (uint32_t)rows;
   a.norm_w = norm_w; a.eps = eps;
   if (n == 1) return t == MSQ_Q8_0 ? launch_mv_tok<DecQ8_0, 1>(st, s, ta) : launch_mv_tok_t<1>(st, t, s, ta);
-  if (t == MSQ_Q8_0) return launch_mv_tok<DecQ8_0, 4>(st, s, ta);
-  return T == 4 ? launch_mv_tok_t<4>(st, t, s, ta) : launch_mv_tok_t<8>(st, t, s, ta);
+  if (t == MSQ_Q8_0) return T == 2 ? launch_mv_tok<DecQ8_0, 2>(st, s, ta) : launch_mv_tok<DecQ8_0, 4>(st, s, ta);
+  return T == 2 ? launch_mv_tok_t<2>(st, t, s, ta) : T == 4 ? launch_mv_tok_t<4>(st, t, s, ta) : launch_mv_tok_t<8>(st, t, s, ta);
 }
 
 }  // namespace msq
