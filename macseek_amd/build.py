@@ -25,7 +25,8 @@ def sources():
 # The token matvec kernel takes what its first loads need (activations, then weight rows) as twelve leading words in the
 # same way.
 EXTRA = {"msq_moe.hip": ["-mllvm", "-amdgpu-kernarg-preload-count=2"],
-         "msq_matvec.hip": ["-mllvm", "-amdgpu-kernarg-preload-count=12"]}
+         "msq_matvec.hip": ["-mllvm", "-amdgpu-kernarg-preload-count=12"],
+         "msq_router.hip": ["-mllvm", "-amdgpu-kernarg-preload-count=6"]}  # x, W, dim, n_exp of the fused router: 11.1 -> 10.8 us
 
 
 # What the compiler reports per kernel (-Rpass-analysis=kernel-resource-usage) is kept beside the library: registers, LDS

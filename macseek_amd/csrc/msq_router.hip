@@ -113,11 +113,10 @@ __global__ __launch_bounds__(256) void router_topk_kernel(const float* __restric
 // counter, one increment per workgroup: n_exp / 4 of them contend, not n_exp) selects from the keys, then re-arms the
 // counter. W is F32 (QT = MSQ_F32) or BF16. No bit of the result depends on which workgroup is last.
 template <int QT>
-__global__ __launch_bounds__(256) void router_fused_kernel(const float* __restrict__ x, const void* __restrict__ W,
-                                                           const float* __restrict__ bias, float* logits, RouterRec* recs,
-                                                           uint32_t* counter, int* __restrict__ ids,
-                                                           float* __restrict__ wts, uint32_t dim, uint32_t n_exp,
-                                                           float route_scale) {
+__global__ __launch_bounds__(256) void router_fused_kernel(const float* __restrict__ x, const void* __restrict__ W, uint32_t dim,
+                                                           uint32_t n_exp, const float* __restrict__ bias, float* logits,
+                                                           RouterRec* recs, uint32_t* counter, int* __restrict__ ids,
+                                                           float* __restrict__ wts, float route_scale) {
   __shared__ uint32_t last;
   const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6, e = blockIdx.x * 4u + wave;
   // the row's weights are requested U vectors per lane at a time before any is used: with one wave per row the loop is
@@ -373,12 +372,12 @@ int msq_router_fused(void* stream, int wtype, const MsqBuffer* x, const MsqBuffe
   hipStream_t st = (hipStream_t)stream;
   if (wtype == MSQ_F32)
     hipLaunchKernelGGL((router_fused_kernel<MSQ_F32>), grid, block, 0, st, (const float*)bptr(x), (const void*)bptr(W),
-                       (const float*)bptr(bias), logits, recs, counter, (int*)bptr_mut(ids), (float*)bptr_mut(w), (uint32_t)dim,
-                       (uint32_t)n_exp, route_scale);
+                       (uint32_t)dim, (uint32_t)n_exp, (const float*)bptr(bias), logits, recs, counter, (int*)bptr_mut(ids),
+                       (float*)bptr_mut(w), route_scale);
   else
     hipLaunchKernelGGL((router_fused_kernel<MSQ_BF16>), grid, block, 0, st, (const float*)bptr(x), (const void*)bptr(W),
-                       (const float*)bptr(bias), logits, recs, counter, (int*)bptr_mut(ids), (float*)bptr_mut(w), (uint32_t)dim,
-                       (uint32_t)n_exp, route_scale);
+                       (uint32_t)dim, (uint32_t)n_exp, (const float*)bptr(bias), logits, recs, counter, (int*)bptr_mut(ids),
+                       (float*)bptr_mut(w), route_scale);
   MSQ_HIP(hipGetLastError());
   return MSQ_OK;
 }
