@@ -39,32 +39,38 @@ constexpr int kMoeChunkRows = 128;  // rows a workgroup finishes between two syn
 // 5e-7 stays out of its denormals.
 constexpr float kHScale = 128.f;
 
+// Field order: the scalar cache fetches the argument block line by line (64 bytes), one miss after the other, so what
+// a kernel needs before its first weight row can be requested sits together at the front -- gate/up finds it in the
+// first line (the block starts 8 bytes into the segment, behind the table address), down in the first two -- and the
+// by-value expert addresses, unused when a table is passed, at the end.
 struct MoeArgs {
   const float* x;        // [dim]
-  float* h;              // scratch: [(n_routed + 1)][inter]
+  uint32_t dim, inter;
+  uint32_t ks;           // K-split waves
+  uint32_t n_routed;     // h row of the shared expert
+  uint32_t run_routed;   // experts this launch computes: routed ones (0 or 1) ...
+  uint32_t run_shared;   // ... and / or the shared one
+  // activations staged through LDS (padded rows of XLds): word offset in dynamic LDS, or read straight from device
+  // memory when stage_x is 0 (rows too long for LDS)
+  uint32_t xs_off, stage_x;
+  uint32_t grid_routed;  // gate/up: workgroups [0, grid_routed) take routed rows, the rest shared rows
+  uint32_t rows_per_wg_r, rb_gu_r, rows_per_wg_s;  // gate/up: virtual rows (expert * inter + row) per workgroup; row bytes
+  uint32_t rb_gu_s;      // row bytes: shared gate/up
+  uint32_t rows_per_wg;  // down: rows of y per workgroup
+  uint32_t rb_d_r, rb_d_s;  // row bytes: routed down, shared down
+  const uint8_t* sdown;
   float* y;              // [dim], accumulated
+  // Second copy of h as fp16, scaled by kHScale and rounded by the gate/up kernel: the form in which the down kernel's
+  // X32 decoders multiply it (half the bytes for every workgroup of the down kernel to stage, and no conversion there).
+  // Null when the down kernel's decoder pair does not read it (kHalfH).
+  _Float16* h16;
+  float* h;              // scratch: [(n_routed + 1)][inter]
+  const uint8_t *sgate, *sup;
   const float* wts;      // [n_routed] routing weights (device memory)
   const uint64_t* table; // kMaxRouted x {gate, up, down} device addresses, or null to use the arrays below
   const uint8_t* gate[kMaxRouted];
   const uint8_t* up[kMaxRouted];
   const uint8_t* down[kMaxRouted];
-  const uint8_t *sgate, *sup, *sdown;
-  uint32_t n_routed;     // h row of the shared expert
-  uint32_t run_routed;   // experts this launch computes: routed ones (0 or 1) ...
-  uint32_t run_shared;   // ... and / or the shared one
-  uint32_t dim, inter;
-  uint32_t rb_gu_r, rb_d_r, rb_gu_s, rb_d_s;  // row bytes: routed gate/up, routed down, shared gate/up, shared down
-  uint32_t ks;           // K-split waves
-  uint32_t grid_routed;  // gate/up: workgroups [0, grid_routed) take routed rows, the rest shared rows
-  uint32_t rows_per_wg_r, rows_per_wg_s;  // gate/up: virtual rows (expert * inter + row) per workgroup
-  uint32_t rows_per_wg;  // down: rows of y per workgroup
-  // activations staged through LDS (padded rows of XLds): word offset in dynamic LDS, or read straight from device
-  // memory when stage_x is 0 (rows too long for LDS)
-  uint32_t xs_off, stage_x;
-  // Second copy of h as fp16, scaled by kHScale and rounded by the gate/up kernel: the form in which the down kernel's
-  // X32 decoders multiply it (half the bytes for every workgroup of the down kernel to stage, and no conversion there).
-  // Null when the down kernel's decoder pair does not read it (kHalfH).
-  _Float16* h16;
 };
 
 // h value i of the layer: fp32 for the caller's eyes, and the fp16 form that the down kernel would otherwise make of it
