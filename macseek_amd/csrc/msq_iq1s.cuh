@@ -75,12 +75,12 @@ __device__ __forceinline__ float dpp_maxf(float v) {
 // through three DPP exchanges. A batch of K items per thread is requested (xq_issue) before it is quantized and
 // stored (xq_finish), so a caller can put its other loads in flight in between.
 template <int K>
-struct XqBatch { float4 v[K]; };
+struct XqBatch { f4_t v[K]; };  // (plain vector types: arrays of the HIP struct types can end up in scratch memory)
 template <int K>
 __device__ __forceinline__ XqBatch<K> xq_issue(const float* src, uint32_t n4, uint32_t base, uint32_t nt) {
   XqBatch<K> b;
 #pragma unroll
-  for (int k = 0; k < K; k++) b.v[k] = ((const float4*)src)[min(base + k * nt, n4 - 1u)];
+  for (int k = 0; k < K; k++) b.v[k] = ((const f4_t*)src)[min(base + k * nt, n4 - 1u)];
   return b;
 }
 template <int K>
@@ -88,7 +88,7 @@ __device__ __forceinline__ void xq_finish(uint32_t* dst, const XqBatch<K>& b, ui
 #pragma unroll
   for (int k = 0; k < K; k++) {
     const uint32_t i = base + k * nt;  // groups of eight lanes are in range, or out of it, together (n4 % 8 == 0)
-    const float4 v = b.v[k];
+    const float4 v = {b.v[k].x, b.v[k].y, b.v[k].z, b.v[k].w};
     float m = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
     m = dpp_maxf<0x141>(m); m = dpp_maxf<0xB1>(m); m = dpp_maxf<0x4E>(m);
     const int e = xq_exponent(m);
@@ -132,11 +132,11 @@ struct DecIQ1SQ {
   // ---- tables. The grid comes from device memory (32 KB, two entries per 16-byte item; issue_tables requests a
   // thread's items, finish_tables writes each into both copies); the two small tables are computed.
   static constexpr uint32_t ITEMS = MSQ_IQ1S_GRID_N;  // 16-byte items of the image
-  struct TblRegs { uint4 v[2]; };
+  struct TblRegs { u32x4 v[2]; };
   __device__ static TblRegs issue_tables(uint32_t tid, uint32_t nt) {
     TblRegs r;
 #pragma unroll
-    for (int j = 0; j < 2; j++) r.v[j] = ((const uint4*)g_tbl_iq1s8.w)[min(tid + j * nt, ITEMS - 1u)];
+    for (int j = 0; j < 2; j++) r.v[j] = ((const u32x4*)g_tbl_iq1s8.w)[min(tid + j * nt, ITEMS - 1u)];
     return r;
   }
   __device__ static void finish_tables(uint32_t* lds, const TblRegs& r, uint32_t tid, uint32_t nt) {
@@ -149,10 +149,10 @@ struct DecIQ1SQ {
       lds[LUT_LO_AT + b] = ((b & 7u) << 3) | (((b >> 3) & 7u) << 11) | (((b >> 6) & 3u) << 19);
     }
     // image byte o = 16 i = (b << 7) | (sign << 6) | (h << 3) goes to LDS byte (b << 8) | (c << 7) | (o & 127)
-    auto put = [&](uint32_t i, const uint4& v) {
+    auto put = [&](uint32_t i, const u32x4& v) {
       const uint32_t o = 16u * i, at = (((o & ~127u) << 1) | (o & 127u)) >> 2;
-      *(uint4*)(lds + GRID_AT + at) = v;
-      *(uint4*)(lds + GRID_AT + at + 32u) = v;
+      *(u32x4*)(lds + GRID_AT + at) = v;
+      *(u32x4*)(lds + GRID_AT + at + 32u) = v;
     };
 #pragma unroll
     for (int j = 0; j < 2; j++)
@@ -163,7 +163,7 @@ struct DecIQ1SQ {
       // writes per launch)
       uint32_t t2 = tid;
       asm volatile("" : "+v"(t2));
-      for (uint32_t i0 = t2 + 2u * nt; i0 < ITEMS; i0 += nt) put(i0, ((const uint4*)g_tbl_iq1s8.w)[i0]);
+      for (uint32_t i0 = t2 + 2u * nt; i0 < ITEMS; i0 += nt) put(i0, ((const u32x4*)g_tbl_iq1s8.w)[i0]);
     }
   }
   __device__ static void fill_lds(uint32_t* lds, uint32_t tid, uint32_t nt) { finish_tables(lds, issue_tables(tid, nt), tid, nt); }
