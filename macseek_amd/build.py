@@ -26,7 +26,8 @@ def sources():
 # same way.
 EXTRA = {"msq_moe.hip": ["-mllvm", "-amdgpu-kernarg-preload-count=2"],
          "msq_matvec.hip": ["-mllvm", "-amdgpu-kernarg-preload-count=12"],
-         "msq_router.hip": ["-mllvm", "-amdgpu-kernarg-preload-count=6"]}  # x, W, dim, n_exp of the fused router: 11.1 -> 10.8 us
+         "msq_router.hip": ["-mllvm", "-amdgpu-kernarg-preload-count=6"],  # x, W, dim, n_exp of the fused router: 11.1 -> 10.8 us
+         "msq_matmul.hip": ["-mllvm", "-amdgpu-kernarg-preload-count=14"]}  # the fused matmul's arguments: 2-3 % at 64 / 128 tokens
 
 
 # What the compiler reports per kernel (-Rpass-analysis=kernel-resource-usage) is kept beside the library: registers, LDS

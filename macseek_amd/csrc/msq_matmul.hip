@@ -169,7 +169,8 @@ int launch_mm_t(hipStream_t st, MmArgs a) {
     a.slice_stages = (uint32_t)((nstages + kz - 1) / kz);
     kz = (nstages + a.slice_stages - 1) / a.slice_stages;
     a.partials = kz > 1 ? partials : nullptr;
-    hipLaunchKernelGGL((mm_fused_kernel<F, WV, TM, X_F32>), dim3((unsigned)gx, (unsigned)gy, (unsigned)kz), dim3(64 * WV), lds, st, a);
+    hipLaunchKernelGGL((mm_fused_kernel<F, WV, TM, X_F32>), dim3((unsigned)gx, (unsigned)gy, (unsigned)kz), dim3(64 * WV), lds, st, a.X, a.W, a.Y,
+                       a.n, a.rows, a.cols, a.x_stride, a.row_bytes, a.accumulate, a.slice_stages, a.partials);
     if (a.partials)
       hipLaunchKernelGGL(mm_reduce_kernel, dim3((unsigned)((cnt + 255) / 256)), dim3(256), 0, st, (const float*)a.partials, a.Y, cnt,
                          (uint32_t)kz, a.accumulate);

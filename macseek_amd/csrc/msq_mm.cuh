@@ -72,7 +72,12 @@ constexpr int kMmKStage = 128, kMmPitch = kMmKStage * 2 + 16;  // bytes per stag
 
 // WV waves (16 weight rows each) x TM token tiles per workgroup
 template <class F, int WV, int TM, bool X_F32>
-__global__ __launch_bounds__(64 * WV) void mm_fused_kernel(const MmArgs a) {
+__global__ __launch_bounds__(64 * WV) void mm_fused_kernel(const void* X_, const uint8_t* W_, float* Y_, uint32_t n_, uint32_t rows_,
+                                                           uint32_t cols_, uint32_t x_stride_, uint32_t row_bytes_, uint32_t accumulate_,
+                                                           uint32_t slice_stages_, float* partials_) {
+  // (the fields of MmArgs one by one: built with kernel-argument preload the leading fourteen words are in scalar
+  // registers when the wave starts, instead of one trip to memory away)
+  const MmArgs a{X_, W_, Y_, n_, rows_, cols_, x_stride_, row_bytes_, accumulate_, slice_stages_, partials_};
   constexpr int NT = 64 * WV, TOK = 16 * TM, ABUF = TOK * kMmPitch;
   constexpr int GRAN = TOK * (kMmKStage / 8);           // 16-byte granules (8 halves) per stage
   constexpr int AG = (GRAN + NT - 1) / NT;              // per thread
