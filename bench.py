@@ -31,9 +31,9 @@ HBM_PEAK_GBPS = 8000.0
 
 # HBM bytes per launch of the decode gate/up kernel, from the FETCH_SIZE / WRITE_SIZE counter runs of this workload
 # (KiB per dispatch, scaled by what the same counters read for a 1 GiB copy: x2.000 and x1.000): 42.92 MB + 0.06 MB
-GU_TRAFFIC_BYTES = 43047559
+GU_TRAFFIC_BYTES = 43046740
 # HBM bytes of the launches of the prefill gate/up GEMM together (same counters, same scaling), configs[3]
-PF_GU_TRAFFIC_BYTES = 4327709897
+PF_GU_TRAFFIC_BYTES = 4326887234
 
 
 def cores():
