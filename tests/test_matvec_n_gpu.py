@@ -23,6 +23,9 @@ CASES = [  # (type, rows, cols, groups, n, accumulate): tests/test_quant_matvec_
     (O.Q8_0, 64, 16384, 1, 4, False),         # the widest rows the dot-product kernel takes
     (O.Q6_K, 32, 18432, 1, 8, True), (O.F16, 48, 9216, 1, 9, False),  # wider: MFMA kernel, several K sub-chunks per wave
     (O.IQ2_XXS, 64, 20480, 1, 2, False),      # wider, few tokens: n decode matvecs
+    # two tokens have a kernel instantiation of their own
+    (O.Q8_0, 2304, 5120, 1, 2, True), (O.IQ1_S, 2304, 5120, 1, 2, False), (O.IQ2_XXS, 4096, 2304, 2, 2, False),
+    (O.IQ4_NL, 1024, 4096, 1, 2, True), (O.F16, 300, 1280, 1, 2, False),
 ]
 BASELINE5 = [(O.Q6_K, 1536, 7168), (O.Q5_K, 512, 7168), (O.IQ4_NL, 7168, 4096), (O.BF16, 384, 7168)]
 CASES += [(t, r, c, 1, n, False) for (t, r, c) in BASELINE5 for n in (1, 2, 4, 8, 16)]
