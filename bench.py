@@ -6,7 +6,8 @@
 A "step" is one pass of the hot path over one batch of synthetic input, inputs resident in HBM:
   moe_decode (default; BASELINE configs[2])  one token through a 384-expert MoE layer: 6 routed IQ1_S experts
              (gate/up 2048x7168, down 7168x2048) + 1 shared IQ2_XXS expert, SwiGLU; every step routes to a fresh
-             seeded top-6 set, so expert weights stream from HBM (3.3 GB resident, far above the last-level cache)
+             seeded top-6 set and takes the next of 24 copies of the shared expert, so all weights stream from HBM
+             (3.3 GB + 0.27 GB resident, far above the last-level cache)
   matvec     (BASELINE configs[1])  one single-expert decode matvec, IQ1_S or IQ2_XXS, 4096x7168, weights rotated
              over >= 2 GiB of distinct copies
   q8_0       (BASELINE configs[0])  Q8_0 4096x4096 matvec, same rotation
@@ -29,11 +30,22 @@ METRIC = "MoE decode matvec GB/s (% of HBM peak) + prefill MoE GEMM TFLOP/s (% M
 HBM_PEAK_GBPS = 8000.0
 
 
-# HBM bytes per launch of the decode gate/up kernel, from the FETCH_SIZE / WRITE_SIZE counter runs of this workload
-# (KiB per dispatch, scaled by what the same counters read for a 1 GiB copy: x2.000 and x1.000): 42.92 MB + 0.06 MB
-GU_TRAFFIC_BYTES = 43046740
-# HBM bytes of the launches of the prefill gate/up GEMM together (same counters, same scaling), configs[3]
-PF_GU_TRAFFIC_BYTES = 4326887234
+def profile_traffic(name, line_start):
+    """HBM bytes that profiles/<name> records for the line that starts with `line_start`: the summaries of the
+    FETCH_SIZE / WRITE_SIZE counter runs give such a line's total as "= <MB> MB per launch" or ": <MB> MB per step" (KiB per
+    dispatch scaled by what the same counters read for a 1 GiB copy; the file says how). None when the file or the
+    line is missing, so a stale constant can never stand in for a measurement."""
+    import re
+    try:
+        with open(os.path.join(ROOT, "profiles", name)) as f:
+            for l in f:
+                if l.startswith(line_start):
+                    m = re.search(r"[=:]\s*([0-9.]+) MB per (?:launch|step)", l)
+                    if m:
+                        return int(round(float(m.group(1)) * 1e6))
+    except OSError:
+        pass
+    return None
 
 
 def cores():
@@ -73,30 +85,38 @@ def event_ms_per_launch(torch, launch, n):
 
 
 def graph_ms_per_launch(torch, launch, n):
-    """Average duration of one launch when n launches of the same kernel run back to back: the n launches are captured
-    in one HIP graph (no host in the loop) and one replay is timed with a HIP event pair on the replay's stream."""
+    """Average duration of one launch when launches of the same kernel run back to back: n launches are captured in one
+    HIP graph (no host in the loop); after 20 ms of untimed replays, three regions of back-to-back replays, each inside
+    one HIP event pair on the replay's stream and at least 10 ms long, are timed; the median region counts."""
     g = torch.cuda.CUDAGraph()
     torch.cuda.synchronize()
     with torch.cuda.graph(g):
         for i in range(n):
             launch(i)
-    g.replay()
-    torch.cuda.synchronize()
-    best = None
-    for _ in range(3):
+
+    def region(replays):
         a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         a.record()
-        g.replay()
+        for _ in range(replays):
+            g.replay()
         b.record()
         torch.cuda.synchronize()
-        t = a.elapsed_time(b) / n
-        best = t if best is None else min(best, t)
-    return float(best)
+        return a.elapsed_time(b)
+
+    done, spent = 0, 0.0
+    while spent < 20.0:
+        spent += region(2)
+        done += 2
+    R = int(min(20000, max(1, -(-10.0 // max(spent / done, 1e-4)))))
+    return float(np.median([region(R) / (R * n) for _ in range(3)]))
 
 
 def timed_graph(torch, enqueue_steps, steps, warmup):
-    """Captures `steps` back-to-back steps in one HIP graph (the loop is launch-bound from Python otherwise), replays
-    it `warmup` times untimed, then times five replays one by one and returns (the fastest, all five) in ms per step."""
+    """Captures `steps` back-to-back steps in one HIP graph (from Python the loop is launch-bound otherwise) and times
+    replays of it with HIP events on the replay's stream: after at least `warmup` steps and 50 ms of untimed replays,
+    five regions of R back-to-back replays each, every region inside ONE event pair and at least 10 ms long, so that
+    neither the host's graph-launch latency nor the clock ramp of an idle device sits in a region. Returns (median
+    region in ms per step, all five, R)."""
     g = torch.cuda.CUDAGraph()
     side = torch.cuda.Stream()
     side.wait_stream(torch.cuda.current_stream())
@@ -106,17 +126,24 @@ def timed_graph(torch, enqueue_steps, steps, warmup):
     torch.cuda.synchronize()
     with torch.cuda.graph(g):
         enqueue_steps(steps)
-    reps = max(1, (warmup + steps - 1) // steps) if warmup > 0 else 0
-    for _ in range(reps):
-        g.replay()
-    torch.cuda.synchronize()
-    reps_ms = []
-    for _ in range(5):  # each timed region is one replay = exactly `steps` steps between device synchronisations
-        t0 = time.perf_counter()
-        g.replay()
+
+    def region(replays):
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for _ in range(replays):
+            g.replay()
+        b.record()
         torch.cuda.synchronize()
-        reps_ms.append((time.perf_counter() - t0) * 1e3 / steps)
-    return min(reps_ms), reps_ms
+        return a.elapsed_time(b)
+
+    done, spent, reps = 0, 0.0, max(1, -(-warmup // steps))
+    while done * steps < warmup or spent < 50.0:
+        spent += region(reps)
+        done += reps
+    per_replay = max(spent / done, 1e-4)
+    R = int(min(20000, max(1, -(-10.0 // per_replay))))
+    regions = [region(R) / (R * steps) for _ in range(5)]
+    return float(np.median(regions)), regions, R
 
 
 # ------------------------------------------------------------------------------------------------ MoE decode layer
@@ -132,7 +159,11 @@ def bench_moe_decode(torch, args):
     sgu_b, sdn_b = q.row_bytes(ts, DIM) * INTER, q.row_bytes(ts, INTER) * DIM
     per_exp = 2 * gu_b + dn_b
     arena = gen_blocks(torch, tr, NE * per_exp // 50, 0.01, 1, dev)
-    shared = gen_blocks(torch, ts, (2 * sgu_b + sdn_b) // 66, 0.01, 2, dev)
+    # the shared expert in N_SHARED distinct copies, one per step in turn: like the routed experts it then streams from
+    # HBM (a 40-layer token loop never finds a layer's shared expert in the 256 MB last-level cache either)
+    N_SHARED = 24
+    sh_b = 2 * sgu_b + sdn_b
+    shared = gen_blocks(torch, ts, N_SHARED * sh_b // 66, 0.01, 2, dev)
     base = arena.data_ptr()
     n_sets = max(args.steps, 64)
     # seeded fp32 router: logits ~ N(0,1) over 384 experts, top-6, weights = softmax over the selected logits
@@ -160,7 +191,8 @@ def bench_moe_decode(torch, args):
         a = q.MoeDecodeArgs()
         a.t_gate_up = a.t_down = tr
         a.t_shared, a.n_routed, a.has_shared, a.dim, a.inter = ts, TOPK, True, DIM, INTER
-        a.shared = q.ExpertSlot(sh.sub(0, sgu_b), sh.sub(sgu_b, sgu_b), sh.sub(2 * sgu_b, sdn_b))
+        so = (i % N_SHARED) * sh_b
+        a.shared = q.ExpertSlot(sh.sub(so, sgu_b), sh.sub(so + sgu_b, sgu_b), sh.sub(so + 2 * sgu_b, sdn_b))
         a.weights = q.Buffer.of(wts_d).sub(i * 24, 24)
         a.x, a.y, a.scratch = q.Buffer.of(x), q.Buffer.of(y), q.Buffer.of(scratch)
         calls.append((a.c(), q.Buffer.of(tables_d).sub(i * 144, 144).c()))
@@ -175,7 +207,7 @@ def bench_moe_decode(torch, args):
         for i in range(n):
             run_part(i, q.MoePart.All)
 
-    ms_step, ms_reps = timed_graph(torch, enqueue, args.steps, args.warmup)
+    ms_step, ms_reps, replays = timed_graph(torch, enqueue, args.steps, args.warmup)
     w_bytes = TOPK * per_exp + 2 * sgu_b + sdn_b
     h_bytes = (TOPK + 1) * INTER * 4
     step_bytes = w_bytes + DIM * 4 + 2 * h_bytes + 2 * DIM * 4
@@ -201,7 +233,7 @@ def bench_moe_decode(torch, args):
     for k in range(TOPK):
         o = int(ids[i0, k]) * per_exp
         G.append(host(arena[o:o + gu_b])); U.append(host(arena[o + gu_b:o + 2 * gu_b])); D.append(host(arena[o + 2 * gu_b:o + per_exp]))
-    G.append(host(shared[:sgu_b])); U.append(host(shared[sgu_b:2 * sgu_b])); D.append(host(shared[2 * sgu_b:]))
+    G.append(host(shared[:sgu_b])); U.append(host(shared[sgu_b:2 * sgu_b])); D.append(host(shared[2 * sgu_b:sh_b]))
     xh = host(x)
     t0 = time.perf_counter()
     n_cpu = 0
@@ -233,13 +265,14 @@ def bench_moe_decode(torch, args):
                   "layer_pct_of_1GiB_stream_read": 100 * value / s_big}
 
     return {
-        "value": value, "ms_per_step": ms_step, "ms_per_step_of_each_replay": ms_reps,
+        "value": value, "ms_per_step": ms_step, "ms_per_step_of_each_region": ms_reps, "replays_timed": replays,
+        "timing": "median of five regions, each %d back-to-back replays of a %d-step HIP graph inside one HIP event pair" % (replays, args.steps),
         "dtype": "int8 IQ1_S codebook x 16-bit block-fixed-point activations (i32, gate/up), f16 x f16 (IQ2_XXS shared expert, down); f32 accumulate",
         "config": {"workload": "BASELINE configs[2]: batch-1 MoE decode layer, 384 experts IQ1_S 7168x2048 (3.3 GB resident), "
                                "top-6 of a seeded softmax router + 1 shared IQ2_XXS expert, SwiGLU; fresh top-6 per step",
                    "bytes_per_step": step_bytes, "experts": NE, "top_k": TOPK, "dim": DIM, "inter": INTER},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBPS,
-                     "traffic": GU_TRAFFIC_BYTES, "traffic_source": "profiles/moe_hbm_traffic_fetch_write.txt", "kernel": "moe_gu_kernel<DecIQ1SQ,DecIQ2XXS>", "bytes_per_launch": gu_bytes,
+                     "traffic": profile_traffic("moe_hbm_traffic_fetch_write.txt", "moe_gu_kernel<"), "traffic_source": "profiles/moe_hbm_traffic_fetch_write.txt", "kernel": "moe_gu_kernel<DecIQ1SQ,DecIQ2XXS>", "bytes_per_launch": gu_bytes,
                      "avg_launch_us": gu_graph * 1e3,
                      "timing": "HIP event pair around one graph replay of %d back-to-back launches of this kernel" % n_ev,
                      "eager_event_pair_us": {"mean": gu_mean * 1e3, "median": gu_med * 1e3, "min": gu_min * 1e3},
@@ -276,7 +309,7 @@ def bench_matvec(torch, args, t, rows, cols, d_sigma, label):
         if rc != 0:
             raise RuntimeError(L.msq_last_error().decode())
 
-    ms_step, ms_reps = timed_graph(torch, lambda n: [launch(i) for i in range(n)], args.steps, args.warmup)
+    ms_step, ms_reps, replays = timed_graph(torch, lambda n: [launch(i) for i in range(n)], args.steps, args.warmup)
     step_bytes = mat_b + 4 * cols + 4 * rows
     value = step_bytes / (ms_step * 1e-3) / 1e9
     e_mean, e_med, e_min = event_ms_per_launch(torch, launch, min(max(args.steps, 50), 400))
@@ -302,7 +335,7 @@ def bench_matvec(torch, args, t, rows, cols, d_sigma, label):
             break
     s_read = stream_read_GBps(torch, step_bytes, arena)
     return {
-        "value": value, "ms_per_step": ms_step, "ms_per_step_of_each_replay": ms_reps,
+        "value": value, "ms_per_step": ms_step, "ms_per_step_of_each_region": ms_reps, "replays_timed": replays,
         "dtype": "f32" if t == q.QType.Q8_0 else "f16 activations, f32 accumulate",
         "config": {"workload": label, "bytes_per_step": step_bytes, "rows": rows, "cols": cols, "weight_copies": copies},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBPS,
@@ -375,14 +408,17 @@ def bench_moe_prefill(torch, steps, warmup, with_cpu=True):
         if rc != 0:
             raise RuntimeError(L.msq_last_error().decode())
 
-    for _ in range(max(1, warmup)):
+    for _ in range(max(3, warmup)):
         call()
     torch.cuda.synchronize()
-    t0 = time.perf_counter()
+    steps = max(steps, 4)  # a timed region of at least 10 ms
+    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    ev0.record()
     for _ in range(steps):
         call()
+    ev1.record()
     torch.cuda.synchronize()
-    ms_step = (time.perf_counter() - t0) * 1e3 / steps
+    ms_step = ev0.elapsed_time(ev1) / steps
     flops = 2.0 * 3 * DIM * INTER * total
     value = flops / (ms_step * 1e-3) / 1e12
     # dominant kernel: the routed gate/up GEMM (two thirds of the FLOPs), timed alone through the phase skip mask
@@ -413,7 +449,7 @@ def bench_moe_prefill(torch, steps, warmup, with_cpu=True):
                    "tokens_per_expert_median": float(np.median(counts[used])), "flops_per_step": flops,
                    "weight_bytes_touched": int(len(used)) * per_exp},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": achieved / MFMA_PEAK_TFLOPS,
-                     "traffic": PF_GU_TRAFFIC_BYTES, "traffic_source": "profiles/moe_prefill_hbm_traffic_fetch_write.txt",
+                     "traffic": profile_traffic("moe_prefill_hbm_traffic_fetch_write.txt", "gate/up ("), "traffic_source": "profiles/moe_prefill_hbm_traffic_fetch_write.txt",
                      "kernel": "moe_pf_block_kernel<BlkIQ2XXS, gate/up> (two launches: blocks of 49..112 entries of the popular experts; items of one to three token tiles)",
                      "gate_up_time_split": split,
                      "flops_per_launch": gu_flops,
@@ -503,15 +539,17 @@ def bench_stream(torch, args):
 
 
 def bench_issue_probe(torch, args):
-    """Instruction-issue probes (msq_issue_probe): ns per instruction group and SIMD for vector ops, matrix-core ops and
+    """Instruction-issue probes (libmsq_probe.so, a measurement tool outside the library): ns per instruction group and SIMD for vector ops, matrix-core ops and
     LDS reads, alone and interleaved, at 1, 2 and 4 waves per SIMD (one workgroup per CU) and 8 (two workgroups)."""
-    from macseek_amd import _lib
-    from macseek_amd import quant as q
-    L = _lib.load()
+    from macseek_amd import build as B
+    if not os.path.exists(B.PROBE_OUT):
+        raise RuntimeError("bench.py: %s is missing; build it with `python -m macseek_amd.build`" % B.PROBE_OUT)
+    P = C.CDLL(B.PROBE_OUT)  # the probe is no part of libmsq.so
+    P.msq_probe_issue.restype = C.c_int
+    P.msq_probe_issue.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_size_t]
     dev = torch.device("cuda:0")
     cus = torch.cuda.get_device_properties(0).multi_processor_count
     sink = torch.zeros(4 * cus * 4, dtype=torch.uint8, device=dev)
-    sb = q.Buffer.of(sink).c()
     VALU, MFMA16, MFMA4, MFMA8, LDS, VINT, VPK, VFMA = 1, 2, 4, 8, 16, 32, 64, 128
     mixes = [("valu32", VALU), ("mfma16_f16_x8", MFMA16), ("mfma_fp4_fp6_x8", MFMA4), ("mfma_fp8_x8", MFMA8), ("lds_b32_x16", LDS),
              ("valu32+mfma16_f16_x8", VALU | MFMA16), ("valu32+mfma_fp4_fp6_x8", VALU | MFMA4), ("valu32+lds_b32_x16", VALU | LDS),
@@ -523,9 +561,10 @@ def bench_issue_probe(torch, args):
         row = {"waves_per_simd": wps}
         for name, mask in mixes:
             def launch(i):
-                rc = L.msq_issue_probe(C.c_void_p(torch.cuda.current_stream().cuda_stream), mask, grid, block, iters, C.byref(sb))
+                rc = P.msq_probe_issue(C.c_void_p(torch.cuda.current_stream().cuda_stream), mask, grid, block, iters,
+                                       C.c_void_p(sink.data_ptr()), sink.numel())
                 if rc != 0:
-                    raise RuntimeError(L.msq_last_error().decode())
+                    raise RuntimeError("msq_probe_issue failed: %d" % rc)
             ms = graph_ms_per_launch(torch, launch, 3)
             # one iteration of one wave = one group set; a SIMD runs wps waves: ns per group set and SIMD
             row[name] = round(ms * 1e6 / iters / wps, 2)
@@ -618,6 +657,74 @@ def bench_matvec_n(torch, args):
                          "traffic": None, "kernel": "mv_tok_kernel<DecQ6K, 1, 8>", "bytes_per_launch": head["bytes"],
                          "avg_launch_us": head["us_per_launch"], "timing": "HIP event pair around one graph replay of 200 back-to-back launches"},
             "cpu_baseline": cpu, "pct_of_hbm_peak": 100 * head["GBps"] / HBM_PEAK_GBPS}
+
+
+def bench_table(torch, args):
+    """The reference's per-matrix table (bench/qmatvec.mm:93-157, docs/modules/quant.md:160-187) in one run: every real
+    projection shape of the reference plus BASELINE's configs[0], [1] and [4] shapes, one msq_matvec per step, weights
+    rotated over >= 512 MiB of distinct copies so every launch streams from HBM. Per row: weight MB, us per launch,
+    GB/s of algorithmic bytes (W + 4 cols + 4 rows), the fraction of the 8 TB/s roofline and of what a kernel that only
+    reads (msq_bw_probe, 1 GiB, same run) gets on this device. value = the Q8_0 4096x4096 row (configs[0])."""
+    from macseek_amd import _lib, quant as q
+    L = _lib.load()
+    dev = torch.device("cuda:0")
+    T = q.QType
+    shapes = [
+        (T.Q8_0, 4096, 4096, 1, "BASELINE configs[0]"),
+        (T.IQ1_S, 4096, 7168, 1, "configs[1] gate/up"), (T.IQ1_S, 7168, 4096, 1, "configs[1] down"),
+        (T.IQ2_XXS, 4096, 7168, 1, "configs[1] gate/up"), (T.IQ2_XXS, 7168, 4096, 1, "configs[1] down"),
+        (T.Q6_K, 1536, 7168, 1, "configs[4] Q"), (T.Q5_K, 512, 7168, 1, "configs[4] KV"),
+        (T.IQ4_NL, 7168, 4096, 1, "configs[4] output"), (T.BF16, 384, 7168, 1, "configs[4] router"),
+        # the reference's own table (bench/qmatvec.mm:93-110)
+        (T.Q6_K, 1280, 5120, 1, "attn_q_a"), (T.Q5_K, 1280, 5120, 1, "attn_q_a"),
+        (T.Q6_K, 32768, 1280, 1, "attn_q_b"), (T.Q5_K, 32768, 1280, 1, "attn_q_b"),
+        (T.Q6_K, 512, 5120, 1, "attn_kv"), (T.Q6_K, 8192, 4096, 8, "attn_output_a"),
+        (T.Q6_K, 5120, 8192, 1, "attn_output_b"), (T.Q5_K, 5120, 8192, 1, "attn_output_b"),
+        (T.IQ1_S, 2304, 5120, 1, "exp gate/up"), (T.IQ1_S, 5120, 2304, 1, "exp down"),
+        (T.IQ2_XXS, 2304, 5120, 1, "exp gate/up"), (T.IQ2_XXS, 5120, 2304, 1, "exp down"),
+        (T.Q6_K, 2304, 5120, 1, "shexp gate/up"), (T.Q6_K, 5120, 2304, 1, "shexp down"),
+        (T.Q8_0, 2304, 5120, 1, "shexp gate/up"), (T.Q8_0, 5120, 2304, 1, "shexp down"),
+        (T.Q6_K, 129280, 5120, 1, "output head"), (T.Q6_K, 25600, 6144, 1, "engram_kv"),
+        (T.F32, 384, 5120, 1, "router"), (T.F32, 24, 20480, 1, "hc_fn"),
+        (T.BF16, 512, 5120, 1, "compressor_kv"), (T.BF16, 4096, 1280, 1, "indexer q_b"),
+        (T.F16, 5120, 5120, 1, "f16 synthetic"),
+        (T.IQ1_S, 32768, 5120, 1, "big synthetic"), (T.IQ2_XXS, 32768, 5120, 1, "big synthetic"),
+    ]
+    pool = torch.randint(0, 256, (1 << 30,), dtype=torch.uint8, device=dev)  # raw bytes: timing only (as the reference's table)
+    bw = stream_read_GBps(torch, 1 << 30, pool)
+    rows_out = []
+    for t, rows, cols, groups, what in shapes:
+        nb = q.row_bytes(t, cols) * rows
+        pitch = (nb + 255) // 256 * 256
+        copies = int(min(max(2, -(-(512 << 20) // pitch)), (1 << 30) // pitch, 256))
+        x = torch.randn(cols * groups, device=dev)
+        y = torch.zeros(rows, device=dev)
+        Wb = [q.Buffer.of(pool).sub(i * pitch, nb).c() for i in range(copies)]
+        xb, yb = q.Buffer.of(x).c(), q.Buffer.of(y).c()
+
+        def launch(i):
+            rc = L.msq_matvec(C.c_void_p(torch.cuda.current_stream().cuda_stream), int(t), C.byref(Wb[i % copies]), rows, cols,
+                              C.byref(xb), C.byref(yb), 0, groups, None)
+            if rc != 0:
+                raise RuntimeError(L.msq_last_error().decode())
+        ms = graph_ms_per_launch(torch, launch, max(copies, 16))
+        byt = nb + 4 * cols * groups + 4 * rows
+        gbps = byt / (ms * 1e-3) / 1e9
+        rows_out.append({"type": q.type_name(t), "tensor": what, "shape": "%d->%d%s" % (cols, rows, " g%d" % groups if groups > 1 else ""),
+                         "MB": round(nb / 1e6, 2), "us": round(ms * 1e3, 2), "GBps": round(gbps, 1),
+                         "frac_of_8TBps": round(gbps / HBM_PEAK_GBPS, 4), "pct_of_stream_read": round(100 * gbps / bw, 1)})
+    head = rows_out[0]
+    print("%-8s %-20s %-16s %9s %8s %8s %7s %9s" % ("type", "tensor", "shape", "MB", "us", "GB/s", "%8TB/s", "%stream"), file=sys.stderr)
+    for r in rows_out:
+        print("%-8s %-20s %-16s %9.2f %8.2f %8.1f %7.1f %9.1f" % (r["type"], r["tensor"], r["shape"], r["MB"], r["us"], r["GBps"],
+                                                                   100 * r["frac_of_8TBps"], r["pct_of_stream_read"]), file=sys.stderr)
+    return {"value": head["GBps"], "ms_per_step": head["us"] * 1e-3, "dtype": "f32 activations (Q8_0, dense) / f16-staged activations (block formats), f32 accumulate",
+            "config": {"workload": "decode matvec table: the reference's projection shapes + BASELINE configs[0], [1], [4]; one step = one msq_matvec of "
+                                   "the Q8_0 4096x4096 row", "stream_read_GBps_1GiB": bw, "rows": rows_out},
+            "roofline": {"bound": "hbm", "achieved": head["GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": head["GBps"] / HBM_PEAK_GBPS,
+                         "traffic": None, "kernel": "decode matvec (mv_tok_kernel, mv_kernel or mv_ring_kernel by shape)", "avg_launch_us": head["us"],
+                         "timing": "HIP event pair around back-to-back replays of a graph of >= 16 launches, >= 10 ms per region"},
+            "cpu_baseline": None, "pct_of_hbm_peak": 100 * head["GBps"] / HBM_PEAK_GBPS}
 
 
 def bench_router(torch, args):
@@ -743,7 +850,7 @@ def main():
     ap.add_argument("--steps", type=int, default=500)
     ap.add_argument("--warmup", type=int, default=100)
     ap.add_argument("--workload", default="moe_decode",
-                    choices=["moe_decode", "moe_prefill", "matvec_iq1s", "matvec_iq2xxs", "q8_0", "matvec_n", "router", "matmul", "stream", "copy_calibration", "issue_probe"])
+                    choices=["moe_decode", "moe_prefill", "matvec_iq1s", "matvec_iq2xxs", "q8_0", "matvec_n", "router", "matmul", "stream", "copy_calibration", "issue_probe", "table"])
     ap.add_argument("--one-stream", action="store_true",
                     help="profiling runs: msq_moe_prefill keeps its launches on one stream (MSQ_MOEP_ONE_STREAM=1), so that "
                          "per-kernel durations and counters are not those of two kernels sharing the device")
@@ -790,6 +897,8 @@ def main():
         r = bench_issue_probe(torch, args)
     elif args.workload == "router":
         r = bench_router(torch, args)
+    elif args.workload == "table":
+        r = bench_table(torch, args)
     elif args.workload == "matvec_n":
         r = bench_matvec_n(torch, args)
     elif args.workload == "matvec_iq1s":
@@ -802,7 +911,7 @@ def main():
            "ms_per_step": r["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
            "dtype": r["dtype"], "data": "synthetic", "config": r["config"], "roofline": r["roofline"],
            "cpu_baseline": r["cpu_baseline"], "pct_of_hbm_peak": r["pct_of_hbm_peak"]}
-    for k in ("ms_per_step_of_each_replay", "stream_read_reference"):
+    for k in ("ms_per_step_of_each_region", "replays_timed", "timing", "stream_read_reference"):
         if k in r:
             out[k] = r[k]
     if args.workload == "moe_decode" and not args.gpu_only:

@@ -139,14 +139,6 @@ int msq_dequant(void* stream, int qtype, const MsqBuffer* W, int64_t n_elems, co
  * used by bench/qmatvec.mm:18-31). */
 int msq_bw_probe(void* stream, const MsqBuffer* src, size_t bytes, const MsqBuffer* sink);
 
-/* Instruction-issue probe (no reference counterpart; the reference prices its kernels against a bandwidth probe only):
- * `grid` workgroups of `block` threads each run `iters` iterations of a fixed instruction group per wave. `mask` ORs
- * the groups: 1 = 32 vector ops, 2 = 8 fp16 16x16x32 matrix ops, 4 = 8 block-scaled fp4 x fp6 16x16x128 matrix ops,
- * 8 = 8 fp8 16x16x128 matrix ops, 16 = 16 random 32-bit LDS reads, 32 = 32 integer vector ops, 64 = 32 packed-fp16
- * multiplies, 128 = 32 fp32 fused multiply-adds; supported mixes: 1, 2, 4, 8, 16, 32, 64, 128, 1|2, 1|4, 1|16, 1|4|16,
- * 32|2, 64|2, 128|2. `sink` holds >= 4 * grid bytes. The benchmark turns the timings into ns per issue slot. */
-int msq_issue_probe(void* stream, int mask, int grid, int block, int iters, const MsqBuffer* sink);
-
 /* ---------------------------------------------------------------------------------------------- MoE, one token */
 
 /* reference: kMaxRouted / kExpertDim / kExpertInter (quant.hpp:49). The reference hard-codes the expert shape; here
@@ -254,7 +246,8 @@ size_t msq_moe_prefill_scratch_bytes(int total_entries, int n_tokens, int n_exp,
 
 /* reference: ms::q::encode_moe_prefill (quant.hpp:118, quant.mm:433-612). Enqueues gather, grouped gate/up GEMM +
  * SwiGLU, grouped down GEMM and the ordered reduction into Y. Activations and H are staged as fp16 and weights enter
- * the matrix instructions as fp16 (the whole weight rounded once), as in the reference's tiles. The call only enqueues
+ * the matrix instructions as fp16 like the reference's tiles (IQ1_S / IQ2_XXS: the sub-block scale is rounded to fp16 and
+ * its product with the grid value is rounded again, where the reference rounds the fp32 product once). The call only enqueues
  * (no host copy, no wait, no allocation) and can be captured in a HIP graph. Two of its launches are independent and
  * run side by side: one is forked onto a stream that the library owns (one per device, created by msq_init() or by the
  * first call outside a capture) and joined back before the call's later launches, all through events, so the caller

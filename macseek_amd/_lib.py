@@ -76,7 +76,6 @@ SIGNATURES = {
     "msq_matmul": (C.c_int, [C.c_void_p, C.c_int, _BP, C.c_int, C.c_int, _BP, _BP, C.c_int, C.c_int]),
     "msq_dequant": (C.c_int, [C.c_void_p, C.c_int, _BP, C.c_int64, _BP]),
     "msq_bw_probe": (C.c_int, [C.c_void_p, _BP, C.c_size_t, _BP]),
-    "msq_issue_probe": (C.c_int, [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, _BP]),
     "msq_moe_decode_scratch_bytes": (C.c_size_t, [C.c_int]),
     "msq_moe_decode": (C.c_int, [C.c_void_p, C.POINTER(MsqMoeDecodeArgs)]),
     "msq_moe_decode_table": (C.c_int, [C.c_void_p, C.POINTER(MsqMoeDecodeArgs), _BP]),

@@ -237,7 +237,9 @@ int msq_f32_to_f16(void* stream, const MsqBuffer* X, const MsqBuffer* X16, size_
 
 int msq_matmul_h(void* stream, int t, const MsqBuffer* W, int rows, int cols, const MsqBuffer* X16, const MsqBuffer* Y, int n,
                  int accumulate, int x_stride) {
-  if (!mm_type_ok(t) || rows < 1 || cols < 1 || cols % 128 || n < 1 || (x_stride && x_stride < cols)) return unsupported("matmul", t, rows, cols);
+  // (a row is whole blocks: for the 256-weight formats a multiple of 128 columns is not enough)
+  if (!mm_type_ok(t) || rows < 1 || cols < 1 || cols % 128 || cols % msq_type_block_elems(t) || n < 1 || (x_stride && x_stride < cols))
+    return unsupported("matmul", t, rows, cols);
   const int xs = x_stride ? x_stride : cols;
   if (!buf_ok(W, msq_type_row_bytes(t, cols) * (size_t)rows) || !buf_ok(X16, ((size_t)(n - 1) * xs + cols) * 2) ||
       !buf_ok(Y, (size_t)n * rows * 4) || ((uintptr_t)bptr(X16) & 1) || ((uintptr_t)bptr(Y) & 3))
@@ -255,7 +257,7 @@ int msq_matmul_h(void* stream, int t, const MsqBuffer* W, int rows, int cols, co
 
 int msq_matmul(void* stream, int t, const MsqBuffer* W, int rows, int cols, const MsqBuffer* X, const MsqBuffer* Y, int n,
                int accumulate) {
-  if (!mm_type_ok(t) || rows < 1 || cols < 1 || cols % 128 || n < 1) return unsupported("matmul", t, rows, cols);
+  if (!mm_type_ok(t) || rows < 1 || cols < 1 || cols % 128 || cols % msq_type_block_elems(t) || n < 1) return unsupported("matmul", t, rows, cols);
   if (!buf_ok(W, msq_type_row_bytes(t, cols) * (size_t)rows) || !buf_ok(X, (size_t)n * cols * 4) || !buf_ok(Y, (size_t)n * rows * 4) ||
       ((uintptr_t)bptr(X) & 15) || ((uintptr_t)bptr(Y) & 3))
     return fail(MSQ_ERR_ARGUMENT, "macseek quant: matmul: buffer missing, too small or misaligned (type %s rows %d cols %d n %d)",

@@ -217,7 +217,10 @@ struct FragDense16 {
 
 // ================================================================================================ block fragments
 // For the 256-weight codebook formats the large-token GEMM uses a second decomposition: the payload is the whole weight,
-// scale included, rounded to fp16 (what the reference's prefill kernels feed their matrix units), so a wave accumulates
+// scale included, as fp16 (the reference's prefill kernels feed their matrix units dequantized fp16 tiles too; they
+// round d * scale * grid once, src/kernels/quant_moe_prefill.metal:137-167, where finish() below rounds twice: the
+// sub-block scale to fp16, then its product with the grid value, 2^-11 relative per weight at worst instead of
+// 2^-12; the scale in fp32 would cost a second multiply per register), so a wave accumulates
 // all of K in the matrix cores without touching the accumulators in between. Lane (row n, chunk q) owns the sub-blocks 2 q and 2 q + 1 of its row's block
 // (16 contiguous bytes of IQ2_XXS), so no lane loads a byte twice; step j (0..7) of a block therefore covers, for chunk
 // q, the 8 columns col_of(q, j) .. + 7 of the block, and the activation operand is read with the same mapping.
@@ -283,8 +286,8 @@ struct BlkIQ2XXS {
     const uint8_t* t8 = (const uint8_t*)tbl;
     return {*(const uint4*)(t8 + GRID_AT + ((g8 & 0xFF00u) | cg)), *(const uint4*)(t8 + ((s8 & 0x7F00u) | cg))};
   }
-  // weight = fp16(d (2 s + 1) / 8) * (+-grid), rounded to fp16 like the reference's dequantized tiles
-  // (src/kernels/quant_moe_prefill.metal:153-167): the whole scale rides in the payload
+  // weight = fp16(fp16(d (2 s + 1) / 8) * (+-grid)): the whole scale rides in the payload, rounded to fp16 before the
+  // multiply (the reference's tile rounds the fp32 product once, src/kernels/quant_moe_prefill.metal:153-167)
   __device__ static void finish(const Raw& r, int j, const Look& k, uint32_t (&h)[4]) {
     const uint32_t a1 = r.w[2 * (j >> 2) + 1];
     const float m = (half_bits_to_float(r.d) * 0.125f) * (float)(((a1 >> 27) & 0x1Eu) | 1u);
@@ -313,8 +316,8 @@ struct BlkIQ1S {
     const int l = j & 3;
     return {((const uint4*)tbl)[((qs >> (8 * l)) & 0xFFu) | (((qh >> (3 * l)) & 7u) << 8)]};
   }
-  // weight = fp16(d (2 s + 1)) * (grid + delta), rounded to fp16 like the reference's dequantized tiles
-  // (src/kernels/quant_moe_prefill.metal:137-147)
+  // weight = fp16(fp16(d (2 s + 1)) * (grid + delta)): scale rounded to fp16, product rounded again (the reference's
+  // tile rounds the fp32 product once, src/kernels/quant_moe_prefill.metal:137-147)
   __device__ static void finish(const Raw& r, int j, const Look& k, uint32_t (&h)[4]) {
     const uint32_t qh = (j >> 2) ? r.qh >> 16 : r.qh & 0xFFFFu;
     const uint32_t d2 = (qh & 0x8000u) ? 0xB000B000u : 0x30003000u;          // -+ 1/8 in both halves

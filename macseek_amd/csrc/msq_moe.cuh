@@ -19,19 +19,6 @@
 
 namespace msq {
 
-#ifdef MSQ_EXP_NOLOOP  // experiment builds: the row loops never run, what remains is the launch's fixed cost
-#define MSQ_EXP_LOOP_COND && a_never
-#else
-#define MSQ_EXP_LOOP_COND
-#endif
-
-#ifdef MSQ_EXP_TIMELINE  // experiment builds: wall-clock stamps (100 MHz) per workgroup, wave and point
-__device__ uint64_t g_timeline[512 * 16 * 8];
-#define MSQ_TL(k) do { if ((threadIdx.x & 63u) == 0 && blockIdx.x < 512u) g_timeline[(blockIdx.x * 16u + (threadIdx.x >> 6)) * 8u + (k)] = wall_clock64(); } while (0)
-#else
-#define MSQ_TL(k) do {} while (0)
-#endif
-
 constexpr int kMaxRouted = 6;
 constexpr int kMoeChunkRows = 128;  // rows a workgroup finishes between two synchronisations
 // The down kernel multiplies h by this power of two before it is rounded to fp16 pairs and divides the row sums by it:
@@ -301,7 +288,6 @@ __device__ __forceinline__ void moe_gu_run_ring(const MoeArgs& a, const uint64_t
       pv++; pr++;
       if (!shared && pr == a.inter && pv < w1) { pr = 0; pe++; set_expert(); }
     };
-    if (first) MSQ_TL(1);
     // Half of the ring is requested before the tables and activations, the other half behind them: loads return in
     // order, so with the whole ring ahead the prologue's small reads wait for four row pairs, and with none ahead the
     // first rows start a memory trip late (gate/up of the one-token layer: 16.9 us with 4 or 0 pairs first, 16.6 / 16.4
@@ -309,11 +295,9 @@ __device__ __forceinline__ void moe_gu_run_ring(const MoeArgs& a, const uint64_t
 #pragma unroll
     for (int s = 0; s < NR / 2; s++) fetch(s);
     if (first) {  // tables and activations arrive while the first weight rows are in flight
-      MSQ_TL(2);
       if constexpr (requires { D::QUANT_X; }) {
         if (a.stage_x) {
           D::finish_tables(tbl, tr, tid, blockDim.x);
-          MSQ_TL(3);
           stage_xq<2>(smem + a.xs_off, a.x, a.dim, tid, blockDim.x, &xb);
           __syncthreads();
           xr = D::load_x(XQLds{smem + a.xs_off}, unit);
@@ -336,7 +320,6 @@ __device__ __forceinline__ void moe_gu_run_ring(const MoeArgs& a, const uint64_t
       }
       if (!valid) xr = typename D::X{};
       first = false;
-      MSQ_TL(4);
     }
 #pragma unroll
     for (int s = NR / 2; s < NR; s++) fetch(s);
@@ -351,9 +334,8 @@ __device__ __forceinline__ void moe_gu_run_ring(const MoeArgs& a, const uint64_t
       pg_[0] = D::pre(rg[0], tbl); pu_[0] = D::pre(ru[0], tbl);
       pg_[1] = D::pre(rg[1], tbl); pu_[1] = D::pre(ru[1], tbl);
       D::lookup(rg[0], pg_[0], tbl, lanec, lg[0]); D::lookup(ru[0], pu_[0], tbl, lanec, lu[0]);
-      [[maybe_unused]] const bool a_never = a.dim == 1u;
       static_assert(NS == 1 && NR % 2 == 0 && NR >= 4, "two row pairs per fold, table reads two pairs ahead");
-      for (uint32_t r0 = w0; r0 < w1 MSQ_EXP_LOOP_COND; r0 += NR) {
+      for (uint32_t r0 = w0; r0 < w1; r0 += NR) {
 #pragma unroll
         for (int half = 0; half < NR / 2; half++) {
           float acc[4];  // value 2 j + m: row pair j of this half, m = 0 gate, 1 up
@@ -381,8 +363,7 @@ __device__ __forceinline__ void moe_gu_run_ring(const MoeArgs& a, const uint64_t
     } else {
     typename D::Look lk[2];  // stage t of a row pair uses lk[t & 1]; 2 NS stages per row pair keep the parity fixed
     if (w0 < w1) lk[0] = D::lookup(rg[0], 0, tbl);
-    [[maybe_unused]] const bool a_never = a.dim == 1u;
-    for (uint32_t r0 = w0; r0 < w1 MSQ_EXP_LOOP_COND; r0 += NR) {
+    for (uint32_t r0 = w0; r0 < w1; r0 += NR) {
 #pragma unroll
       for (int half = 0; half < 2; half++) {
         float acc[NR];  // value 2 j + m: row pair j of this half, m = 0 gate, 1 up
@@ -417,9 +398,7 @@ __device__ __forceinline__ void moe_gu_run_ring(const MoeArgs& a, const uint64_t
       }
     }
     }
-    MSQ_TL(5);
     __syncthreads();
-    MSQ_TL(6);
     // thread q sums the partials of (row q / 2, matrix q % 2); gate and up then meet in the even lane
     for (uint32_t q0 = 0; q0 < 2 * n; q0 += blockDim.x) {
       const uint32_t q = q0 + tid;
@@ -434,7 +413,6 @@ __device__ __forceinline__ void moe_gu_run_ring(const MoeArgs& a, const uint64_t
       }
     }
     __syncthreads();
-    MSQ_TL(7);
   }
 }
 
@@ -454,7 +432,6 @@ __global__ __launch_bounds__(1024) void moe_gu_kernel(const uint64_t* table, con
   constexpr int TBL = DR::LDS_WORDS > DS::LDS_WORDS ? DR::LDS_WORDS : DS::LDS_WORDS;
   __shared__ __attribute__((aligned(16))) uint32_t tbl[TBL > 0 ? TBL : 4];
   extern __shared__ __attribute__((aligned(16))) uint32_t smem[];
-  MSQ_TL(0);
   if (blockIdx.x < a.grid_routed) moe_gu_run<DR>(a, table, tbl, smem, false, blockIdx.x);
   else moe_gu_run<DS>(a, table, tbl, smem, true, blockIdx.x - a.grid_routed);
 }

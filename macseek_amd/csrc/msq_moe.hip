@@ -40,19 +40,21 @@ bool routed_type_ok(int t) { return t == MSQ_IQ1_S || t == MSQ_IQ2_XXS; }
 bool shared_type_ok(int t) { return t == MSQ_Q6_K || t == MSQ_Q8_0 || t == MSQ_IQ2_XXS || t == MSQ_IQ1_S; }
 
 template <class DR, class DS>
-void launch_gu_t(dim3 g, dim3 b, size_t lds, hipStream_t st, const MoeArgs& a) {
-  allow_large_lds(moe_gu_kernel<DR, DS>, lds);
+int launch_gu_t(dim3 g, dim3 b, size_t lds, hipStream_t st, const MoeArgs& a) {
+  if (const int rc = allow_large_lds(moe_gu_kernel<DR, DS>, lds)) return rc;
   hipLaunchKernelGGL((moe_gu_kernel<DR, DS>), g, b, lds, st, a.table, a);
+  return MSQ_OK;
 }
 template <class DR, class DS>
-void launch_down_t(dim3 g, dim3 b, size_t lds, hipStream_t st, const MoeArgs& a) {
+int launch_down_t(dim3 g, dim3 b, size_t lds, hipStream_t st, const MoeArgs& a) {
   if (b.x <= 768) {
-    allow_large_lds(moe_down_kernel<DR, DS, 768>, lds);
+    if (const int rc = allow_large_lds(moe_down_kernel<DR, DS, 768>, lds)) return rc;
     hipLaunchKernelGGL((moe_down_kernel<DR, DS, 768>), g, b, lds, st, a.table, a);
   } else {
-    allow_large_lds(moe_down_kernel<DR, DS, 1024>, lds);
+    if (const int rc = allow_large_lds(moe_down_kernel<DR, DS, 1024>, lds)) return rc;
     hipLaunchKernelGGL((moe_down_kernel<DR, DS, 1024>), g, b, lds, st, a.table, a);
   }
+  return MSQ_OK;
 }
 // launch-shape knobs for experiments (the reference exposes MACSEEK_MOE_* the same way, quant.mm:274-276)
 int env_int(const char* name, int dflt) {
@@ -79,20 +81,19 @@ size_t place_x(MoeArgs& a, size_t lds, uint32_t cols_r, uint32_t cols_s) {
 template <class D> struct DownDec { using T = D; };
 template <> struct DownDec<DecIQ1SQ> { using T = DecIQ1S; };
 // dispatch over (routed type, shared type); cols_r / cols_s: activations the routed / shared part stages (0 = none)
+// returns MSQ_OK, a launch's error, or MSQ_ERR_UNSUPPORTED (without a message) when no kernel serves the type pair
 template <bool DOWN>
-size_t dispatch(int tr, int ts, dim3 g, dim3 b, size_t part_bytes, uint32_t cols_r, uint32_t cols_s, hipStream_t st, MoeArgs& a) {
+int dispatch(int tr, int ts, dim3 g, dim3 b, size_t part_bytes, uint32_t cols_r, uint32_t cols_s, hipStream_t st, MoeArgs& a) {
 #define MSQ_MOE_CASE(TR, DRT, TS, DST)                                                            \
   if (tr == TR && ts == TS) {                                                                     \
     if constexpr (DOWN) {                                                                         \
       using R = typename DownDec<DRT>::T;                                                         \
       using S = typename DownDec<DST>::T;                                                         \
       const size_t lds = place_x<R, S, true>(a, part_bytes, cols_r, cols_s);                      \
-      launch_down_t<R, S>(g, b, lds, st, a);                                                      \
-      return lds;                                                                                 \
+      return launch_down_t<R, S>(g, b, lds, st, a);                                               \
     } else {                                                                                      \
       const size_t lds = place_x<DRT, DST, false>(a, part_bytes, cols_r, cols_s);                 \
-      launch_gu_t<DRT, DST>(g, b, lds, st, a);                                                    \
-      return lds;                                                                                 \
+      return launch_gu_t<DRT, DST>(g, b, lds, st, a);                                             \
     }                                                                                             \
   }
   MSQ_MOE_CASE(MSQ_IQ1_S, DecIQ1SQ, MSQ_Q6_K, DecQ6K)
@@ -104,7 +105,7 @@ size_t dispatch(int tr, int ts, dim3 g, dim3 b, size_t part_bytes, uint32_t cols
   MSQ_MOE_CASE(MSQ_IQ2_XXS, DecIQ2XXS, MSQ_IQ2_XXS, DecIQ2XXS)
   MSQ_MOE_CASE(MSQ_IQ2_XXS, DecIQ2XXS, MSQ_IQ1_S, DecIQ1SQ)
 #undef MSQ_MOE_CASE
-  return 0;
+  return MSQ_ERR_UNSUPPORTED;
 }
 
 int moe_decode_impl(hipStream_t st, const MsqMoeDecodeArgs* p, const MsqBuffer* table, int part, bool need_table) {
@@ -145,6 +146,8 @@ int moe_decode_impl(hipStream_t st, const MsqMoeDecodeArgs* p, const MsqBuffer* 
   if (routed_live && (gu_r || d_r)) {
     if (need_table) {
       if (!buf_ok(table, (size_t)kMaxRouted * 24)) return fail(MSQ_ERR_ARGUMENT, "macseek quant: moe_decode: table missing or too small");
+      // (the kernels read the table through the scalar cache, which ignores an address's low bits)
+      if ((uintptr_t)bptr(table) & 7) return fail(MSQ_ERR_ARGUMENT, "macseek quant: moe_decode: table not 8-byte aligned");
       a.table = (const uint64_t*)bptr(table);
     } else {
       for (int i = 0; i < nr; i++) {
@@ -195,9 +198,10 @@ int moe_decode_impl(hipStream_t st, const MsqMoeDecodeArgs* p, const MsqBuffer* 
     if (g_r) { a.rows_per_wg_r = (uint32_t)((rows_r + g_r - 1) / g_r); g_r = (rows_r + a.rows_per_wg_r - 1) / a.rows_per_wg_r; }
     if (g_s) { a.rows_per_wg_s = (uint32_t)((rows_s + g_s - 1) / g_s); g_s = (rows_s + a.rows_per_wg_s - 1) / a.rows_per_wg_s; }
     a.grid_routed = (uint32_t)g_r;
-    if (!dispatch<false>(p->t_gate_up, ts, dim3((unsigned)(g_r + g_s)), dim3(threads), part_bytes, g_r ? (uint32_t)dim : 0u,
-                         g_s ? (uint32_t)dim : 0u, st, a))
-      return unsupported("moe_decode type combo", p->t_gate_up, 0, 0);
+    const int rc = dispatch<false>(p->t_gate_up, ts, dim3((unsigned)(g_r + g_s)), dim3(threads), part_bytes, g_r ? (uint32_t)dim : 0u,
+                                   g_s ? (uint32_t)dim : 0u, st, a);
+    if (rc == MSQ_ERR_UNSUPPORTED) return unsupported("moe_decode type combo", p->t_gate_up, 0, 0);
+    if (rc != MSQ_OK) return rc;
     MSQ_HIP(hipGetLastError());
   }
   // 2) down for all experts, accumulated into y
@@ -208,8 +212,11 @@ int moe_decode_impl(hipStream_t st, const MsqMoeDecodeArgs* p, const MsqBuffer* 
     const int ne = run_d_r ? nr : 1;
     const int wpg = ne * ks;
     if (wpg > 16) return unsupported("moe_decode inter too large for the down kernel", p->t_down, dim, inter);
-    int rw = p->d_rsg > 0 ? p->d_rsg : env_d_rsg > 0 ? env_d_rsg : std::max(1, 16 / wpg);
-    if (rw * wpg > 16) rw = std::max(1, 16 / wpg);
+    // at most 12 waves where a row-group fits them: 170 registers per lane instead of 128 (the 1024-thread
+    // instantiations of some decoder pairs spill a few registers; they remain for row-groups of 13 to 16 waves)
+    const int max_waves = wpg <= 12 ? 12 : 16;
+    int rw = p->d_rsg > 0 ? p->d_rsg : env_d_rsg > 0 ? env_d_rsg : std::max(1, max_waves / wpg);
+    if (rw * wpg > max_waves) rw = std::max(1, max_waves / wpg);
     const int threads = 64 * rw * wpg;
     a.ks = (uint32_t)ks;
     a.run_routed = run_d_r; a.run_shared = d_s;
@@ -218,9 +225,10 @@ int moe_decode_impl(hipStream_t st, const MsqMoeDecodeArgs* p, const MsqBuffer* 
     const long total = std::max<long>(1, (long)cus * std::max(1, env_d_wgs));
     a.rows_per_wg = (uint32_t)((dim + total - 1) / total);
     const long grid = (dim + a.rows_per_wg - 1) / a.rows_per_wg;
-    if (!dispatch<true>(p->t_down, ts, dim3((unsigned)grid), dim3(threads), part_bytes, (uint32_t)((run_d_r ? nr : 0) * inter),
-                        d_s ? (uint32_t)inter : 0u, st, a))
-      return unsupported("moe_decode type combo", p->t_down, 0, 0);
+    const int rc = dispatch<true>(p->t_down, ts, dim3((unsigned)grid), dim3(threads), part_bytes, (uint32_t)((run_d_r ? nr : 0) * inter),
+                                  d_s ? (uint32_t)inter : 0u, st, a);
+    if (rc == MSQ_ERR_UNSUPPORTED) return unsupported("moe_decode type combo", p->t_down, 0, 0);
+    if (rc != MSQ_OK) return rc;
     MSQ_HIP(hipGetLastError());
   }
   return MSQ_OK;
@@ -230,12 +238,6 @@ int moe_decode_impl(hipStream_t st, const MsqMoeDecodeArgs* p, const MsqBuffer* 
 }  // namespace msq
 
 using namespace msq;
-
-#ifdef MSQ_EXP_TIMELINE
-extern "C" int msq_exp_timeline(void* host_out) {
-  return (int)hipMemcpyFromSymbol(host_out, HIP_SYMBOL(g_timeline), sizeof(uint64_t) * 512 * 16 * 8, 0, hipMemcpyDeviceToHost);
-}
-#endif
 
 extern "C" {
 

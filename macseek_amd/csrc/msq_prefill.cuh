@@ -434,11 +434,113 @@ __global__ __launch_bounds__(64 * pf_blk_waves(T)) void moe_pf_block_kernel(cons
   }
 }
 
-// A piece of the scratch header, handed over by value in the kernel arguments (the argument block holds 4 KB)
-constexpr int kHdrChunkWords = 960;
+// ------------------------------------------------------------------------------------------------ scratch header
+// The header of the prefill scratch (expert addresses, entry offsets, the shared expert's token tiles, the work items
+// of the block GEMM) is built on the device. What only the host knows travels in kernel arguments: a raw image
+//   word 0 n_exp | 1 has_shared | 2 n_tokens | 3 total | 4, 5 base address | 6 address mode | 7 unused
+//   words 8 .. 8 + n_exp: entry offsets offs[0 .. n_exp]
+//   then 3 addresses per expert (gate, up, down; the shared expert last): mode 0 one word each, (address - base) / 4;
+//   mode 1 two words each
+// cut into pieces of kHdrChunkWords (the argument block holds 4 KB). Every launch stores its piece behind the header;
+// the last one then expands the image: addresses and offsets as the GEMM kernels read them, and the work items --
+// an expert of m entries gives m / 112 blocks of 112 entries and one of m % 112 -- grouped by the token tiles a block
+// fills, seven-tile blocks first, one-tile blocks last, inside a group in expert order (a counting sort over seven
+// buckets: nothing in it depends on timing, so the table is the same on every run).
+constexpr int kHdrChunkWords = 960, kHdrRawHead = 8, kHdrThreads = 1024;
 struct HdrChunk { uint32_t w[kHdrChunkWords]; };
-__global__ __launch_bounds__(256) void moe_pf_header_kernel(uint32_t* dst, const HdrChunk c, uint32_t n) {
-  for (uint32_t i = threadIdx.x; i < n; i += blockDim.x) dst[i] = c.w[i];
+struct HdrBuild {
+  uint32_t* raw;        // the image, behind the header
+  uint64_t* ptrs;       // (n_exp + 1) x {gate, up, down}
+  uint32_t* offs;       // n_exp + 2
+  uint32_t* tiles;      // shared expert: {n_exp, first token} per 16 tokens
+  uint32_t* items;      // routed items, then the shared expert's
+  uint32_t build;       // 1: this launch holds the image's last piece and expands it
+};
+__host__ __device__ constexpr uint32_t pf_item_bucket(uint32_t cnt) { return 7u - (cnt + 15u) / 16u; }  // cnt in 1..112
+
+// exclusive prefix of v over the workgroup's threads; total = sum over all; wsum: 17 words of LDS
+__device__ __forceinline__ uint32_t hdr_scan(uint32_t v, uint32_t* wsum, uint32_t tid, uint32_t& total) {
+  const uint32_t lane = tid & 63u, wave = tid >> 6;
+  uint32_t inc = v;
+#pragma unroll
+  for (int d = 1; d < 64; d <<= 1) {
+    const uint32_t t = (uint32_t)__shfl_up((int)inc, d, 64);
+    if (lane >= (uint32_t)d) inc += t;
+  }
+  if (lane == 63u) wsum[wave] = inc;
+  __syncthreads();
+  if (tid == 0) {
+    uint32_t run = 0;
+    for (uint32_t w = 0; w < kHdrThreads / 64; w++) { const uint32_t t = wsum[w]; wsum[w] = run; run += t; }
+    wsum[kHdrThreads / 64] = run;
+  }
+  __syncthreads();
+  total = wsum[kHdrThreads / 64];
+  const uint32_t r = wsum[wave] + inc - v;
+  __syncthreads();
+  return r;
+}
+
+__global__ __launch_bounds__(kHdrThreads) void moe_pf_header_kernel(const HdrBuild b, const HdrChunk c, uint32_t word0, uint32_t nwords) {
+  __shared__ uint32_t wsum[kHdrThreads / 64 + 1];
+  const uint32_t tid = threadIdx.x;
+  for (uint32_t i = tid; i < nwords; i += kHdrThreads) b.raw[word0 + i] = c.w[i];
+  if (!b.build) return;
+  __syncthreads();  // the image's earlier pieces were stored by earlier launches, the last one just now
+  const uint32_t* raw = b.raw;
+  const uint32_t ne = raw[0], has_shared = raw[1], n = raw[2], total = raw[3], mode = raw[6];
+  const uint64_t base = (uint64_t)raw[4] | ((uint64_t)raw[5] << 32);
+  const uint32_t* roffs = raw + kHdrRawHead;
+  const uint32_t* rp = roffs + ne + 1;
+  for (uint32_t i = tid; i < 3u * (ne + has_shared); i += kHdrThreads)
+    b.ptrs[i] = mode ? ((uint64_t)rp[2 * i] | ((uint64_t)rp[2 * i + 1] << 32)) : base + 4ull * rp[i];
+  for (uint32_t i = tid; i <= ne; i += kHdrThreads) b.offs[i] = roffs[i];
+  if (tid == 0) b.offs[ne + 1] = total + n;
+  if (has_shared)
+    for (uint32_t i = tid; i < (n + 15u) / 16u; i += kHdrThreads) { b.tiles[2 * i] = ne; b.tiles[2 * i + 1] = 16u * i; }
+  // routed items: this thread's experts [j0, j1)
+  const uint32_t per = (ne + kHdrThreads - 1) / kHdrThreads, j0 = min(ne, tid * per), j1 = min(ne, j0 + per);
+  uint32_t cnt[7] = {0, 0, 0, 0, 0, 0, 0};
+  for (uint32_t j = j0; j < j1; j++) {
+    const uint32_t m = roffs[j + 1] - roffs[j], r = m % 112u;
+    cnt[0] += m / 112u;
+    if (r) {
+      const uint32_t bk = pf_item_bucket(r);
+#pragma unroll
+      for (int k = 0; k < 7; k++) cnt[k] += bk == (uint32_t)k;
+    }
+  }
+  uint32_t at[7], first = 0;  // where this thread's items of each bucket start
+#pragma unroll
+  for (int k = 0; k < 7; k++) {
+    uint32_t tot;
+    at[k] = first + hdr_scan(cnt[k], wsum, tid, tot);
+    first += tot;
+  }
+  for (uint32_t j = j0; j < j1; j++) {
+    const uint32_t m = roffs[j + 1] - roffs[j], q = m / 112u, r = m % 112u;
+    for (uint32_t k = 0; k < q; k++) {
+      uint32_t* it = b.items + 3 * (size_t)at[0]++;
+      it[0] = j; it[1] = 112u * k; it[2] = 112u;
+    }
+    if (r) {
+      const uint32_t bk = pf_item_bucket(r);
+      uint32_t pos = 0;
+#pragma unroll
+      for (int k = 0; k < 7; k++)
+        if (bk == (uint32_t)k) pos = at[k]++;
+      uint32_t* it = b.items + 3 * (size_t)pos;
+      it[0] = j; it[1] = 112u * q; it[2] = r;
+    }
+  }
+  // the shared expert's items follow: blocks of 112 tokens, then the rest
+  if (has_shared) {
+    const uint32_t q = n / 112u, r = n % 112u;
+    for (uint32_t k = tid; k < q + (r ? 1u : 0u); k += kHdrThreads) {
+      uint32_t* it = b.items + 3 * (size_t)(first + k);
+      it[0] = ne; it[1] = 112u * k; it[2] = k < q ? 112u : r;
+    }
+  }
 }
 
 // Xg[i] = fp16(X[src(i)]): i < total gathers token tok[i]; rows total .. total + n - 1 are the tokens themselves. One

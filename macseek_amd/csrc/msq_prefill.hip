@@ -14,11 +14,22 @@ namespace msq {
 namespace {
 
 size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
-size_t header_bytes(int total, int n, int n_exp) {
-  const size_t tiles = (size_t)n_exp + total / 16 + n / 16 + 4;  // token tiles of up to 16 entries
-  const size_t items = 2 * (size_t)n_exp + total / kPfBlkTokens + n / kPfBlkTokens + 4;  // blocks of more than 48 entries + remainders
-  return align256(24 * (size_t)(n_exp + 1) + 4 * (size_t)(n_exp + 2) + 8 * tiles + 12 * items);
+// header: addresses | offsets | the shared expert's token tiles | work items | raw image (see moe_pf_header_kernel)
+struct HdrLayout { size_t ptrs, offs, tiles, items, raw, bytes; };
+HdrLayout header_layout(int total, int n, int n_exp) {
+  HdrLayout h;
+  const size_t tiles = (size_t)n / 16 + 2;                                          // the shared expert's
+  const size_t items = 2 * ((size_t)n_exp + 1) + (size_t)total / kPfBigTokens + (size_t)n / kPfBigTokens;  // m / 112 blocks + a rest per expert
+  const size_t raw_words = kHdrRawHead + ((size_t)n_exp + 1) + 6 * ((size_t)n_exp + 1);
+  h.ptrs = 0;
+  h.offs = 24 * (size_t)(n_exp + 1);
+  h.tiles = h.offs + 4 * (size_t)(n_exp + 2);
+  h.items = h.tiles + 8 * tiles;
+  h.raw = h.items + 12 * items;
+  h.bytes = align256(h.raw + 4 * raw_words);
+  return h;
 }
+size_t header_bytes(int total, int n, int n_exp) { return header_layout(total, n, n_exp).bytes; }
 bool routed_ok(int t) { return t == MSQ_IQ1_S || t == MSQ_IQ2_XXS; }
 bool shared_ok(int t) { return t == MSQ_Q6_K || t == MSQ_Q8_0 || t == MSQ_IQ2_XXS || t == MSQ_IQ1_S; }
 
@@ -72,14 +83,20 @@ int launch_block_tt(hipStream_t st, PfBlkArgs a) {
 struct SideStream { hipStream_t stream = nullptr; hipEvent_t fork = nullptr, join = nullptr; bool ok = false; };
 std::mutex g_side_mu;
 SideStream g_side[16];
+// The device's side stream, or null when this call has to stay on the caller's stream: the fork is switched off, the
+// objects do not exist yet and `st` is being captured, or the side stream still belongs to a stream capture that `st`
+// is not part of (work forked from a capturing stream pulls the side stream into that capture until the capture ends;
+// an eager call, or a call under another capture, must not enqueue into it). Call with g_side_mu held.
 SideStream* side_stream(hipStream_t st) {
   static const bool off = [] { const char* e = getenv("MSQ_MOEP_ONE_STREAM"); return e && *e && atoi(e) != 0; }();
   int dev = 0;
   if (off || hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 16) return nullptr;
   SideStream& s = g_side[dev];
+  hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+  unsigned long long cid = 0;
+  if (st && hipStreamGetCaptureInfo(st, &cs, &cid) != hipSuccess) { (void)hipGetLastError(); return nullptr; }
   if (!s.ok) {
-    hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
-    if (hipStreamIsCapturing(st, &cs) != hipSuccess || cs != hipStreamCaptureStatusNone) return nullptr;
+    if (cs != hipStreamCaptureStatusNone) return nullptr;
     if (hipStreamCreateWithFlags(&s.stream, hipStreamNonBlocking) != hipSuccess ||
         hipEventCreateWithFlags(&s.fork, hipEventDisableTiming) != hipSuccess ||
         hipEventCreateWithFlags(&s.join, hipEventDisableTiming) != hipSuccess) {
@@ -88,6 +105,11 @@ SideStream* side_stream(hipStream_t st) {
     }
     s.ok = true;
   }
+  hipStreamCaptureStatus ss = hipStreamCaptureStatusNone;
+  unsigned long long sid = 0;
+  if (hipStreamGetCaptureInfo(s.stream, &ss, &sid) != hipSuccess) { (void)hipGetLastError(); return nullptr; }
+  if (ss != hipStreamCaptureStatusNone && !(cs == hipStreamCaptureStatusActive && ss == hipStreamCaptureStatusActive && cid == sid))
+    return nullptr;
   return &s;
 }
 
@@ -189,107 +211,79 @@ int msq_moe_prefill(void* stream, const MsqMoePrefillArgs* p) {
   // src/kernels/quant.mm:520-522)
   const char* skip_env = getenv("MSQ_MOEP_SKIP");
   const int skip = skip_env && *skip_env ? atoi(skip_env) : 0;
-  // ---- header: expert pointer table, offsets, token-tile tables (routed tiles first, then the shared expert's)
-  const size_t hbytes = header_bytes(total, n, ne);
-  std::vector<uint8_t> hdr(hbytes, 0);
-  uint64_t* ptrs = (uint64_t*)hdr.data();
-  uint32_t* offs = (uint32_t*)(hdr.data() + 24 * (size_t)(ne + 1));
-  uint32_t* tiles = offs + (ne + 2);
-  for (int j = 0; j < ne; j++) {
-    ptrs[3 * j] = (uint64_t)(uintptr_t)bptr(&p->slots[j].gate);
-    ptrs[3 * j + 1] = (uint64_t)(uintptr_t)bptr(&p->slots[j].up);
-    ptrs[3 * j + 2] = (uint64_t)(uintptr_t)bptr(&p->slots[j].down);
-    offs[j] = (uint32_t)p->offs[j];
-  }
-  offs[ne] = (uint32_t)total;
-  offs[ne + 1] = (uint32_t)(total + n);
-  if (p->has_shared) {
-    ptrs[3 * ne] = (uint64_t)(uintptr_t)bptr(&p->shared.gate);
-    ptrs[3 * ne + 1] = (uint64_t)(uintptr_t)bptr(&p->shared.up);
-    ptrs[3 * ne + 2] = (uint64_t)(uintptr_t)bptr(&p->shared.down);
-  }
-  uint32_t nt_routed = 0, nt_shared = 0;
-  for (int j = 0; j < ne; j++)
-    for (int t0 = 0; t0 < p->offs[j + 1] - p->offs[j]; t0 += 16) { tiles[2 * nt_routed] = (uint32_t)j; tiles[2 * nt_routed + 1] = (uint32_t)t0; nt_routed++; }
-  if (p->has_shared)
-    for (int t0 = 0; t0 < n; t0 += 16) { tiles[2 * (nt_routed + nt_shared)] = (uint32_t)ne; tiles[2 * (nt_routed + nt_shared) + 1] = (uint32_t)t0; nt_shared++; }
-  // work items of the block GEMM, largest first (they take longest)
-  uint32_t* items = tiles + 2 * (size_t)(nt_routed + nt_shared);
+  // ---- header. The host only counts the work items per class (the launches' grids); the tables themselves are built
+  // on the device from a raw image that travels in kernel arguments (moe_pf_header_kernel): nothing is read from host
+  // memory after this call returns, the call never waits for the stream, and a stream capture records the values.
+  const HdrLayout hl = header_layout(total, n, ne);
+  const uint32_t nt_shared = p->has_shared ? (uint32_t)((n + 15) / 16) : 0u;
   uint32_t ni_routed = 0, ni_shared = 0;
   uint32_t nc_routed[3] = {0, 0, 0}, nc_shared[3] = {0, 0, 0};  // items of more than 48 entries / three tiles / two tiles
-  {
-    // an expert's entries are cut into blocks of kPfBigTokens while more than kPfBlkTokens remain, then one block of
-    // at most kPfBlkTokens
-    auto cut = [](std::vector<std::array<uint32_t, 3>>& v, uint32_t e, int m) {
-      int t0 = 0;
-      while (m - t0 > kPfBlkTokens) { const int c = std::min(kPfBigTokens, m - t0); v.push_back({e, (uint32_t)t0, (uint32_t)c}); t0 += c; }
-      if (m - t0 > 0) v.push_back({e, (uint32_t)t0, (uint32_t)(m - t0)});
-    };
-    auto emit = [&](std::vector<std::array<uint32_t, 3>>& v, uint32_t* dst, uint32_t* nc) {
-      std::stable_sort(v.begin(), v.end(), [](const auto& x, const auto& y) { return x[2] > y[2]; });
-      uint32_t k = 0;
-      for (const auto& it : v) {
-        std::copy(it.begin(), it.end(), dst + 3 * (size_t)k++);
-        nc[0] += it[2] > 48; nc[1] += it[2] > 32 && it[2] <= 48; nc[2] += it[2] > 16 && it[2] <= 32;
-      }
-      return k;
-    };
-    std::vector<std::array<uint32_t, 3>> v;
-    for (int j = 0; j < ne; j++) cut(v, (uint32_t)j, p->offs[j + 1] - p->offs[j]);
-    ni_routed = emit(v, items, nc_routed);
-    v.clear();
-    if (p->has_shared) cut(v, (uint32_t)ne, n);
-    ni_shared = emit(v, items + 3 * (size_t)ni_routed, nc_shared);
-  }
-  uint8_t* sc = bptr_mut(&p->scratch);
-  // The header travels in kernel arguments, a few KB per launch: nothing is read from host memory after this call
-  // returns, the call never waits for the stream, and a stream capture records the values themselves. The gather does
-  // not read the header: the header's launches (a dozen, each a few microseconds of launch latency) go to the side
-  // stream when there is one and are joined behind the gather.
-  auto write_header = [&](hipStream_t hs) {
-    const size_t used = 24 * (size_t)(ne + 1) + 4 * (size_t)(ne + 2) + 8 * (size_t)(nt_routed + nt_shared) +
-                        12 * (size_t)(ni_routed + ni_shared);
-    const size_t words = (used + 3) / 4;
-    for (size_t w0 = 0; w0 < words; w0 += kHdrChunkWords) {
-      HdrChunk c;
-      const uint32_t n = (uint32_t)std::min<size_t>(kHdrChunkWords, words - w0);
-      memcpy(c.w, hdr.data() + 4 * w0, 4 * (size_t)n);  // hdr is padded to a multiple of 256 bytes
-      hipLaunchKernelGGL(moe_pf_header_kernel, dim3(1), dim3(256), 0, hs, (uint32_t*)sc + w0, c, n);
-    }
+  auto count = [](int m, uint32_t& ni, uint32_t* nc) {  // an expert of m entries: m / 112 blocks of 112 and one of m % 112
+    const uint32_t q = (uint32_t)(m / kPfBigTokens), r = (uint32_t)(m % kPfBigTokens);
+    ni += q + (r ? 1u : 0u);
+    nc[0] += q + (r > 48 ? 1u : 0u); nc[1] += r > 32 && r <= 48; nc[2] += r > 16 && r <= 32;
   };
+  for (int j = 0; j < ne; j++) count(p->offs[j + 1] - p->offs[j], ni_routed, nc_routed);
+  if (p->has_shared) count(n, ni_shared, nc_shared);
+  uint8_t* sc = bptr_mut(&p->scratch);
+  {
+    const int nptr = 3 * (ne + (p->has_shared ? 1 : 0));
+    std::vector<uint64_t> ptrs((size_t)nptr);
+    for (int j = 0; j < ne; j++) {
+      ptrs[3 * j] = (uint64_t)(uintptr_t)bptr(&p->slots[j].gate);
+      ptrs[3 * j + 1] = (uint64_t)(uintptr_t)bptr(&p->slots[j].up);
+      ptrs[3 * j + 2] = (uint64_t)(uintptr_t)bptr(&p->slots[j].down);
+    }
+    if (p->has_shared) {
+      ptrs[3 * ne] = (uint64_t)(uintptr_t)bptr(&p->shared.gate);
+      ptrs[3 * ne + 1] = (uint64_t)(uintptr_t)bptr(&p->shared.up);
+      ptrs[3 * ne + 2] = (uint64_t)(uintptr_t)bptr(&p->shared.down);
+    }
+    // addresses as one word each, (address - lowest address) / 4, when they all lie within 16 GiB of the lowest and
+    // are 4 bytes apart (expert matrices are 4-byte aligned); else in full
+    uint64_t base = nptr ? *std::min_element(ptrs.begin(), ptrs.end()) : 0;
+    bool rel = true;
+    for (uint64_t v : ptrs) rel = rel && !((v - base) & 3) && ((v - base) >> 2) <= 0xFFFFFFFFull;
+    std::vector<uint32_t> raw;
+    raw.reserve(kHdrRawHead + (size_t)ne + 1 + (rel ? 1 : 2) * (size_t)nptr);
+    raw.insert(raw.end(), {(uint32_t)ne, p->has_shared ? 1u : 0u, (uint32_t)n, (uint32_t)total, (uint32_t)base, (uint32_t)(base >> 32),
+                           rel ? 0u : 1u, 0u});
+    for (int j = 0; j < ne; j++) raw.push_back((uint32_t)p->offs[j]);
+    raw.push_back((uint32_t)total);
+    for (uint64_t v : ptrs) {
+      if (rel) raw.push_back((uint32_t)((v - base) >> 2));
+      else { raw.push_back((uint32_t)v); raw.push_back((uint32_t)(v >> 32)); }
+    }
+    HdrBuild hb{};
+    hb.raw = (uint32_t*)(sc + hl.raw); hb.ptrs = (uint64_t*)(sc + hl.ptrs); hb.offs = (uint32_t*)(sc + hl.offs);
+    hb.tiles = (uint32_t*)(sc + hl.tiles); hb.items = (uint32_t*)(sc + hl.items);
+    for (size_t w0 = 0; w0 < raw.size(); w0 += kHdrChunkWords) {
+      HdrChunk c;
+      const uint32_t nw = (uint32_t)std::min<size_t>(kHdrChunkWords, raw.size() - w0);
+      memcpy(c.w, raw.data() + w0, 4 * (size_t)nw);
+      hb.build = w0 + nw == raw.size() ? 1u : 0u;
+      hipLaunchKernelGGL(moe_pf_header_kernel, dim3(1), dim3(kHdrThreads), 0, st, hb, c, (uint32_t)w0, nw);
+    }
+    MSQ_HIP(hipGetLastError());
+  }
+  const size_t hbytes = hl.bytes;
   const size_t rows = (size_t)total + n;
   uint16_t* Xg = (uint16_t*)(sc + hbytes);
   uint16_t* H = (uint16_t*)((uint8_t*)Xg + align256(rows * dim * 2));
   float* Z = (float*)((uint8_t*)H + align256(rows * inter * 2));
-  const uint64_t* d_ptrs = (const uint64_t*)sc;
-  const uint32_t* d_offs = (const uint32_t*)(sc + 24 * (size_t)(ne + 1));
-  const uint32_t* d_tiles = d_offs + (ne + 2);
-  const uint32_t* d_items = d_tiles + 2 * (size_t)(nt_routed + nt_shared);
+  const uint64_t* d_ptrs = (const uint64_t*)(sc + hl.ptrs);
+  const uint32_t* d_offs = (const uint32_t*)(sc + hl.offs);
+  const uint32_t* d_tiles = (const uint32_t*)(sc + hl.tiles);
+  const uint32_t* d_items = (const uint32_t*)(sc + hl.items);
+  const bool any_routed = total > 0;
 
   // 1) gather + convert
   const uint32_t grows = (uint32_t)(total + (p->has_shared ? n : 0));
-  auto gather = [&]() {
-    if (grows > 0 && !(skip & 1)) {
-      const dim3 grid(grows), block(256);
-      const int* tok = total > 0 ? (const int*)bptr(&p->tok) : nullptr;
-      if (p->x_is_bf16) hipLaunchKernelGGL((moe_pf_gather_kernel<true>), grid, block, 0, st, (const void*)bptr(&p->X), Xg, tok, (uint32_t)total, grows, (uint32_t)dim);
-      else hipLaunchKernelGGL((moe_pf_gather_kernel<false>), grid, block, 0, st, (const void*)bptr(&p->X), Xg, tok, (uint32_t)total, grows, (uint32_t)dim);
-    }
-  };
-  {
-    std::lock_guard<std::mutex> lock(g_side_mu);
-    SideStream* s = (grows > 0 && !(skip & 1)) ? side_stream(st) : nullptr;
-    if (s) {
-      MSQ_HIP(hipEventRecord(s->fork, st));
-      MSQ_HIP(hipStreamWaitEvent(s->stream, s->fork, 0));
-      write_header(s->stream);
-      MSQ_HIP(hipEventRecord(s->join, s->stream));
-      gather();
-      MSQ_HIP(hipStreamWaitEvent(st, s->join, 0));
-    } else {
-      write_header(st);
-      gather();
-    }
+  if (grows > 0 && !(skip & 1)) {
+    const dim3 grid(grows), block(256);
+    const int* tok = total > 0 ? (const int*)bptr(&p->tok) : nullptr;
+    if (p->x_is_bf16) hipLaunchKernelGGL((moe_pf_gather_kernel<true>), grid, block, 0, st, (const void*)bptr(&p->X), Xg, tok, (uint32_t)total, grows, (uint32_t)dim);
+    else hipLaunchKernelGGL((moe_pf_gather_kernel<false>), grid, block, 0, st, (const void*)bptr(&p->X), Xg, tok, (uint32_t)total, grows, (uint32_t)dim);
     MSQ_HIP(hipGetLastError());
   }
   PfArgs a{};
@@ -314,30 +308,36 @@ int msq_moe_prefill(void* stream, const MsqMoePrefillArgs* p) {
       return launch_block<GU>(type, gs, b, nc[0], nc[1], nc[2], skip, which);
     }
     a.A = A; a.N = N; steps(K); a.row_bytes = (uint32_t)row_bytes;
-    a.tiles = d_tiles + (shared ? 2 * (size_t)nt_routed : 0); a.ntiles = shared ? nt_shared : nt_routed;
+    // (the token-tile kernel only ever serves a Q6_K / Q8_0 shared expert: routed experts are codebook formats)
+    a.tiles = d_tiles; a.ntiles = shared ? nt_shared : 0u;
+    if (!a.ntiles) return MSQ_OK;
     return launch_gemm<GU>(type, gs, a, cus);
   };
   int rc;
-  const bool routed_gu = nt_routed && !(skip & 2), routed_dn = nt_routed && !(skip & 8);
+  const bool routed_gu = any_routed && !(skip & 2), routed_dn = any_routed && !(skip & 8);
   const int both = kBig | kSmall;
   // The routed experts' two item classes as two pipelines (see SideStream) when both exist and a side stream does
   bool forked = false;
   if ((routed_gu || routed_dn) && block_path(p->t_gate_up) && block_path(p->t_down) && nc_routed[0] > 0 &&
       ni_routed > nc_routed[0] && !(skip & 256) && (skip & (64 | 128)) != (64 | 128)) {
     std::lock_guard<std::mutex> lock(g_side_mu);
-    if (SideStream* s = side_stream(st)) {
+    SideStream* s = side_stream(st);
+    if (s && hipEventRecord(s->fork, st) == hipSuccess && hipStreamWaitEvent(s->stream, s->fork, 0) == hipSuccess) {
       forked = true;
-      MSQ_HIP(hipEventRecord(s->fork, st));
-      MSQ_HIP(hipStreamWaitEvent(s->stream, s->fork, 0));
       rc = routed_gu ? gemm(std::true_type{}, p->t_gate_up, false, Xg, (uint32_t)dim, (uint32_t)inter, rb_gu, s->stream, kBig) : MSQ_OK;
       if (rc == MSQ_OK && routed_dn) rc = gemm(std::false_type{}, p->t_down, false, H, (uint32_t)inter, (uint32_t)dim, rb_d, s->stream, kBig);
-      MSQ_HIP(hipEventRecord(s->join, s->stream));
+      // whatever happened above, the side stream is joined back before anything else can fail: a caller's capture is
+      // never left with an unjoined stream
+      const hipError_t ej = hipEventRecord(s->join, s->stream);
+      const hipError_t ew = ej == hipSuccess ? hipStreamWaitEvent(st, s->join, 0) : ej;
+      if (rc == MSQ_OK && ew != hipSuccess) rc = hip_fail(ew, "joining the side stream");
       if (rc == MSQ_OK && routed_gu) rc = gemm(std::true_type{}, p->t_gate_up, false, Xg, (uint32_t)dim, (uint32_t)inter, rb_gu, st, kSmall);
       if (rc == MSQ_OK && nt_shared && !(skip & 4)) rc = gemm(std::true_type{}, p->t_shared, true, Xg, (uint32_t)dim, (uint32_t)inter, rb_sgu, st, both);
       if (rc == MSQ_OK && routed_dn) rc = gemm(std::false_type{}, p->t_down, false, H, (uint32_t)inter, (uint32_t)dim, rb_d, st, kSmall);
       if (rc == MSQ_OK && nt_shared && !(skip & 16)) rc = gemm(std::false_type{}, p->t_shared, true, H, (uint32_t)inter, (uint32_t)dim, rb_sd, st, both);
-      MSQ_HIP(hipStreamWaitEvent(st, s->join, 0));  // the side stream is joined whatever happened above
       if (rc != MSQ_OK) return rc;
+    } else {
+      (void)hipGetLastError();
     }
   }
   if (!forked) {
@@ -349,11 +349,11 @@ int msq_moe_prefill(void* stream, const MsqMoePrefillArgs* p) {
     if (nt_shared && !(skip & 16) && (rc = gemm(std::false_type{}, p->t_shared, true, H, (uint32_t)inter, (uint32_t)dim, rb_sd, st, both))) return rc;
   }
   // 4) ordered reduction into Y
-  if ((nt_routed || nt_shared) && !(skip & 32)) {
+  if ((any_routed || nt_shared) && !(skip & 32)) {
     const dim3 grid((dim / 4 + 255) / 256, (unsigned)n), block(256);
     hipLaunchKernelGGL(moe_pf_reduce_kernel, grid, block, 0, st, (const float*)Z, (float*)bptr_mut(&p->Y),
                        p->k_per_token > 0 ? (const int*)bptr(&p->slot_of) : nullptr, (uint32_t)n, (uint32_t)total, (uint32_t)dim,
-                       (uint32_t)(nt_routed ? p->k_per_token : 0), (uint32_t)(p->has_shared ? 1 : 0));
+                       (uint32_t)(any_routed ? p->k_per_token : 0), (uint32_t)(p->has_shared ? 1 : 0));
     MSQ_HIP(hipGetLastError());
   }
   return MSQ_OK;

@@ -1,3 +1,6 @@
+// NOT part of libmsq.so: a measurement tool of the benchmark, built into a shared object of its own (libmsq_probe.so)
+// that only `bench.py --workload issue_probe` loads.
+//
 // Instruction-issue probes: how fast one SIMD of this device issues the instruction kinds the decode and prefill
 // kernels are built from, alone and mixed, at a chosen number of waves per SIMD. The design decisions that rest on
 // these figures (vector-issue ceiling of a table decode, whether matrix-core work hides behind vector work) can be
@@ -15,7 +18,8 @@
 //   VFMA   32 x v_fma_f32 (four chains)
 // and the mixes VALU+MFMA16, VALU+MFMA4, VALU+LDS, VALU+LDS+MFMA4, VINT+MFMA16, VPK+MFMA16, VFMA+MFMA16 (groups
 // interleaved 4 : 1 in program order).
-#include "msq_host.h"
+#include <hip/hip_runtime.h>
+#include <stdint.h>
 
 namespace msq {
 
@@ -112,11 +116,12 @@ static void launch_probe(hipStream_t st, int grid, int block, uint32_t* sink, ui
 
 using namespace msq;
 
-extern "C" int msq_issue_probe(void* stream, int mask, int grid, int block, int iters, const MsqBuffer* sink) {
-  if (grid < 1 || block < 64 || block > 1024 || block % 64 || iters < 1 || !buf_ok(sink, (size_t)grid * 4))
-    return fail(MSQ_ERR_ARGUMENT, "macseek quant: issue_probe: bad launch shape or sink too small (grid %d block %d iters %d)", grid, block, iters);
+// mask ORs the groups above (1 VALU, 2 MFMA16, 4 MFMA4, 8 MFMA8, 16 LDS, 32 VINT, 64 VPK, 128 VFMA); sink holds at least
+// 4 * grid bytes of device memory. Returns 0, -1 for a bad launch shape or an unknown mix, or the HIP error code.
+extern "C" int msq_probe_issue(void* stream, int mask, int grid, int block, int iters, void* sink, size_t sink_bytes) {
+  if (grid < 1 || block < 64 || block > 1024 || block % 64 || iters < 1 || !sink || sink_bytes < (size_t)grid * 4) return -1;
   hipStream_t st = (hipStream_t)stream;
-  uint32_t* s = (uint32_t*)bptr_mut(sink);
+  uint32_t* s = (uint32_t*)sink;
   switch (mask) {
     case P_VALU: launch_probe<P_VALU>(st, grid, block, s, iters); break;
     case P_MFMA16: launch_probe<P_MFMA16>(st, grid, block, s, iters); break;
@@ -133,8 +138,7 @@ extern "C" int msq_issue_probe(void* stream, int mask, int grid, int block, int 
     case P_VFMA: launch_probe<P_VFMA>(st, grid, block, s, iters); break;
     case P_VFMA | P_MFMA16: launch_probe<P_VFMA | P_MFMA16>(st, grid, block, s, iters); break;
     case P_VALU | P_LDS | P_MFMA4: launch_probe<P_VALU | P_LDS | P_MFMA4>(st, grid, block, s, iters); break;
-    default: return fail(MSQ_ERR_ARGUMENT, "macseek quant: issue_probe: unknown instruction mix %d", mask);
+    default: return -1;
   }
-  MSQ_HIP(hipGetLastError());
-  return MSQ_OK;
+  return (int)hipGetLastError();
 }

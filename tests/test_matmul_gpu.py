@@ -120,5 +120,16 @@ def test_matmul_misuse(dev):
         q.encode_matmul(e, q.QType.Q6_K, W, 16, 192, v, v, 4)  # cols % 128 (quant.mm:196)
     with pytest.raises(q.QuantError, match="matmul unsupported"):
         q.encode_matmul(e, q.QType.Q6_K, W, 16, 256, v, v, 0)
+    # a multiple of 128 columns that is not whole 256-weight blocks: refused on the host, on both routes and entry points
+    # (nothing is launched: the output keeps its bytes)
+    out = torch.full((2048 * 16,), 7.0, dtype=torch.float32, device=dev)
+    for t in (q.QType.Q6_K, q.QType.Q5_K, q.QType.IQ1_S, q.QType.IQ2_XXS):
+        for n in (4, 512):  # the fused kernel's range and the materialising route's
+            with pytest.raises(q.QuantError, match=r"matmul unsupported \(type \S+ rows 16 cols 384\)"):
+                q.encode_matmul(e, t, W, 16, 384, v, q.Buffer.of(out), n)
+            with pytest.raises(q.QuantError, match=r"matmul unsupported \(type \S+ rows 16 cols 384\)"):
+                q.encode_matmul_h(e, t, W, 16, 384, v, q.Buffer.of(out), n)
+    e.wait()
+    assert bool((out == 7.0).all())
     with pytest.raises(q.QuantError, match="f32_to_f16 unsupported"):
         q.encode_f32_to_f16(e, v, v, 6)

@@ -65,11 +65,13 @@ class Layer:
         return O.moe_decode(*self.types, self.n_routed, self.shared, self.dim, self.inter, self.G, self.U, self.D,
                             W6, self.x, self.y0)
 
-    def check(self, y, h=None, what="", h_tol=2e-5, y_tol=5e-5):
+    def check(self, y, h=None, what="", h_tol=2e-5, y_tol=5e-5, chain_tol=1e-4):
         """Stage-wise parity (the reference test checks h, then y: tests/test_quant_moe.mm:82-92):
         h against the oracle's h; y against the float64 down projection of the h the GPU produced (so stage 2 is
         judged on its own inputs), both in the reference's metric and in the north-star metric
-        max |dy| <= 1e-3 * (sum_e ||Wd_e[r]||_2 ||h_e||_2 + |y0[r]|); finally the whole chain against the oracle."""
+        max |dy| <= 1e-3 * (sum_e ||Wd_e[r]||_2 ||h_e||_2 + |y0[r]|); finally the whole chain -- y against the down
+        projection of the ORACLE's h, which is the reference test's y check (tests/test_quant_moe.mm:88-93, 5e-5) --
+        to chain_tol (CHAIN_TOL below says where the reference's bound holds and where it does not)."""
         ry, ymag, rh, hs = self.oracle()
         got = y.cpu().numpy().astype(np.float64)
         assert np.all(np.isfinite(got))
@@ -93,7 +95,7 @@ class Layer:
             ns_err = float(np.max(np.abs(got - y2) / (scale + 1e-30)))
         print(f"  {what} h_err {h_err:.2e} y_err {y_err:.2e} north-star {ns_err:.2e} chain {chain_err:.2e}")
         # the reference's own bounds for its F32-activation kernels: h 2e-5, y 5e-5 (tests/test_quant_moe.mm:82-93)
-        assert h_err <= h_tol and y_err <= y_tol and ns_err <= 1e-3 and chain_err <= 5e-3
+        assert h_err <= h_tol and y_err <= y_tol and ns_err <= 1e-3 and chain_err <= chain_tol
         return ry
 
 
@@ -122,6 +124,29 @@ H_TOL = {(T.IQ2_XXS, T.IQ1_S, T.IQ2_XXS, 1, True, 1.0, 256, 16384): 6e-5}
 Y_TOL = {(T.IQ1_S, T.IQ1_S, T.IQ2_XXS, 6, True, 0.02, 7168, 2048): 8e-5}
 
 
+# Whole chain (y against the down projection of the oracle's h). What it measures is the rounding of x in gate/up carried
+# through SwiGLU and the down projection: 2^-16 of a 32-column unit's largest value for IQ1_S gate/up, fp16 for the other
+# block formats, none for a Q8_0 shared expert. The reference's kernels take x as F32 and its test holds 5e-5
+# (tests/test_quant_moe.mm:92-93). Asserted here: 5e-5 where gate/up of the heavy expert rounds x finer than fp16
+# (REF_CHAIN: the Q8_0 shared expert, weight 1, keeps x in fp32), 1e-4 otherwise, and for the inputs on which SwiGLU
+# saturates or x sits high in the fp16 range -- h stops growing with x, its error does not -- the bound given below
+# (measured value in brackets).
+REF_CHAIN = {(T.IQ1_S, T.IQ2_XXS, T.Q8_0, 6, True, 1.0, 5120, 2304),   # [2.4e-5]
+             (T.IQ2_XXS, T.IQ2_XXS, T.Q6_K, 6, True, 1.0, 5120, 2304),  # [4.6e-5]
+             (T.IQ2_XXS, T.IQ1_S, T.IQ1_S, 5, True, 1.0, 7168, 2048),   # [4.3e-5]
+             (T.IQ1_S, T.IQ1_S, T.Q8_0, 2, True, 1.0, 32768, 256),      # [3.5e-5]
+             (T.IQ2_XXS, T.IQ1_S, T.IQ2_XXS, 1, True, 1.0, 256, 16384)}  # [2.7e-5]
+CHAIN_TOL = {(T.IQ1_S, T.IQ1_S, T.Q6_K, 6, True, 40.0, 5120, 2304): 6e-4,      # [4.3e-4] clamp-heavy
+             (T.IQ1_S, T.IQ1_S, T.IQ2_XXS, 1, True, 40.0, 512, 256): 1.5e-3,   # [1.0e-3] clamp-heavy, 512-column rows
+             (T.IQ1_S, T.IQ1_S, T.IQ2_XXS, 6, True, 1500.0, 7168, 2048): 5e-4,  # [3.3e-4] clamp-heavy
+             (T.IQ1_S, T.IQ1_S, T.IQ2_XXS, 6, True, 1.0, 7168, 2048): 1.5e-4}   # [1.2e-4] fp16-staged IQ2_XXS shared expert, weight 1
+BASELINE_CHAIN_TOL = 2e-4  # the same layer with the 384-expert arena (tests/test_full_size_gpu.py) [1.4e-4]
+
+
+def chain_tol_of(case):
+    return 5e-5 if case in REF_CHAIN else CHAIN_TOL.get(case, 1e-4)
+
+
 @pytest.mark.parametrize("gu,dn,sh,nr,shared,xs,dim,inter", CASES)
 def test_moe_decode_vs_oracle(dev, gu, dn, sh, nr, shared, xs, dim, inter):
     L = Layer(gu, dn, sh, nr, shared, dim, inter, xs)
@@ -130,7 +155,8 @@ def test_moe_decode_vs_oracle(dev, gu, dn, sh, nr, shared, xs, dim, inter):
     q.encode_moe_decode(e, L.args(y))
     e.wait()
     L.check(y, L.scratch, f"gu={O.TYPE_NAMES[gu]} down={O.TYPE_NAMES[dn]} shared={O.TYPE_NAMES[sh] if shared else '-'} routed={nr} xs={xs}",
-            h_tol=H_TOL.get((gu, dn, sh, nr, shared, xs, dim, inter), 2e-5), y_tol=Y_TOL.get((gu, dn, sh, nr, shared, xs, dim, inter), 5e-5))
+            h_tol=H_TOL.get((gu, dn, sh, nr, shared, xs, dim, inter), 2e-5), y_tol=Y_TOL.get((gu, dn, sh, nr, shared, xs, dim, inter), 5e-5),
+            chain_tol=chain_tol_of((gu, dn, sh, nr, shared, xs, dim, inter)))
 
 
 @pytest.mark.parametrize("dim,inter,sh", [(5120, 2304, O.Q6_K), (7168, 2048, O.IQ2_XXS)])
@@ -152,13 +178,14 @@ def test_table_variant_and_parts(dev, dim, inter, sh):
         return y, L.scratch.clone()
 
     y_all, h_all = run([q.MoePart.All])
-    L.check(y_all, h_all, "table All")
+    ctol = 1e-4 if sh == O.Q6_K else 1.5e-4  # measured 6.8e-5 / 9.9e-5 (fp16-staged shared expert: see CHAIN_TOL)
+    L.check(y_all, h_all, "table All", chain_tol=ctol)
     y_bound, h_bound = run(None, bound=True)
     assert torch.equal(y_all, y_bound) and torch.equal(h_all, h_bound)  # same kernels, pointers by value or by table
     y2, h2 = run([q.MoePart.SharedGu, q.MoePart.AfterSharedGu])
     assert torch.equal(y_all, y2) and torch.equal(h_all, h2)            # bit-identical (quant.hpp:80)
     y3, _ = run([q.MoePart.Shared, q.MoePart.Routed])
-    ry = L.check(y3, None, "Shared + Routed")
+    ry = L.check(y3, None, "Shared + Routed", chain_tol=ctol)
     assert float((y3 - y_all).abs().max()) <= 1e-5 * float(np.max(np.abs(ry)))  # tests/test_dec_sync.mm: 1e-5 max|y|
     y4, h4 = run([q.MoePart.Shared])
     y5, h5 = run([q.MoePart.SharedGu, q.MoePart.SharedDown])
@@ -190,6 +217,10 @@ def test_moe_decode_misuse(dev):
     a.scratch = a.scratch.sub(0, 64)
     with pytest.raises(q.QuantError, match="scratch too small"):
         q.encode_moe_decode(e, a)
+    # an expert address table that is not 8-byte aligned is refused on the host (the kernels read it with scalar loads)
+    tbl = torch.zeros(20, dtype=torch.int64, device=dev)
+    with pytest.raises(q.QuantError, match="table not 8-byte aligned"):
+        q.encode_moe_decode_table(e, L.args(y), q.Buffer.of(tbl).sub(4, 152))
     a = L.args(y)
     a.n_routed, a.has_shared = 0, False   # nothing to do: silent return, y untouched (quant.mm:269)
     q.encode_moe_decode(e, a)

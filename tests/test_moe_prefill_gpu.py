@@ -233,3 +233,49 @@ def test_moe_prefill_misuse(dev):
     a.t_gate_up = q.QType.Q5_K
     with pytest.raises(q.QuantError, match="moe_prefill types unsupported"):
         q.encode_moe_prefill(q.Enc(), a)
+
+
+def test_moe_prefill_eager_call_while_another_stream_captures(dev):
+    """The library forks part of a call onto a stream of its own. While a caller's capture is open that stream belongs
+    to the capture; a second call from another stream in that window -- eager, with its own scratch -- must neither be
+    swallowed by the capture nor fail: it stays on its caller's stream, runs at once and gives the eager result, and
+    the captured graph still replays the eager result afterwards."""
+    c = build(O.IQ2_XXS, O.IQ1_S, O.Q8_0, 600, 6, 20, True, "sizes", 512, 256)
+    y_eager, same = run_gpu(c)
+    assert same
+    total = len(c["tok"])
+    keep = [up(c["tok"]), up(c["wt"]), up(c["slot_of"])]
+    nbytes = q.moe_prefill_scratch_bytes(total, c["n"], c["n_exp"], c["dim"], c["inter"])
+    Xd = up(c["X"])
+    Y = [up(c["Y0"].copy()) for _ in range(2)]
+    scr = [torch.empty(nbytes, dtype=torch.uint8, device="cuda:0") for _ in range(2)]
+
+    def args(i):
+        a = q.MoePrefillArgs()
+        a.t_gate_up, a.t_down, a.t_shared = c["types"]
+        a.n_tokens, a.n_exp, a.slots, a.offs = c["n"], c["n_exp"], c["slots"][:c["n_exp"]], list(c["offs"])
+        a.tok, a.wt, a.slot_of = q.Buffer.of(keep[0]), q.Buffer.of(keep[1]), q.Buffer.of(keep[2])
+        a.k_per_token, a.has_shared, a.shared = c["k"], True, c["slots"][c["n_exp"]]
+        a.X, a.Y, a.scratch = q.Buffer.of(Xd), q.Buffer.of(Y[i]), q.Buffer.of(scr[i])
+        a.dim, a.inter, a.x_is_bf16 = c["dim"], c["inter"], False
+        return a
+
+    other = torch.cuda.Stream()
+    host = torch.empty_like(Y[1], device="cpu").pin_memory()
+    want = y_eager.cpu()
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g, capture_error_mode="relaxed"):
+        q.encode_moe_prefill(q.Enc(torch.cuda.current_stream()), args(0))
+        # the capture is still open: an eager call on another stream
+        q.encode_moe_prefill(q.Enc(other), args(1))
+        with torch.cuda.stream(other):
+            host.copy_(Y[1], non_blocking=True)
+        other.synchronize()
+        ran_eagerly = bool(torch.equal(host, want))
+    assert ran_eagerly, "the eager call did not run (or ran wrongly) while the other stream was capturing"
+    assert torch.equal(Y[0].cpu(), torch.from_numpy(c["Y0"])), "the captured call ran during the capture"
+    g.replay()
+    torch.cuda.synchronize()
+    assert torch.equal(Y[0], y_eager)
+

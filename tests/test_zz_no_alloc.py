@@ -30,7 +30,7 @@ def test_static_scratch_entry_point_matches_caller_scratch(dev):
     big = Layer(O.IQ1_S, O.IQ1_S, O.IQ2_XXS, 6, True, 7168, 2048)
     y_ref, y_static = run_both(big)
     assert torch.equal(y_ref, y_static)
-    big.check(y_static, None, "static scratch, 7168/2048")
+    big.check(y_static, None, "static scratch, 7168/2048", chain_tol=1.5e-4)
     # second call, smaller layer: the array still holds the first call's h rows beyond the new layer's
     small = Layer(O.IQ1_S, O.IQ2_XXS, O.Q8_0, 2, True, 512, 256, seed=300)
     y_ref, y_static = run_both(small)
@@ -39,6 +39,41 @@ def test_static_scratch_entry_point_matches_caller_scratch(dev):
     # and the first shape again
     y_ref, y_static = run_both(big)
     assert torch.equal(y_ref, y_static)
+
+
+def test_static_entry_point_allocates_nothing_and_can_be_captured(dev):
+    """What the entry point exists for: a call enqueues and allocates nothing, so it can sit inside a HIP graph. After
+    one warm-up call (the first call on a device looks the array's address up and sets the kernels' LDS limits) the
+    device's free memory is the same before and after a call, and a graph that holds the call repeats the eager result
+    bit for bit on every replay, with eager work and synchronizations between the replays."""
+    L = Layer(O.IQ1_S, O.IQ1_S, O.IQ2_XXS, 6, True, 7168, 2048)
+    y0 = up(L.y0.copy())
+    y_eager, y_graph = up(L.y0.copy()), up(L.y0.copy())
+    e = q.Enc()
+
+    def static_args(y):
+        a = L.args(y)
+        a.scratch = q.Buffer()
+        return a
+
+    q.encode_moe_decode_static(e, static_args(y_eager))  # warm-up
+    e.wait()
+    y_eager.copy_(y0)
+    torch.cuda.synchronize()
+    free_before = torch.cuda.mem_get_info()[0]
+    q.encode_moe_decode_static(e, static_args(y_eager))
+    e.wait()
+    assert torch.cuda.mem_get_info()[0] == free_before
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        q.encode_moe_decode_static(q.Enc(torch.cuda.current_stream()), static_args(y_graph))
+    for rep in range(4):
+        y_graph.copy_(y0)
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(y_graph, y_eager), f"replay {rep} differs from the eager result"
+        _ = (y0 * 2).sum().item()  # eager work between the replays
 
 
 def test_static_scratch_limit(dev):
