@@ -55,7 +55,7 @@ __global__ __launch_bounds__(1024) void bw_probe_kernel(const uint4* __restrict_
 namespace {
 
 // Launch shape of the decode matvec. units = cols / UNIT columns-slices per row; a wave covers 64 * iters of them.
-struct MvShape { int iters, ks, rw, rpw, unit; };
+struct MvShape { int iters, ks, rw, rpw, unit; int per_cu = 1; };  // per_cu: persistent workgroups per CU (mv_tok_kernel)
 
 int mv_unit(int t) { return msq_type_block_elems(t) == 1 ? 8 : 32; }
 
@@ -153,9 +153,13 @@ int launch_mv(hipStream_t st, const MvShape& s, MvArgs& a) {
   return MSQ_OK;
 }
 
+int env_knob_early(const char* name, int dflt) {
+  const char* v = getenv(name);
+  return v && *v ? atoi(v) : dflt;
+}
 // Launch shape of the small-N matvec: workgroups of at most 8 waves (the kernel keeps T activation slices per lane
 // and is built for 512 threads), one or two units per lane.
-bool mv_tok_shape(int t, int rows, int cols, int groups, int token_groups, const MsqMvCfg* cfg, MvShape* s) {
+bool mv_tok_shape(int t, int rows, int cols, int groups, int n, int token_groups, const MsqMvCfg* cfg, MvShape* s) {
   const int unit = mv_unit(t);
   const int units = cols / unit;
   int iters = 1;
@@ -171,7 +175,17 @@ bool mv_tok_shape(int t, int rows, int cols, int groups, int token_groups, const
   if (rw * ks > 8) return false;
   // rows per wave per tile: one workgroup per CU, one tile each, is what measures fastest (a wave prefetches along its
   // run of rows; every tile ends in a workgroup-wide reduction)
-  const long wgs = std::max(1, device_info().cus / token_groups);
+  // One token, a matrix without a codebook table that is large (48 MB: the launch is bound by the bytes a CU keeps in
+  // flight, and a wave still walks a long run of rows) or dense and at least 8 MB (nothing to decode): two workgroups
+  // per CU. Measured, one / two workgroups: Q6_K 129280x5120 165 / 132 us, Q6_K 25600x6144 43.6 / 29.9, F16 5120x5120
+  // 13.7 / 11.2, BF16 4096x1280 6.75 / 5.2; the block formats between 5 and 35 MB lose up to 1.5 us with two.
+  const bool table = t == MSQ_IQ1_S || t == MSQ_IQ2_XXS;
+  static const int env_wgs = env_knob_early("MSQ_MV_WGS", 0);
+  const bool free_shape = !(cfg && (cfg->nr > 0 || cfg->rsg > 0 || cfg->ks > 0));
+  const double bytes = (double)msq_type_row_bytes(t, cols) * rows;
+  const bool two = !table && (bytes >= 48e6 || (unit == 8 && bytes >= 8e6));
+  const int per_cu = (n == 1 && free_shape) ? (env_wgs > 0 ? env_wgs : two ? 2 : 1) : 1;
+  const long wgs = std::max(1, per_cu * device_info().cus / token_groups);
   int rpw = (int)std::min<long>(32, std::max<long>(1, (rows + wgs * rw - 1) / (wgs * rw)));
   if (cfg && cfg->nr > 0) rpw = std::min(cfg->nr, 64);
   const int rpg = rows / groups;
@@ -180,7 +194,7 @@ bool mv_tok_shape(int t, int rows, int cols, int groups, int token_groups, const
     while (rw > 1 && rpg % (rw * rpw)) rw /= 2;
     if (rpg % (rw * rpw)) return false;
   }
-  *s = {iters, ks, rw, rpw, unit};
+  *s = {iters, ks, rw, rpw, unit, per_cu};
   return true;
 }
 
@@ -224,8 +238,9 @@ int launch_mv_tok(hipStream_t st, const MvShape& s, MvTokArgs& ta) {
       return MSQ_OK;
     }
   }
-  // persistent workgroups, one per CU over all token groups
-  const int gx = (int)std::min<long>(a.ntiles, std::max(1, device_info().cus / gy));
+  // persistent workgroups, one per CU over all token groups (two for a large matrix: MvShape::per_cu)
+  const int per_cu = (T == 1 && !a.norm_w && (lds + kStaticLds<D>) * s.per_cu <= (size_t)kMaxLds) ? s.per_cu : 1;
+  const int gx = (int)std::min<long>(a.ntiles, std::max(1, per_cu * device_info().cus / gy));
   const dim3 grid((unsigned)gx, (unsigned)gy);
   if (s.iters == 1) launch(mv_tok_kernel<D, 1, T>, grid);
   else if constexpr (D::UNIT == 8) launch(mv_tok_kernel<D, 2, T>, grid);
@@ -290,7 +305,7 @@ int matvec_tok(hipStream_t st, int t, const uint8_t* W, int rows, int cols, cons
   // tokens per pass over the weights: one, two, four or eight (Q8_0 keeps fp32 activations, 32 registers per token: four at most)
   const int T = n <= 2 ? n : (t == MSQ_Q8_0 || n <= 4) ? 4 : 8;
   MvShape s;
-  if (!mv_tok_shape(t, rows, cols, groups, (n + T - 1) / T, cfg, &s)) return MSQ_ERR_UNSUPPORTED;
+  if (!mv_tok_shape(t, rows, cols, groups, n, (n + T - 1) / T, cfg, &s)) return MSQ_ERR_UNSUPPORTED;
   if (n == 1 && !tok_serves_single(t, rows, cols, s, cfg)) return MSQ_ERR_UNSUPPORTED;
   MvTokArgs ta{};
   MvArgs& a = ta.m;
@@ -334,7 +349,7 @@ int msq_matvec_cfg(int t, int rows, int cols, MsqMvCfg* out) {
   if (!mv_type_ok(t) || rows < 1 || cols < 1 || cols % mv_col_multiple(t)) return unsupported("matvec_cfg", t, rows, cols);
   MsqMvCfg env;
   const MsqMvCfg* cfg = effective_cfg(nullptr, false, &env);
-  const bool tok = mv_tok_shape(t, rows, cols, 1, 1, cfg, &s) && tok_serves_single(t, rows, cols, s, cfg);  // as msq_matvec decides
+  const bool tok = mv_tok_shape(t, rows, cols, 1, 1, 1, cfg, &s) && tok_serves_single(t, rows, cols, s, cfg);  // as msq_matvec decides
   if (!tok && !mv_shape(t, rows, cols, 1, cfg, &s)) return unsupported("matvec_cfg", t, rows, cols);
   out->nr = s.rpw; out->rsg = s.rw; out->ks = s.ks;
   return MSQ_OK;

@@ -390,6 +390,9 @@ __global__ __launch_bounds__(512) void mv_tok_kernel(const uint8_t* W_, uint32_t
     // Four rows in flight pay for the codebook formats at one token (a row slice is 8 bytes per lane: IQ1_S 4096x7168
     // 8.5 -> 7.5 us); the others move 18 to 34 bytes per lane and row, and the rows repeated at the end of a run cost
     // them more than the deeper ring gains (Q8_0 4096x4096 8.4 -> 9.8 us, Q6_K 1536x7168 6.2 -> 7.8 us).
+    // Large matrices are bound by the bytes a CU keeps in flight (two rows per wave of six to eight waves: about 20 KB,
+    // half of what the memory system needs at its latency); there a second workgroup per CU (mv_tok_shape) does more
+    // than a deeper ring (Q6_K 129280x5120: 165 us as it was, 145 with four rows in flight, 132 with two workgroups).
     constexpr int NR = (T == 1 && requires { D::STAGES; }) ? 4 : 1;
     typename D::Raw ring[NR][ITERS];
 #pragma unroll
