@@ -16,6 +16,7 @@
 
 #include "msq_device.cuh"
 #include "msq_iq1s.cuh"
+#include "msq_iq2xxsq.cuh"
 
 namespace msq {
 
@@ -86,6 +87,10 @@ __device__ __forceinline__ float swiglu(float g, float u, float w) {  // quant_m
   u = fminf(fmaxf(u, -10.f), 10.f);
   return g / (1.f + expf(-g)) * u * w;
 }
+
+// the register batch in which a decoder with quantized activations holds its table items between request and store
+template <class D> struct TblRegsOf { struct type {}; };
+template <class D> requires requires { typename D::TblRegs; } struct TblRegsOf<D> { using type = typename D::TblRegs; };
 
 // Rows a wave keeps in flight per prefetch group: as many as fit about 24 registers of raw block bytes per buffer.
 template <class D>
@@ -255,7 +260,7 @@ __device__ __forceinline__ void moe_gu_run_ring(const MoeArgs& a, const uint64_t
   bool first = true;
   // The loads of the prologue (grid items, activations) need nothing but kernel arguments: they are requested before
   // the expert addresses are looked up, and stored to LDS after the first weight rows have been requested.
-  [[maybe_unused]] DecIQ1SQ::TblRegs tr;
+  [[maybe_unused]] typename TblRegsOf<D>::type tr;
   [[maybe_unused]] XqBatch<2> xb;
   if constexpr (requires { D::QUANT_X; }) {
     tr = D::issue_tables(tid, blockDim.x);

@@ -15,9 +15,9 @@ REPORT = os.path.join(os.path.dirname(__file__), "..", "macseek_amd", "libmsq.ke
 NO_SCRATCH = [
     "13mv_tok_kernel",                                              # decode matvec and small-N matvec, every format
     "14mv_ring_kernel",
-    "13moe_gu_kernelINS_8DecIQ1SQENS_9DecIQ2XXS",                   # BASELINE configs[2]
+    "13moe_gu_kernelINS_8DecIQ1SQENS_10DecIQ2XXSQ",                   # BASELINE configs[2]
     "15moe_down_kernelINS_7DecIQ1SENS_9DecIQ2XXSELi768",
-    "13moe_gu_kernelINS_9DecIQ2XXSES1_",                            # IQ2_XXS routed + IQ2_XXS shared
+    "13moe_gu_kernelINS_10DecIQ2XXSQES1_",                            # IQ2_XXS routed + IQ2_XXS shared
     "19moe_pf_block_kernel",                                        # prefill grouped GEMM, BASELINE configs[3]
     "15mm_fused_kernel", "16mm_reduce_kernel",                      # fused prefill matmul
     "19router_fused_kernel",
