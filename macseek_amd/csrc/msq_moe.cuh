@@ -17,6 +17,7 @@
 #include "msq_device.cuh"
 #include "msq_iq1s.cuh"
 #include "msq_iq2xxsq.cuh"
+#include "msq_q6kq.cuh"
 
 namespace msq {
 
@@ -170,15 +171,26 @@ __device__ __forceinline__ void moe_gu_run_direct(const MoeArgs& a, const uint64
       }
     }
     if (first) {  // tables and activations arrive while the first weight rows are in flight
-      const CopyJob jobs[3] = {tbl_job_of<D>(0, 0u, true), tbl_job_of<D>(1, 0u, true),
-                               {(const uint4*)a.x, (uint32_t)(smem - tbl) + a.xs_off, a.stage_x ? a.dim / 4u : 0u, 3u}};
-      copy_jobs<4>(tbl, jobs, tid, blockDim.x);
-      if (a.stage_x) {
-        __syncthreads();
-        xr = D::load_x(XLds{(const float*)(smem + a.xs_off)}, unit);
+      if constexpr (requires { D::QUANT_X; }) {  // quantized activations (no table)
+        if (a.stage_x) {
+          stage_xq<2>(smem + a.xs_off, a.x, a.dim, tid, blockDim.x);
+          __syncthreads();
+          xr = D::load_x(XQLds{smem + a.xs_off}, unit);
+        } else {
+          xr = D::load_x(a.x, unit);
+          __syncthreads();
+        }
       } else {
-        xr = D::load_x(a.x, unit);
-        __syncthreads();
+        const CopyJob jobs[3] = {tbl_job_of<D>(0, 0u, true), tbl_job_of<D>(1, 0u, true),
+                                 {(const uint4*)a.x, (uint32_t)(smem - tbl) + a.xs_off, a.stage_x ? a.dim / 4u : 0u, 3u}};
+        copy_jobs<4>(tbl, jobs, tid, blockDim.x);
+        if (a.stage_x) {
+          __syncthreads();
+          xr = D::load_x(XLds{(const float*)(smem + a.xs_off)}, unit);
+        } else {
+          xr = D::load_x(a.x, unit);
+          __syncthreads();
+        }
       }
       first = false;
     }

@@ -81,6 +81,7 @@ size_t place_x(MoeArgs& a, size_t lds, uint32_t cols_r, uint32_t cols_s) {
 template <class D> struct DownDec { using T = D; };
 template <> struct DownDec<DecIQ1SQ> { using T = DecIQ1S; };
 template <> struct DownDec<DecIQ2XXSQ> { using T = DecIQ2XXS; };
+template <> struct DownDec<DecQ6KQ> { using T = DecQ6K; };
 // dispatch over (routed type, shared type); cols_r / cols_s: activations the routed / shared part stages (0 = none)
 // returns MSQ_OK, a launch's error, or MSQ_ERR_UNSUPPORTED (without a message) when no kernel serves the type pair
 template <bool DOWN>
@@ -97,11 +98,11 @@ int dispatch(int tr, int ts, dim3 g, dim3 b, size_t part_bytes, uint32_t cols_r,
       return launch_gu_t<DRT, DST>(g, b, lds, st, a);                                             \
     }                                                                                             \
   }
-  MSQ_MOE_CASE(MSQ_IQ1_S, DecIQ1SQ, MSQ_Q6_K, DecQ6K)
+  MSQ_MOE_CASE(MSQ_IQ1_S, DecIQ1SQ, MSQ_Q6_K, DecQ6KQ)
   MSQ_MOE_CASE(MSQ_IQ1_S, DecIQ1SQ, MSQ_Q8_0, DecQ8_0)
   MSQ_MOE_CASE(MSQ_IQ1_S, DecIQ1SQ, MSQ_IQ2_XXS, DecIQ2XXSQ)
   MSQ_MOE_CASE(MSQ_IQ1_S, DecIQ1SQ, MSQ_IQ1_S, DecIQ1SQ)
-  MSQ_MOE_CASE(MSQ_IQ2_XXS, DecIQ2XXSQ, MSQ_Q6_K, DecQ6K)
+  MSQ_MOE_CASE(MSQ_IQ2_XXS, DecIQ2XXSQ, MSQ_Q6_K, DecQ6KQ)
   MSQ_MOE_CASE(MSQ_IQ2_XXS, DecIQ2XXSQ, MSQ_Q8_0, DecQ8_0)
   MSQ_MOE_CASE(MSQ_IQ2_XXS, DecIQ2XXSQ, MSQ_IQ2_XXS, DecIQ2XXSQ)
   MSQ_MOE_CASE(MSQ_IQ2_XXS, DecIQ2XXSQ, MSQ_IQ1_S, DecIQ1SQ)

@@ -96,4 +96,4 @@ def test_placed_experts_run_the_moe_layer(dev, tmp_path):
     ry, ymag, _, _ = O.moe_decode(O.IQ1_S, O.IQ2_XXS, O.Q6_K, 6, True, dim, inter, Gs, Us, Ds, w, x, y0)
     err = float(np.max(np.abs(yd.cpu().numpy() - ry) / (ymag + 1e-12)))
     print(f"  MoE layer on experts placed from a GGUF file: chain error {err:.2e}")
-    assert err <= 3e-4  # whole chain, fp16-staged Q6_K shared expert on 1024-column rows (measured 2.0e-4)
+    assert err <= 1.5e-4  # whole chain on the smallest layer shape, 512-column rows and 256-column h rows (measured 8.7e-5)

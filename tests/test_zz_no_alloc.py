@@ -7,7 +7,7 @@ import torch
 
 import oracle as O
 from macseek_amd import quant as q
-from test_moe_decode_gpu import Layer
+from test_moe_decode_gpu import SMALL_SHAPE_CHAIN_TOL, Layer
 from util import up
 
 pytestmark = pytest.mark.gpu
@@ -30,12 +30,12 @@ def test_static_scratch_entry_point_matches_caller_scratch(dev):
     big = Layer(O.IQ1_S, O.IQ1_S, O.IQ2_XXS, 6, True, 7168, 2048)
     y_ref, y_static = run_both(big)
     assert torch.equal(y_ref, y_static)
-    big.check(y_static, None, "static scratch, 7168/2048", chain_tol=1.5e-4)
+    big.check(y_static, None, "static scratch, 7168/2048")
     # second call, smaller layer: the array still holds the first call's h rows beyond the new layer's
     small = Layer(O.IQ1_S, O.IQ2_XXS, O.Q8_0, 2, True, 512, 256, seed=300)
     y_ref, y_static = run_both(small)
     assert torch.equal(y_ref, y_static)
-    small.check(y_static, None, "static scratch, 512/256")
+    small.check(y_static, None, "static scratch, 512/256", chain_tol=SMALL_SHAPE_CHAIN_TOL)
     # and the first shape again
     y_ref, y_static = run_both(big)
     assert torch.equal(y_ref, y_static)
