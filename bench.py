@@ -577,6 +577,46 @@ def bench_issue_probe(torch, args):
             "roofline": None, "cpu_baseline": None, "pct_of_hbm_peak": None}
 
 
+def bench_handover_probe(torch, args):
+    """What a device-wide hand-over inside one launch costs (libmsq_probe.so: handover_probe_kernel), the step a
+    single-launch MoE layer needs between gate/up and down: per workgroup, microseconds from its start until its h
+    stores are acknowledged, its arrival is counted, all 256 arrivals are seen, and all of h (28 KB) has been read back
+    with device-scope loads; flat counter and two-level (per-XCD) counter, median and slowest workgroup over 50 launches."""
+    from macseek_amd import build as B
+    P = C.CDLL(B.PROBE_OUT)
+    P.msq_probe_handover.restype = C.c_int
+    P.msq_probe_handover.argtypes = [C.c_void_p, C.c_int, C.c_void_p, C.c_uint32, C.c_int, C.c_uint32, C.c_uint32, C.c_void_p, C.c_void_p]
+    dev = torch.device("cuda:0")
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    h_words = 7 * 2048 // 2  # seven h rows of 2048 values as fp16
+    h = torch.zeros(h_words, dtype=torch.int32, device=dev)
+    out = torch.zeros(5 * cus, dtype=torch.int64, device=dev)
+    sink = torch.zeros(cus, dtype=torch.int32, device=dev)
+    res = {}
+    for mode, name in ((0, "flat_counter"), (1, "two_level_counter")):
+        rows = []
+        for epoch in range(60):
+            rc = P.msq_probe_handover(C.c_void_p(torch.cuda.current_stream().cuda_stream), cus, C.c_void_p(h.data_ptr()), h_words, mode, epoch,
+                                      20000, C.c_void_p(out.data_ptr()), C.c_void_p(sink.data_ptr()))
+            if rc != 0:
+                raise RuntimeError("msq_probe_handover failed: %d" % rc)
+            torch.cuda.synchronize()
+            o = out.cpu().numpy().reshape(cus, 5)
+            if not o[:, 4].all():
+                raise RuntimeError("hand-over probe: a workgroup gave up waiting (mode %s, launch %d)" % (name, epoch))
+            if epoch >= 10:
+                rows.append(o[:, :4].astype(np.float64) / 100.0)  # 100 MHz ticks -> us
+        a = np.stack(rows)  # [launch][workgroup][stamp]
+        med, worst = np.median(np.median(a, axis=1), axis=0), np.median(np.max(a, axis=1), axis=0)
+        res[name] = {"median_wg_us": {"stores_acknowledged": med[0], "arrival_counted": med[1], "all_arrived": med[2], "h_read_back": med[3]},
+                     "slowest_wg_us": {"stores_acknowledged": worst[0], "arrival_counted": worst[1], "all_arrived": worst[2], "h_read_back": worst[3]}}
+    v = res["two_level_counter"]["slowest_wg_us"]["h_read_back"]
+    return {"value": v, "unit": "us", "ms_per_step": v * 1e-3, "dtype": "device-scope stores, atomics and loads",
+            "config": {"workload": "in-kernel device-wide hand-over of h (28 KB) among %d workgroups, one per CU; stamps per workgroup from its own start" % cus,
+                       "results": res},
+            "roofline": None, "cpu_baseline": None, "pct_of_hbm_peak": None}
+
+
 def bench_copy_calibration(torch, args):
     """A device-to-device copy of known size (1 GiB read, 1 GiB written per launch): the reference that the FETCH_SIZE /
     WRITE_SIZE counters of a profiling run are scaled by."""
@@ -850,7 +890,7 @@ def main():
     ap.add_argument("--steps", type=int, default=500)
     ap.add_argument("--warmup", type=int, default=100)
     ap.add_argument("--workload", default="moe_decode",
-                    choices=["moe_decode", "moe_prefill", "matvec_iq1s", "matvec_iq2xxs", "q8_0", "matvec_n", "router", "matmul", "stream", "copy_calibration", "issue_probe", "table"])
+                    choices=["moe_decode", "moe_prefill", "matvec_iq1s", "matvec_iq2xxs", "q8_0", "matvec_n", "router", "matmul", "stream", "copy_calibration", "issue_probe", "handover_probe", "table"])
     ap.add_argument("--one-stream", action="store_true",
                     help="profiling runs: msq_moe_prefill keeps its launches on one stream (MSQ_MOEP_ONE_STREAM=1), so that "
                          "per-kernel durations and counters are not those of two kernels sharing the device")
@@ -895,6 +935,8 @@ def main():
         r = bench_copy_calibration(torch, args)
     elif args.workload == "issue_probe":
         r = bench_issue_probe(torch, args)
+    elif args.workload == "handover_probe":
+        r = bench_handover_probe(torch, args)
     elif args.workload == "router":
         r = bench_router(torch, args)
     elif args.workload == "table":
@@ -907,7 +949,7 @@ def main():
         r = bench_matvec(torch, args, q.QType.IQ2_XXS, 4096, 7168, 0.01, "BASELINE configs[1]: single-expert decode matvec IQ2_XXS 4096x7168, batch 1")
     else:
         r = bench_matvec(torch, args, q.QType.Q8_0, 4096, 4096, 0.02, "BASELINE configs[0]: Q8_0 4096x4096 matvec")
-    out = {"metric": METRIC, "value": r["value"], "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+    out = {"metric": METRIC, "value": r["value"], "unit": r.get("unit", "GB/s"), "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
            "ms_per_step": r["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
            "dtype": r["dtype"], "data": "synthetic", "config": r["config"], "roofline": r["roofline"],
            "cpu_baseline": r["cpu_baseline"], "pct_of_hbm_peak": r["pct_of_hbm_peak"]}

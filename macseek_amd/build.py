@@ -10,7 +10,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OUT = os.path.join(HERE, "libmsq.so")
 # the benchmark's instruction-issue probe: a shared object of its own, no part of the library
-PROBE_SRC = os.path.join(CSRC, "probe", "issue_probe.hip")
+PROBE_SRC = [os.path.join(CSRC, "probe", "issue_probe.hip"), os.path.join(CSRC, "probe", "handover_probe.hip")]
 PROBE_OUT = os.path.join(HERE, "libmsq_probe.so")
 OBJDIR = os.path.join(HERE, "csrc", "build")
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
@@ -81,7 +81,7 @@ def build(verbose=True):
         raise RuntimeError("link failed:\n" + r.stdout)
     with open(REPORT, "w") as f:
         json.dump(report, f, indent=1, sort_keys=True)
-    r = subprocess.run([HIPCC] + FLAGS + ["-shared", PROBE_SRC, "-o", PROBE_OUT], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    r = subprocess.run([HIPCC] + FLAGS + ["-shared"] + PROBE_SRC + ["-o", PROBE_OUT], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     if r.returncode != 0:
         raise RuntimeError("hipcc failed for %s:\n%s" % (PROBE_SRC, r.stdout))
     if verbose:
