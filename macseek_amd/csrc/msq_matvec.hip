@@ -220,8 +220,9 @@ int launch_mv_tok(hipStream_t st, const MvShape& s, MvTokArgs& ta) {
   a.ntiles = (a.rows + tile_rows - 1) / tile_rows;
   size_t lds = (size_t)tile_rows * s.ks * 4 * T * 4;  // dynamic LDS: partial sums, staged activations (the table is static)
   const int gy = ((int)ta.n + T - 1) / T;
-  if (D::STAGE_X || a.norm_w) {
-    if (!place_x_row(a, lds, tok_round<D, T>(), kMaxLds - kStaticLds<D>, true)) return MSQ_ERR_UNSUPPORTED;  // one workgroup per CU: all of its LDS
+  if (tok_stages_x<D, T>() || a.norm_w) {
+    // one workgroup per CU: all of its LDS (decoders that stage only in the four-token kernel read directly when a round does not fit)
+    if (!place_x_row(a, lds, tok_round<D, T>(), kMaxLds - kStaticLds<D>, D::STAGE_X)) return MSQ_ERR_UNSUPPORTED;
   }
   auto launch = [&](auto kernel, dim3 grid) {
     allow_large_lds(kernel, lds);
@@ -303,7 +304,12 @@ int matvec_tok(hipStream_t st, int t, const uint8_t* W, int rows, int cols, cons
   MsqMvCfg several;
   if (n > 1) cfg = effective_cfg(cfg, true, &several);
   // tokens per pass over the weights: one, two, four or eight (Q8_0 keeps fp32 activations, 32 registers per token: four at most)
-  const int T = n <= 2 ? n : (t == MSQ_Q8_0 || n <= 4) ? 4 : 8;
+  // ... and groups of four also for more tokens over a small matrix (below 8 MB): every workgroup then fetches four
+  // tokens' activations instead of eight, and the second group finds the weights in the caches (Q5_K 512x7168 at 8 / 16
+  // tokens: 10.4 / 11.1 -> 7.3 / 8.8 us; BF16 384x7168 6.1 / 6.7 -> 5.2 / 6.2; the 9 MB and 16 MB matrices lose at 16)
+  static const int env_t = env_knob("MSQ_MVN_T");
+  const bool small = (double)msq_type_row_bytes(t, cols) * rows < 8e6;
+  const int T = n <= 2 ? n : (t == MSQ_Q8_0 || n <= 4 || env_t == 4 || (small && env_t != 8)) ? 4 : 8;
   MvShape s;
   if (!mv_tok_shape(t, rows, cols, groups, n, (n + T - 1) / T, cfg, &s)) return MSQ_ERR_UNSUPPORTED;
   if (n == 1 && !tok_serves_single(t, rows, cols, s, cfg)) return MSQ_ERR_UNSUPPORTED;

@@ -325,13 +325,20 @@ constexpr int tok_round() {
   return T < g ? T : g;
 }
 
+// Whether the T-token kernel of decoder D takes its activations through LDS: the decoders with STAGE_X always; the other
+// block formats in the four-token instantiation. Their lane slices are short runs (Q6_K: four runs of 32 bytes per
+// token), read straight from device memory for one or two tokens; at four tokens one staged round is faster (Q6_K
+// 1536x7168 8.9 -> 8.5 us, Q5_K 512x7168 7.0 -> 6.5), at eight the two rounds cost more than they save (11.3 -> 12.7).
+template <class D, int T>
+constexpr bool tok_stages_x() { return D::STAGE_X || (T == 4 && D::UNIT == 32); }
+
 // Decoders with STAGE_X take the activations through LDS (contiguous loads, tok_round() tokens per round); with the
 // others every lane reads its slices from device memory, all T tokens' loads in flight at once.
 template <class D, int ITERS, int T, bool NORM = false>
 __global__ __launch_bounds__(512) void mv_tok_kernel(const uint8_t* W_, uint32_t rows_, uint32_t row_bytes_, uint32_t units_, uint32_t ks_,
                                                      uint32_t rpw_, uint32_t ntiles_, uint32_t rows_per_group_, const float* x_,
                                                      uint32_t cols_, const MvTokArgs ta) {
-  constexpr bool STAGE = D::STAGE_X;
+  constexpr bool STAGE = tok_stages_x<D, T>();
   // What the first loads need comes as leading arguments (W_ .. cols_: the fields of the same names in ta.m, delivered
   // in scalar registers with the wave when the file is built with kernel-argument preload) and is used under those
   // names below; the rest is read from the argument block.
@@ -426,6 +433,9 @@ __global__ __launch_bounds__(512) void mv_tok_kernel(const uint8_t* W_, uint32_t
 #pragma unroll
           for (int i = 0; i < ITERS; i++) xr[t][i] = D::load_x(XLds{xs}, unit[i]);
         } else if constexpr (!STAGE) {
+#pragma unroll
+          for (int i = 0; i < ITERS; i++) xr[t][i] = D::load_x(x_of(t), unit[i]);
+        } else if (!D::STAGE_X && !a.stage_x) {  // (rows too long for a round of G in LDS: read directly, as for few tokens)
 #pragma unroll
           for (int i = 0; i < ITERS; i++) xr[t][i] = D::load_x(x_of(t), unit[i]);
         } else {
