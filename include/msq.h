@@ -7,9 +7,13 @@
  *     ordered by the stream, so the reference's explicit Enc::barrier() between them has no counterpart.
  *   - weights are raw GGUF block rows: an [in -> out] matrix is rows = out rows of cols = in elements
  *     (quant.hpp:4); weight bases need 4-byte alignment only, activations / outputs 16-byte alignment
- *     (docs/modules/quant.md:27-30). Activations must be finite and inside the fp16 range, |x| <= 65504 (the block
- *     formats stage them as fp16 pairs, as the reference does for its n > 1 paths; larger values turn into
- *     infinities). MoE routing weights up to 5 keep the down projection's inputs inside that range.
+ *     (docs/modules/quant.md:27-30). Activations must be finite. One token (msq_matvec, msq_matvec_rmsnorm, gate/up of
+ *     the one-token MoE layer) is F32-activation arithmetic like the reference's: the block formats multiply integer
+ *     payloads with activations rounded at 2^-16 of the largest value of their run of 8 to 32 columns (no range limit),
+ *     Q8_0 and the dense types keep fp32. Several tokens (msq_matvec_n from n = 2, the prefill paths) and the down
+ *     projection of the MoE layer stage activations as fp16 pairs, as the reference does for its n > 1 paths: there
+ *     |x| <= 65504 (larger values turn into infinities); MoE routing weights up to 5 keep the down projection's
+ *     inputs inside that range.
  *   - all buffers are caller-owned device memory; MsqBuffer mirrors ms::Buffer {buf, off, size}
  *     (src/core/metal.hpp:11-18).
  *   - misuse is reported, not aborted: functions return 0 on success or a negative MSQ_ERR_* code and leave a
@@ -99,8 +103,9 @@ int msq_rmsnorm(void* stream, const MsqBuffer* x, const MsqBuffer* w, const MsqB
 /* reference: ms::q::encode_matvec_n (quant.hpp:32-35, quant.mm:129-156).
  * Y[n x rows] (+)= X[n x cols] . W^T for n in 1..16 (one weight read serves all n tokens). X row stride is
  * cols * groups, Y row stride is rows. n == 1 is exactly msq_matvec. For n >= 2, rows of up to 16384 columns (dense
- * types: 8192) run in a dot-product kernel that stages activations like msq_matvec does (fp16 pairs for the K / IQ
- * formats, fp32 for Q8_0 and the dense types) and decodes each weight once for up to eight tokens. Wider rows, and
+ * types: 8192) run in a dot-product kernel that stages activations as fp16 pairs for the K / IQ formats (the
+ * reference's numerics from two tokens on), fp32 for Q8_0 and the dense types, and decodes each weight once for up to
+ * eight tokens. Wider rows, and
  * more than eight tokens over a large IQ4_NL / Q8_0 / F16 / BF16 matrix, run on the matrix cores with activations
  * rounded to fp16 (BF16 weights: split into two bf16 terms) and exact weights; the reference rounds activations to
  * fp16 the same way and, from n >= 8, weights too (quant.mm:133-137). Wide F32 matrices, and wide block-diagonal

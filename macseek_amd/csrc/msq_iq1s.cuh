@@ -175,9 +175,10 @@ struct DecIQ1SQ {
     return {{a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w}, {c.x, c.y, c.z, c.w, d.x, d.y, d.z, d.w},
             __builtin_bit_cast(float, x.p[u * kXqWords + 16])};
   }
-  // the same quantization by one lane on its own (rows too long to stage)
-  __device__ static X load_x(const float* x, uint32_t u) {
-    const float4* p = (const float4*)(x + 32u * u);
+  // the same quantization by one lane on its own (rows too long to stage; S: plain memory or the padded LDS rows of XLds)
+  template <class S>
+  __device__ static X load_x(S x, uint32_t u) {
+    const float4* p = (const float4*)xat(x, 32u * u);
     float4 v[8];
     float m = 0.f;
 #pragma unroll

@@ -77,7 +77,8 @@ struct DecIQ2XXSQ {
 
   // ---- activations: as DecIQ1SQ
   __device__ static X load_x(XQLds x, uint32_t u) { return DecIQ1SQ::load_x(x, u); }
-  __device__ static X load_x(const float* x, uint32_t u) { return DecIQ1SQ::load_x(x, u); }
+  template <class S>
+  __device__ static X load_x(S x, uint32_t u) { return DecIQ1SQ::load_x(x, u); }
 
   // ---- block bytes
   struct Off { uint32_t a, d; };
@@ -126,6 +127,16 @@ struct DecIQ2XXSQ {
       hi = __builtin_amdgcn_sdot4((int)w1, (int)x.hi[2 * l + 1], hi, false);
     }
     return (float)((hi << 8) + lo);  // |sum| < 2^25: the conversion rounds at 2^-24 of it
+  }
+  template <class P>
+  __device__ static Raw load(P row, uint32_t u) {
+    const P b = row + (u >> 3) * 66u;
+    const u64_a2 a = ld64(b + 2 + 8 * (u & 7u));
+    return {a.x, a.y, __builtin_bit_cast(_Float16, (uint16_t)ld16(b))};
+  }
+  __device__ static float dot(const Raw& r, const X& x, const uint32_t* lds) {
+    const Look k0 = lookup(r, 0, lds), k1 = lookup(r, 1, lds);
+    return partial(r, k1, x, 1, partial(r, k0, x, 0, 0.f));
   }
   __device__ static float partial(const Raw& r, const Look& k, const X& x, int stage, float acc) {
     acc += stage_sum(k, x, stage);

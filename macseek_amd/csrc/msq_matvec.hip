@@ -7,6 +7,7 @@
 #include "msq_deq.cuh"
 #include "msq_host.h"
 #include "msq_mv.cuh"
+#include "msq_mvq.cuh"
 
 namespace msq {
 
@@ -252,6 +253,15 @@ int launch_mv_tok(hipStream_t st, const MvShape& s, MvTokArgs& ta) {
 
 template <int T>
 int launch_mv_tok_t(hipStream_t st, int t, const MvShape& s, MvTokArgs& ta) {
+  if constexpr (T == 1) {  // one token: the block formats' integer decoders (msq_mvq.cuh)
+    switch (t) {
+      case MSQ_IQ1_S: return launch_mv_tok<DecIQ1SM, 1>(st, s, ta);
+      case MSQ_IQ2_XXS: return launch_mv_tok<DecIQ2XXSM, 1>(st, s, ta);
+      case MSQ_IQ4_NL: return launch_mv_tok<DecIQ4NLQ, 1>(st, s, ta);
+      case MSQ_Q6_K: return launch_mv_tok<DecQ6KQ, 1>(st, s, ta);
+      case MSQ_Q5_K: return launch_mv_tok<DecQ5KQ, 1>(st, s, ta);
+    }
+  }
   switch (t) {
     case MSQ_IQ1_S: return launch_mv_tok<DecIQ1S, T>(st, s, ta);
     case MSQ_IQ2_XXS: return launch_mv_tok<DecIQ2XXS, T>(st, s, ta);
@@ -388,12 +398,12 @@ static int matvec_impl(void* stream, const char* what, int t, const MsqBuffer* W
   a.norm_w = norm_w; a.eps = eps;
   int rc = MSQ_ERR_UNSUPPORTED;
   switch (t) {
-    case MSQ_IQ1_S: rc = launch_mv<DecIQ1S>(st, s, a); break;
-    case MSQ_IQ2_XXS: rc = launch_mv<DecIQ2XXS>(st, s, a); break;
+    case MSQ_IQ1_S: rc = launch_mv<DecIQ1SM>(st, s, a); break;
+    case MSQ_IQ2_XXS: rc = launch_mv<DecIQ2XXSM>(st, s, a); break;
     case MSQ_Q8_0: rc = launch_mv<DecQ8_0>(st, s, a); break;
-    case MSQ_IQ4_NL: rc = launch_mv<DecIQ4NL>(st, s, a); break;
-    case MSQ_Q6_K: rc = launch_mv<DecQ6K>(st, s, a); break;
-    case MSQ_Q5_K: rc = launch_mv<DecQ5K>(st, s, a); break;
+    case MSQ_IQ4_NL: rc = launch_mv<DecIQ4NLQ>(st, s, a); break;
+    case MSQ_Q6_K: rc = launch_mv<DecQ6KQ>(st, s, a); break;
+    case MSQ_Q5_K: rc = launch_mv<DecQ5KQ>(st, s, a); break;
     case MSQ_F32: rc = launch_mv<DecDense<MSQ_F32>>(st, s, a); break;
     case MSQ_F16: rc = launch_mv<DecDense<MSQ_F16>>(st, s, a); break;
     case MSQ_BF16: rc = launch_mv<DecDense<MSQ_BF16>>(st, s, a); break;

@@ -18,7 +18,7 @@ namespace msq {
 
 struct DecQ6KQ {
   static constexpr int UNIT = 32, LDS_WORDS = 0;
-  static constexpr bool STAGE_X = true, QUANT_X = true;
+  static constexpr bool STAGE_X = false, QUANT_X = true;  // (STAGE_X: the decode matvec reads its short runs directly, as DecQ6K)
   // per run k: two words of low bytes, two of high bytes, the scale, and -32 * sum n
   struct X { uint32_t lo[8], hi[8]; float xs[4]; int m32sn[4]; };
   typedef DecQ6K::Raw Raw;
@@ -50,14 +50,16 @@ struct DecQ6KQ {
     }
     return r;
   }
-  // the same quantization by one lane on its own (rows too long to stage): one scale per run of eight columns
-  __device__ static X load_x(const float* x, uint32_t u) {
+  // the same quantization by one lane on its own (rows too long to stage; the decode matvec, from plain memory or the
+  // padded LDS rows of XLds): one scale per run of eight columns
+  template <class S>
+  __device__ static X load_x(S x, uint32_t u) {
     X r;
     const uint32_t j = u & 7u;
     const uint32_t base = 256u * (u >> 3) + 128u * (j >> 2) + 8u * (j & 3u);
 #pragma unroll
     for (int k = 0; k < 4; k++) {
-      const float4* p = (const float4*)(x + base + 32u * k);
+      const float4* p = (const float4*)xat(x, base + 32u * k);
       const float4 a = p[0], b = p[1];
       const float m = fmaxf(fmaxf(fmaxf(fabsf(a.x), fabsf(a.y)), fmaxf(fabsf(a.z), fabsf(a.w))),
                             fmaxf(fmaxf(fabsf(b.x), fabsf(b.y)), fmaxf(fabsf(b.z), fabsf(b.w))));

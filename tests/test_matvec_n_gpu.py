@@ -82,7 +82,11 @@ def test_matvec_n_vs_oracle(dev, t, rows, cols, groups, n, acc):
     # reference bounds: 2e-6 against the half-x reference for its F32-FMA kernel (n < 8), 1e-4 on its tile path (n >= 8),
     # 2e-4 against the F32 reference (tests/test_quant_matvec_n.mm:45-46). Here the tighter one is held at every n
     # (measured: at most 7.8e-7, Q5_K 37 x 256).
-    assert err_h <= 2e-6 and err_f <= 2e-4 and err_ns <= TOL_NORTH_STAR
+    # One token is the decode matvec: F32-activation arithmetic to the reference's 2e-5 (tests/test_quant_matvec.mm:42).
+    if n == 1:
+        assert err_f <= 2e-5 and err_ns <= TOL_NORTH_STAR
+    else:
+        assert err_h <= 2e-6 and err_f <= 2e-4 and err_ns <= TOL_NORTH_STAR
 
 
 def test_matvec_n_misuse_and_untouched_rows(dev):
