@@ -704,7 +704,7 @@ def bench_table(torch, args):
     projection shape of the reference plus BASELINE's configs[0], [1] and [4] shapes, one msq_matvec per step, weights
     rotated over >= 512 MiB of distinct copies so every launch streams from HBM. Per row: weight MB, us per launch,
     GB/s of algorithmic bytes (W + 4 cols + 4 rows), the fraction of the 8 TB/s roofline and of what a kernel that only
-    reads (msq_bw_probe, 1 GiB, same run) gets on this device. value = the Q8_0 4096x4096 row (configs[0])."""
+    reads (msq_bw_probe, 1 GiB, same run) gets on this device. value = the first row (Q8_0 4096x4096, configs[0], unless --only narrows the table)."""
     from macseek_amd import _lib, quant as q
     L = _lib.load()
     dev = torch.device("cuda:0")
@@ -730,6 +730,10 @@ def bench_table(torch, args):
         (T.F16, 5120, 5120, 1, "f16 synthetic"),
         (T.IQ1_S, 32768, 5120, 1, "big synthetic"), (T.IQ2_XXS, 32768, 5120, 1, "big synthetic"),
     ]
+    if args.only:
+        shapes = [r for r in shapes if args.only in "%s %s" % (q.type_name(r[0]), r[4])]
+        if not shapes:
+            raise SystemExit("bench.py: --only %r matches no row of the table" % args.only)
     pool = torch.randint(0, 256, (1 << 30,), dtype=torch.uint8, device=dev)  # raw bytes: timing only (as the reference's table)
     bw = stream_read_GBps(torch, 1 << 30, pool)
     rows_out = []
@@ -758,9 +762,9 @@ def bench_table(torch, args):
     for r in rows_out:
         print("%-8s %-20s %-16s %9.2f %8.2f %8.1f %7.1f %9.1f" % (r["type"], r["tensor"], r["shape"], r["MB"], r["us"], r["GBps"],
                                                                    100 * r["frac_of_8TBps"], r["pct_of_stream_read"]), file=sys.stderr)
-    return {"value": head["GBps"], "ms_per_step": head["us"] * 1e-3, "dtype": "f32 activations (Q8_0, dense) / f16-staged activations (block formats), f32 accumulate",
+    return {"value": head["GBps"], "ms_per_step": head["us"] * 1e-3, "dtype": "f32 activations (Q8_0, dense) / 16-bit block-fixed-point activations and exact integer sums (block formats), f32 accumulate",
             "config": {"workload": "decode matvec table: the reference's projection shapes + BASELINE configs[0], [1], [4]; one step = one msq_matvec of "
-                                   "the Q8_0 4096x4096 row", "stream_read_GBps_1GiB": bw, "rows": rows_out},
+                                   "the first row", "stream_read_GBps_1GiB": bw, "rows": rows_out},
             "roofline": {"bound": "hbm", "achieved": head["GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": head["GBps"] / HBM_PEAK_GBPS,
                          "traffic": None, "kernel": "decode matvec (mv_tok_kernel, mv_kernel or mv_ring_kernel by shape)", "avg_launch_us": head["us"],
                          "timing": "HIP event pair around back-to-back replays of a graph of >= 16 launches, >= 10 ms per region"},
@@ -894,6 +898,8 @@ def main():
     ap.add_argument("--one-stream", action="store_true",
                     help="profiling runs: msq_moe_prefill keeps its launches on one stream (MSQ_MOEP_ONE_STREAM=1), so that "
                          "per-kernel durations and counters are not those of two kernels sharing the device")
+    ap.add_argument("--only", default="",
+                    help="table workload: keep the rows whose 'type tensor' contains this text (profiling one matrix)")
     ap.add_argument("--gpu-only", action="store_true",
                     help="profiling runs: skip the CPU baseline leg and the prefill appendix of the default workload")
     args = ap.parse_args()

@@ -133,6 +133,24 @@ __device__ __forceinline__ u64_a2 buf_ld64(rsrc_t r, uint32_t voff, uint32_t sof
   return {(uint32_t)v[0], (uint32_t)v[1]};
 }
 
+__device__ __forceinline__ u128_a2 buf_ld128(rsrc_t r, uint32_t voff, uint32_t soff) {
+  const auto v = __builtin_amdgcn_raw_buffer_load_b128(r, (int)voff, (int)soff, 0);
+  return {(uint32_t)v[0], (uint32_t)v[1], (uint32_t)v[2], (uint32_t)v[3]};
+}
+// A weight row reached through a buffer descriptor, in the shape of a pointer for the decoders' load() functions
+// (p + bytes, ld16 .. ld128): rs covers a run of rows, soff is the row's byte offset in it -- wave-uniform, so it travels
+// in a scalar register -- and voff the lane's byte offset inside the row, a loop constant. A row's loads then cost no
+// vector arithmetic (a 64-bit pointer per lane costs a multiply-add and an addition per load and row).
+struct BufRow {
+  rsrc_t rs;
+  uint32_t soff, voff;
+  __device__ __forceinline__ BufRow operator+(uint32_t o) const { return {rs, soff, voff + o}; }
+};
+__device__ __forceinline__ uint32_t ld16(const BufRow& p) { return buf_ld16(p.rs, p.voff, p.soff); }
+__device__ __forceinline__ uint32_t ld32(const BufRow& p) { return buf_ld32(p.rs, p.voff, p.soff); }
+__device__ __forceinline__ u64_a2 ld64(const BufRow& p) { return buf_ld64(p.rs, p.voff, p.soff); }
+__device__ __forceinline__ u128_a2 ld128(const BufRow& p) { return buf_ld128(p.rs, p.voff, p.soff); }
+
 #define MSQ_LOADERS(AS)                                                                                               \
   __device__ __forceinline__ uint32_t ld8(const AS uint8_t* p) { return *p; }                                         \
   __device__ __forceinline__ uint32_t ld16(const AS uint8_t* p) { return *(const AS uint16_t*)p; }                    \

@@ -65,6 +65,13 @@ __device__ __forceinline__ void xq_quant4(float4 v, float mult, uint32_t& lo, ui
   lo = __builtin_amdgcn_perm(__builtin_bit_cast(uint32_t, p1), __builtin_bit_cast(uint32_t, p0), 0x06040200u);
   hi = __builtin_amdgcn_perm(q1, q0, 0x07050301u);
 }
+// first product of a v_dot4_i32_i8 chain: the three-operand form with a literal zero addend (the compiler's choice, the
+// two-operand accumulate form, needs an instruction to clear its accumulator first)
+__device__ __forceinline__ int sdot4z(uint32_t a, uint32_t b) {
+  int r;
+  asm("v_dot4_i32_i8 %0, %1, %2, 0" : "=v"(r) : "v"(a), "v"(b));
+  return r;
+}
 template <int CTRL>
 __device__ __forceinline__ float dpp_maxf(float v) {
   const int moved = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, false);

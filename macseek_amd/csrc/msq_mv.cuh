@@ -351,7 +351,9 @@ __global__ __launch_bounds__(512) void mv_tok_kernel(const uint8_t* W_, uint32_t
 
   const uint32_t tid = threadIdx.x, lane = tid & 63u, nwaves = blockDim.x >> 6;
   const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
-  const uint32_t KS = ks_, rw = small_div(wave, KS), ks = wave - rw * KS, RW = small_div(nwaves, KS);
+  // (the quotients come from the vector unit: brought back to scalar registers, the wave's row offsets are scalar too)
+  const uint32_t KS = ks_, rw = (uint32_t)__builtin_amdgcn_readfirstlane((int)small_div(wave, KS)), ks = wave - rw * KS;
+  const uint32_t RW = (uint32_t)__builtin_amdgcn_readfirstlane((int)small_div(nwaves, KS));
   const uint32_t tile_rows = RW * rpw_;
   const uint32_t t0 = blockIdx.y * T;
 
@@ -393,21 +395,23 @@ __global__ __launch_bounds__(512) void mv_tok_kernel(const uint8_t* W_, uint32_t
     const uint32_t row0 = tile_row0 + rw * rpw_;
     const uint32_t last = min(min(row0 + rpw_, rows_) - 1u, rows_ - 1u);  // last row of this wave's run
     // The wave's first NR rows are on their way while the activations are staged; a slot is refilled with the row NR
-    // places ahead before its own bytes are used (rows past the run's last repeat it: no branch around a load).
-    // Four rows in flight pay for the codebook formats at one token (a row slice is 8 bytes per lane: IQ1_S 4096x7168
-    // 8.5 -> 7.5 us); the others move 18 to 34 bytes per lane and row, and the rows repeated at the end of a run cost
-    // them more than the deeper ring gains (Q8_0 4096x4096 8.4 -> 9.8 us, Q6_K 1536x7168 6.2 -> 7.8 us).
-    // Large matrices are bound by the bytes a CU keeps in flight (two rows per wave of six to eight waves: about 20 KB,
-    // half of what the memory system needs at its latency); there a second workgroup per CU (mv_tok_shape) does more
-    // than a deeper ring (Q6_K 129280x5120: 165 us as it was, 145 with four rows in flight, 132 with two workgroups).
-    constexpr int NR = (T == 1 && requires { D::STAGES; }) ? 4 : 1;
+    // places ahead as soon as its bytes are consumed. Rows are reached through a buffer descriptor over the wave's run
+    // (BufRow): the row offset is a scalar, the lane offsets are loop constants, and a refill past the end of the run
+    // takes an empty descriptor (zeros, no memory access) instead of a branch around the load, so that every wait names
+    // an exact number of loads that may stay in flight.
+    // One token keeps four rows in flight per wave (large matrices are bound by the bytes a CU has in flight, and a
+    // second workgroup per CU, mv_tok_shape, adds to them); several tokens, whose activation slices fill the registers, two.
+    constexpr int NR = T == 1 ? 4 : 2;
     typename D::Raw ring[NR][ITERS];
+    const uint32_t run_rows = row0 <= last ? last - row0 + 1u : 0u;
+    const uint8_t* run_base = W_ + (size_t)min(row0, last) * row_bytes_;
+    auto fetch = [&](typename D::Raw (&slot)[ITERS], uint32_t j) {  // row j of the wave's run; past its end: zeros, no memory access
+      const BufRow wr = {make_rsrc(run_base, j < run_rows ? run_rows * row_bytes_ : 0u), j * row_bytes_, 0u};
 #pragma unroll
-    for (int s = 0; s < NR; s++) {
-      const gptr_t wr = as_global(W_) + (size_t)min(row0 + s, last) * row_bytes_;
+      for (int i = 0; i < ITERS; i++) slot[i] = D::load(wr, unit[i]);
+    };
 #pragma unroll
-      for (int i = 0; i < ITERS; i++) ring[s][i] = D::load(wr, unit[i]);
-    }
+    for (int s = 0; s < NR; s++) fetch(ring[s], s);
     if (group != cur_group) {
       // tokens past the last repeat it; their results are never stored
       auto x_of = [&](int t) { return x_ + (size_t)min(t0 + t, ta.n - 1) * ta.x_stride + (size_t)group * a.x_group_stride; };
@@ -454,29 +458,33 @@ __global__ __launch_bounds__(512) void mv_tok_kernel(const uint8_t* W_, uint32_t
       }
       cur_group = group;
     }
-    auto row_dot = [&](const typename D::Raw (&raw)[ITERS], uint32_t j) {
-      float acc[T];
-#pragma unroll
-      for (int t = 0; t < T; t++) {
-        acc[t] = 0.f;
-#pragma unroll
-        for (int i = 0; i < ITERS; i++) {
-          const float v = dec_dot<D>(raw[i], xr[t][i], tbl, unit[i]);
-          acc[t] += valid[i] ? v : 0.f;
-        }
-      }
-      // transposed fold: afterwards acc[0] of lane l is token group8_sel<T>(l) summed over l's 16-lane row
-      row16_fold<T>(acc, lane);
-      if (!(lane & 8u)) part[(((rw * rpw_ + j) * KS + ks) * 4 + (lane >> 4)) * T + group8_sel<T>(lane)] = acc[0];
-    };
+    // RF rows' results are folded over the lanes together (a fold takes up to eight values): afterwards lane l holds
+    // value k = group8_sel(l), row k / T of the group and token k % T, summed over l's 16-lane row
+    constexpr int RF = NR * T <= 8 ? NR : 2 * T <= 8 ? 2 : 1;
     for (uint32_t j0 = 0; j0 < rpw_; j0 += NR) {
 #pragma unroll
-      for (int s = 0; s < NR; s++) {
-        typename D::Raw cur[ITERS];
-        const gptr_t wr = as_global(W_) + (size_t)min(row0 + j0 + s + NR, last) * row_bytes_;
+      for (int f = 0; f < NR; f += RF) {
+        float acc[RF * T];
 #pragma unroll
-        for (int i = 0; i < ITERS; i++) { cur[i] = ring[s][i]; ring[s][i] = D::load(wr, unit[i]); }
-        if (NR == 1 || j0 + s < rpw_) row_dot(cur, j0 + s);  // wave-uniform; no load inside
+        for (int q = 0; q < RF; q++) {
+          const int s = f + q;
+#pragma unroll
+          for (int t = 0; t < T; t++) acc[q * T + t] = 0.f;
+          if (j0 + s < rpw_) {  // wave-uniform; no load inside (a row past the run is not decoded)
+#pragma unroll
+            for (int t = 0; t < T; t++) {
+#pragma unroll
+              for (int i = 0; i < ITERS; i++) {
+                const float v = dec_dot<D>(ring[s][i], xr[t][i], tbl, unit[i]);
+                acc[q * T + t] += valid[i] ? v : 0.f;
+              }
+            }
+          }
+          fetch(ring[s], j0 + s + NR);
+        }
+        row16_fold<RF * T>(acc, lane);
+        const uint32_t k = group8_sel<RF * T>(lane), j = j0 + f + k / T;
+        if (!(lane & 8u) && j < rpw_) part[(((rw * rpw_ + j) * KS + ks) * 4 + (lane >> 4)) * T + k % T] = acc[0];
       }
     }
     __syncthreads();

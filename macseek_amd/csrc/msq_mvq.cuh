@@ -191,8 +191,11 @@ struct DecQ5KQ {
         const uint32_t n = (r.ql[w] >> (4 * run)) & 0x0F0F0F0Fu;
         const uint32_t hb = ((r.qh[w] >> (2 * g + run)) & 0x01010101u) << 4;
         const uint32_t q = n | hb;  // 4 bytes in 0..31
-        lo = __builtin_amdgcn_sdot4((int)q, (int)x.lo[4 * run + w], lo, false);
-        hi = __builtin_amdgcn_sdot4((int)q, (int)x.hi[4 * run + w], hi, false);
+        if (w == 0) { lo = sdot4z(q, x.lo[4 * run]); hi = sdot4z(q, x.hi[4 * run]); }
+        else {
+          lo = __builtin_amdgcn_sdot4((int)q, (int)x.lo[4 * run + w], lo, false);
+          hi = __builtin_amdgcn_sdot4((int)q, (int)x.hi[4 * run + w], hi, false);
+        }
       }
       const uint32_t a = (r.pa >> (8 * run)) & 0xFFu, bq = (r.pb >> (8 * run)) & 0xFFu, c = (r.pc >> (8 * run)) & 0xFFu;
       uint32_t sc, mn;

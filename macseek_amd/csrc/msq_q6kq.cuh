@@ -76,8 +76,9 @@ struct DecQ6KQ {
   __device__ static Raw load(P row, uint32_t u) { return DecQ6K::load(row, u); }
 
   __device__ static float dot(const Raw& r, const X& x, const uint32_t*, uint32_t u) {
-    const uint32_t is = (u >> 1) & 1u;  // which half of the run pair's 16-column scale group: (8 (j & 3)) / 16
-    const float d = half_bits_to_float(r.d);
+    // the lane's four scale bytes 2 k + is, is = (8 (j & 3)) / 16 the half of the run pair's 16-column scale group,
+    // gathered into one word: each is then converted by a byte-select, without a shift of its own
+    const uint32_t sc4 = __builtin_amdgcn_perm(r.sc[1], r.sc[0], (u & 2u) ? 0x07050301u : 0x06040200u);
     float total = 0.f;
 #pragma unroll
     for (int k = 0; k < 4; k++) {
@@ -88,15 +89,17 @@ struct DecQ6KQ {
         const uint32_t n = (src >> (4 * (k >> 1))) & 0x0F0F0F0Fu;
         const uint32_t hb = 2 * k < 4 ? r.qh[w] << (4 - 2 * k) : r.qh[w] >> (2 * k - 4);
         const uint32_t q = (hb & 0x30303030u) | n;  // 4 bytes in 0..63
-        lo = __builtin_amdgcn_sdot4((int)q, (int)x.lo[2 * k + w], lo, false);
-        hi = __builtin_amdgcn_sdot4((int)q, (int)x.hi[2 * k + w], hi, false);
+        if (w == 0) { lo = sdot4z(q, x.lo[2 * k]); hi = sdot4z(q, x.hi[2 * k]); }
+        else {
+          lo = __builtin_amdgcn_sdot4((int)q, (int)x.lo[2 * k + w], lo, false);
+          hi = __builtin_amdgcn_sdot4((int)q, (int)x.hi[2 * k + w], hi, false);
+        }
       }
-      // scale byte index 2 k + is lies in word k >> 1
-      const int sc = (int)(int8_t)((r.sc[k >> 1] >> (8u * ((2u * k & 3u) + is))) & 0xFFu);
+      const float sc = (float)(int)(int8_t)(sc4 >> (8 * k));
       const float s = (float)((hi << 8) + lo + x.m32sn[k]);  // sum (q - 32) n: |.| < 2^24, exact
-      total += (d * (float)sc) * (s * x.xs[k]);
+      total = __builtin_fmaf(sc, s * x.xs[k], total);
     }
-    return total;
+    return half_bits_to_float(r.d) * total;
   }
 };
 
