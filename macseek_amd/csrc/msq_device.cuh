@@ -118,6 +118,7 @@ __device__ __forceinline__ gptr_t as_global(const void* p) { return (gptr_t)p; }
 // Range-checked buffer loads: the descriptor covers `bytes` bytes at `base`; a load whose offset falls outside returns
 // zero without touching memory. A pipelined loop can thus issue its prefetches unconditionally (an empty descriptor for
 // the rows past the end), which keeps the number of loads in flight known at every wait.
+typedef uint32_t __attribute__((ext_vector_type(4))) u32x4;
 typedef __amdgpu_buffer_rsrc_t rsrc_t;
 __device__ __forceinline__ rsrc_t make_rsrc(const void* base, uint32_t bytes) {
   return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)bytes, 0x00020000);
@@ -137,6 +138,10 @@ __device__ __forceinline__ u128_a2 buf_ld128(rsrc_t r, uint32_t voff, uint32_t s
   const auto v = __builtin_amdgcn_raw_buffer_load_b128(r, (int)voff, (int)soff, 0);
   return {(uint32_t)v[0], (uint32_t)v[1], (uint32_t)v[2], (uint32_t)v[3]};
 }
+__device__ __forceinline__ u32x4 buf_ld128v(rsrc_t r, uint32_t voff, uint32_t soff) {
+  const auto v = __builtin_amdgcn_raw_buffer_load_b128(r, (int)voff, (int)soff, 0);
+  return u32x4{(uint32_t)v[0], (uint32_t)v[1], (uint32_t)v[2], (uint32_t)v[3]};
+}
 // A weight row reached through a buffer descriptor, in the shape of a pointer for the decoders' load() functions
 // (p + bytes, ld16 .. ld128): rs covers a run of rows, soff is the row's byte offset in it -- wave-uniform, so it travels
 // in a scalar register -- and voff the lane's byte offset inside the row, a loop constant. A row's loads then cost no
@@ -150,6 +155,37 @@ __device__ __forceinline__ uint32_t ld16(const BufRow& p) { return buf_ld16(p.rs
 __device__ __forceinline__ uint32_t ld32(const BufRow& p) { return buf_ld32(p.rs, p.voff, p.soff); }
 __device__ __forceinline__ u64_a2 ld64(const BufRow& p) { return buf_ld64(p.rs, p.voff, p.soff); }
 __device__ __forceinline__ u128_a2 ld128(const BufRow& p) { return buf_ld128(p.rs, p.voff, p.soff); }
+
+// A weight row whose bytes a wave holds in LDS (see mv_tok_kernel): `base` is the wave's 16-byte-aligned buffer, at + sh
+// the byte offset in it, only 2-byte aligned like the blocks themselves, kept as its aligned part and its low two bits.
+// LDS reads want aligned addresses: a load reads the aligned words that hold its bytes and shifts them into place.
+// (Two fields: the offsets a decoder adds behind the block's are multiples of four, which the compiler can see, so
+// that the split is made once per block and not once per load.)
+struct LdsRow {
+  const uint8_t* base;
+  uint32_t at, sh;
+  __device__ __forceinline__ static LdsRow of(const uint8_t* base, uint32_t off) { return {base, off & ~3u, off & 3u}; }
+  __device__ __forceinline__ LdsRow operator+(uint32_t o) const {
+    const uint32_t t = sh + o;
+    return {base, at + (t & ~3u), t & 3u};
+  }
+};
+__device__ __forceinline__ uint32_t ld16(const LdsRow& p) { return *(const uint16_t*)(p.base + p.at + p.sh); }
+__device__ __forceinline__ uint32_t ld32(const LdsRow& p) {
+  const uint32_t* q = (const uint32_t*)(p.base + p.at);
+  return __builtin_amdgcn_alignbyte(q[1], q[0], p.sh);
+}
+__device__ __forceinline__ u64_a2 ld64(const LdsRow& p) {
+  const uint32_t* q = (const uint32_t*)(p.base + p.at);
+  const uint32_t d0 = q[0], d1 = q[1], d2 = q[2];
+  return {__builtin_amdgcn_alignbyte(d1, d0, p.sh), __builtin_amdgcn_alignbyte(d2, d1, p.sh)};
+}
+__device__ __forceinline__ u128_a2 ld128(const LdsRow& p) {
+  const uint32_t* q = (const uint32_t*)(p.base + p.at);
+  const uint32_t d0 = q[0], d1 = q[1], d2 = q[2], d3 = q[3], d4 = q[4];
+  return {__builtin_amdgcn_alignbyte(d1, d0, p.sh), __builtin_amdgcn_alignbyte(d2, d1, p.sh), __builtin_amdgcn_alignbyte(d3, d2, p.sh),
+          __builtin_amdgcn_alignbyte(d4, d3, p.sh)};
+}
 
 #define MSQ_LOADERS(AS)                                                                                               \
   __device__ __forceinline__ uint32_t ld8(const AS uint8_t* p) { return *p; }                                         \
@@ -270,7 +306,6 @@ __device__ __forceinline__ void copy_words16(uint32_t* dst, const uint32_t* src,
   for (int i = tid; i < nwords / 4; i += nthreads) d[i] = s[i];
 }
 
-typedef uint32_t __attribute__((ext_vector_type(4))) u32x4;
 
 // floor(a / b) for a < 4096 and 0 < b <= 64 in four instructions instead of the forty of an integer division (wave
 // counts and rows of a chunk): (a + 0.5) / b lies at least 1 / 128 away from every integer, and the float product is
@@ -420,6 +455,7 @@ __device__ __forceinline__ X32 load_x32_half(const uint32_t* p) {
 // ---- IQ1_S: {fp16 d; u8 qs[32]; u16 qh[8]}, 50 bytes / 256 weights; unit = one 32-weight sub-block
 struct DecIQ1S {
   static constexpr int UNIT = 32, GRID_WORDS = MSQ_IQ1S_GRID_N * 4, LDS_WORDS = GRID_WORDS + 32;
+  static constexpr uint32_t BLOCK = 50, UPB = 8;  // bytes of a block, units in it
   static constexpr bool STAGE_X = true;
   typedef X32 X;
   struct Raw { uint32_t qs, qh, d; };
@@ -508,6 +544,7 @@ struct DecIQ1S {
 // ---- IQ2_XXS: {fp16 d; u16 qs[32]}, 66 bytes / 256 weights; unit = one 32-weight sub-block (8 bytes)
 struct DecIQ2XXS {
   static constexpr int UNIT = 32, LDS_WORDS = MSQ_IQ2XXS_GRID_N * 4 + 128 * 4;
+  static constexpr uint32_t BLOCK = 66, UPB = 8;  // bytes of a block, units in it
   static constexpr bool STAGE_X = true;
   typedef X32 X;
   struct Raw { uint32_t a0, a1, d; };
@@ -595,6 +632,7 @@ struct DecIQ2XXS {
 // ---- Q8_0: {fp16 d; int8 qs[32]}, 34 bytes / 32 weights; unit = one block, activations kept in fp32
 struct DecQ8_0 {
   static constexpr int UNIT = 32, LDS_WORDS = 0;
+  static constexpr uint32_t BLOCK = 34, UPB = 1;  // bytes of a block, units in it
   static constexpr bool STAGE_X = true;
   struct X { float v[32]; };
   struct Raw { uint32_t q[8]; uint32_t d; };
@@ -630,6 +668,7 @@ struct DecQ8_0 {
 // ---- IQ4_NL: {fp16 d; u8 qs[16]}, 18 bytes / 32 weights; byte j holds columns j (low nibble) and j + 16 (high)
 struct DecIQ4NL {
   static constexpr int UNIT = 32, LDS_WORDS = 256;
+  static constexpr uint32_t BLOCK = 18, UPB = 1;  // bytes of a block, units in it
   static constexpr bool STAGE_X = true;
   struct X { uint32_t v[16]; };  // pair j = (x[j], x[j + 16])
   struct Raw { uint32_t q[4]; uint32_t d; };
@@ -668,6 +707,7 @@ struct DecIQ4NL {
 // 128 h + 32 k + l0 .. + 7 (k = 0..3), which share the bytes ql[64 h + l0 ..], ql[64 h + 32 + l0 ..], qh[32 h + l0 ..].
 struct DecQ6K {
   static constexpr int UNIT = 32, LDS_WORDS = 0;
+  static constexpr uint32_t BLOCK = 210, UPB = 8;  // bytes of a block, units in it
   static constexpr bool STAGE_X = false;
   struct X { uint32_t v[16]; float sx[4]; };
   struct Raw { uint32_t qa[2], qb[2], qh[2], sc[2], d; };
@@ -721,6 +761,7 @@ struct DecQ6K {
 // scale index 2 g) and 64 g + 32 + l0 .. + 15 (high nibbles, scale index 2 g + 1).
 struct DecQ5K {
   static constexpr int UNIT = 32, LDS_WORDS = 0;
+  static constexpr uint32_t BLOCK = 176, UPB = 8;  // bytes of a block, units in it
   static constexpr bool STAGE_X = false;
   struct X { uint32_t v[16]; float sx[2]; };
   struct Raw { uint32_t ql[4], qh[4], pa, pb, pc, dd; };

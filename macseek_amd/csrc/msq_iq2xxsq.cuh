@@ -41,6 +41,7 @@ __device__ __attribute__((aligned(16))) const TblIQ2XXS8 g_tbl_iq2xxs8 = make_iq
 
 struct DecIQ2XXSQ {
   static constexpr int UNIT = 32;
+  static constexpr uint32_t BLOCK = 66, UPB = 8;
   static constexpr int LDS_WORDS = 16384;  // 256 rows of 256 bytes
   static constexpr bool STAGE_X = true, QUANT_X = true;
   static constexpr int STAGES = 2;         // two grid entries (16 weights) per stage

@@ -56,7 +56,7 @@ __global__ __launch_bounds__(1024) void bw_probe_kernel(const uint4* __restrict_
 namespace {
 
 // Launch shape of the decode matvec. units = cols / UNIT columns-slices per row; a wave covers 64 * iters of them.
-struct MvShape { int iters, ks, rw, rpw, unit; int per_cu = 1; };  // per_cu: persistent workgroups per CU (mv_tok_kernel)
+struct MvShape { int iters, ks, rw, rpw, unit; int per_cu = 1; bool stage_w = false; };  // per_cu: persistent workgroups per CU, stage_w: weight rows through LDS (mv_tok_kernel)
 
 int mv_unit(int t) { return msq_type_block_elems(t) == 1 ? 8 : 32; }
 
@@ -195,7 +195,15 @@ bool mv_tok_shape(int t, int rows, int cols, int groups, int n, int token_groups
     while (rw > 1 && rpg % (rw * rpw)) rw /= 2;
     if (rpg % (rw * rpw)) return false;
   }
-  *s = {iters, ks, rw, rpw, unit, per_cu};
+  // Weight rows through LDS (mv_tok_kernel) where it measures faster: Q6_K (five loads per lane and row otherwise) from
+  // 12 MB, Q8_0 (three) from 40 MB -- ring / through LDS: Q6_K 8192x5120 12.3 / 12.0 us, 65536x5120 71.9 / 57.0, Q8_0
+  // 8192x5120 12.9 / 12.2, 65536x5120 82.4 / 67.5. Q5_K and IQ4_NL, whose 16-byte reads from LDS cost five words and four
+  // shifts each, lose 10 to 17 %; the codebook formats are bound by their table lookups. MSQ_MV_STAGEW = 0 / 1 imposes
+  // the choice.
+  static const int env_sw = env_knob_early("MSQ_MV_STAGEW", -1);
+  const bool stage_w = n == 1 && free_shape &&
+                       (env_sw >= 0 ? env_sw > 0 : (t == MSQ_Q6_K && bytes >= 12e6) || (t == MSQ_Q8_0 && bytes >= 40e6));
+  *s = {iters, ks, rw, rpw, unit, per_cu, stage_w};
   return true;
 }
 
@@ -225,6 +233,12 @@ int launch_mv_tok(hipStream_t st, const MvShape& s, MvTokArgs& ta) {
     // one workgroup per CU: all of its LDS (decoders that stage only in the four-token kernel read directly when a round does not fit)
     if (!place_x_row(a, lds, tok_round<D, T>(), kMaxLds - kStaticLds<D>, D::STAGE_X)) return MSQ_ERR_UNSUPPORTED;
   }
+  const bool sw = tok_stages_w<D, 1, T>() && s.iters == 1 && s.stage_w && !a.norm_w;
+  if (sw) {  // the waves' weight-row buffers
+    lds = (lds + 15) / 16 * 16;
+    a.w_off = (uint32_t)(lds / 4);
+    lds += (size_t)(threads / 64) * 4 * wspan_loads<D>() * 1024;  // four slots per wave
+  }
   auto launch = [&](auto kernel, dim3 grid) {
     allow_large_lds(kernel, lds);
     hipLaunchKernelGGL(kernel, grid, dim3(threads), lds, st, a.W, a.rows, a.row_bytes, a.units, a.ks, a.rpw, a.ntiles, a.rows_per_group, a.x, a.cols, ta);
@@ -244,7 +258,9 @@ int launch_mv_tok(hipStream_t st, const MvShape& s, MvTokArgs& ta) {
   const int per_cu = (T == 1 && !a.norm_w && (lds + kStaticLds<D>) * s.per_cu <= (size_t)kMaxLds) ? s.per_cu : 1;
   const int gx = (int)std::min<long>(a.ntiles, std::max(1, per_cu * device_info().cus / gy));
   const dim3 grid((unsigned)gx, (unsigned)gy);
-  if (s.iters == 1) launch(mv_tok_kernel<D, 1, T>, grid);
+  if (sw) {
+    if constexpr (tok_stages_w<D, 1, T>()) launch(mv_tok_kernel<D, 1, T, false, true>, grid);
+  } else if (s.iters == 1) launch(mv_tok_kernel<D, 1, T>, grid);
   else if constexpr (D::UNIT == 8) launch(mv_tok_kernel<D, 2, T>, grid);
   else return MSQ_ERR_UNSUPPORTED;  // two block-format units per lane and T activation slices do not fit the registers
   MSQ_HIP(hipGetLastError());

@@ -32,6 +32,7 @@ struct MvArgs {
   // (xlds_words(cols) words), and whether the plain kernels stage at all (rows too long for LDS are read directly)
   uint32_t xs_off;
   uint32_t stage_x;
+  uint32_t w_off;     // word offset in dynamic LDS of the waves' weight-row buffers (token kernel, one token of a block format)
 };
 
 // The lane's activation slices of one row, from the workgroup's padded LDS copy (staged here, all threads must call)
@@ -332,13 +333,67 @@ constexpr int tok_round() {
 template <class D, int T>
 constexpr bool tok_stages_x() { return D::STAGE_X || (T == 4 && D::UNIT == 32); }
 
+// Whether the T-token kernel of decoder D copies its weight rows through LDS (one token of a block format; see the kernel),
+// the bytes of a wave's slice of a row (its 64 units' blocks; fewer at the end of the row), and the 16-byte pieces per
+// lane that cover a slice at any alignment.
+template <class D, int ITERS, int T>
+constexpr bool tok_stages_w() {
+  if constexpr (requires { D::BLOCK; }) return T == 1 && ITERS == 1;
+  else return false;
+}
+template <class D>
+__host__ __device__ constexpr uint32_t wspan_bytes() {
+  if constexpr (requires { D::BLOCK; }) return (64u / D::UPB) * D::BLOCK;
+  else return 0u;
+}
+template <class D>
+__host__ __device__ constexpr uint32_t wspan_loads() { return (wspan_bytes<D>() + 14u + 1023u) / 1024u; }
+template <class D>
+__device__ __forceinline__ uint32_t wspan_len(uint32_t units, uint32_t ks) {
+  if constexpr (requires { D::BLOCK; }) {
+    constexpr uint32_t SB = 64u / D::UPB;
+    const uint32_t nblk = units / D::UPB, b0 = ks * SB;
+    return (min(b0 + SB, nblk) - b0) * D::BLOCK;
+  } else return 0u;
+}
+
+// Waits until at most N of the wave's vector memory operations are outstanding, and keeps the compiler from moving memory
+// accesses across the wait (s_waitcnt: the count's low four bits in bits 0-3, its high two in bits 14-15; the other
+// counters at their maxima, i.e. not waited for).
+template <int N>
+__device__ __forceinline__ void wait_rows() {
+  static_assert(N >= 0 && N < 64, "s_waitcnt holds six bits of vmcnt");
+  asm volatile("" ::: "memory");
+  __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
+  asm volatile("" ::: "memory");
+}
+
+// the same for a count that is a constant only after unrolling (0 .. 9)
+__device__ __forceinline__ void wait_rows_n(int n) {
+  switch (n) {
+    case 0: wait_rows<0>(); break;
+    case 1: wait_rows<1>(); break;
+    case 2: wait_rows<2>(); break;
+    case 3: wait_rows<3>(); break;
+    case 4: wait_rows<4>(); break;
+    case 5: wait_rows<5>(); break;
+    case 6: wait_rows<6>(); break;
+    case 7: wait_rows<7>(); break;
+    case 8: wait_rows<8>(); break;
+    case 9: wait_rows<9>(); break;
+    default: wait_rows<0>(); break;
+  }
+}
+
 // Decoders with STAGE_X take the activations through LDS (contiguous loads, tok_round() tokens per round); with the
 // others every lane reads its slices from device memory, all T tokens' loads in flight at once.
-template <class D, int ITERS, int T, bool NORM = false>
+template <class D, int ITERS, int T, bool NORM = false, bool SW = false>
 __global__ __launch_bounds__(512) void mv_tok_kernel(const uint8_t* W_, uint32_t rows_, uint32_t row_bytes_, uint32_t units_, uint32_t ks_,
                                                      uint32_t rpw_, uint32_t ntiles_, uint32_t rows_per_group_, const float* x_,
                                                      uint32_t cols_, const MvTokArgs ta) {
   constexpr bool STAGE = tok_stages_x<D, T>();
+  constexpr bool STAGE_W = SW && tok_stages_w<D, ITERS, T>();  // weight rows through LDS: the launch's choice (large matrices)
+  constexpr int WL = STAGE_W ? (int)wspan_loads<D>() : 1;
   // What the first loads need comes as leading arguments (W_ .. cols_: the fields of the same names in ta.m, delivered
   // in scalar registers with the wave when the file is built with kernel-argument preload) and is used under those
   // names below; the rest is read from the argument block.
@@ -402,16 +457,64 @@ __global__ __launch_bounds__(512) void mv_tok_kernel(const uint8_t* W_, uint32_t
     // One token keeps four rows in flight per wave (large matrices are bound by the bytes a CU has in flight, and a
     // second workgroup per CU, mv_tok_shape, adds to them); several tokens, whose activation slices fill the registers, two.
     constexpr int NR = T == 1 ? 4 : 2;
-    typename D::Raw ring[NR][ITERS];
     const uint32_t run_rows = row0 <= last ? last - row0 + 1u : 0u;
+    // ---- one token of a block format, large matrix: the wave's slice of a row -- the consecutive blocks of its 64 units,
+    // one contiguous run of bytes -- is fetched as aligned 16-byte pieces, consecutive lanes consecutive pieces (one to
+    // three loads per lane and row, each cache line requested once), straight into a slot of the wave's own LDS ring
+    // (loads with an LDS destination), and read from there by the decoder's load(). A lane's pieces of a block lie in
+    // the same few cache lines as its neighbours', and fetched lane by lane every one of a decoder's three to six loads
+    // asks for all lines of the slice again; the vector cache then holds several requests per line in its queue, and
+    // that queue, not memory, bounds the launch (Q6_K 129280x5120 with the arithmetic taken out: 133 us with Q6_K's
+    // five loads per lane, 107 with three of them, 89 with one, 85 with two loads of consecutive 16-byte pieces -- the
+    // speed of a plain read).
+    // The compiler does not know that such a load writes LDS: the waits for a slot's loads (wait_rows) and the order of
+    // slot reads and refills are written out below. Loads complete in order, so "at most k row requests outstanding"
+    // means every older one has landed; other loads and stores in flight only make a wait stricter.
+    [[maybe_unused]] typename D::Raw ring[STAGE_W ? 1 : NR][ITERS];
+    [[maybe_unused]] typename D::Raw raw[2];
+    [[maybe_unused]] uint32_t span_at = 0, w_low = 0;  // the slice's byte offset in a row; low address bits of the run's first slice
+    [[maybe_unused]] rsrc_t w_rs, w_none;
+    [[maybe_unused]] uint8_t* wbuf = nullptr;
+    if constexpr (STAGE_W) {
+      constexpr uint32_t SB = 64u / D::UPB;  // blocks of the wave's 64 units
+      const uint32_t nblk = units_ / D::UPB, b0 = ks * SB;
+      span_at = b0 * D::BLOCK;
+      const uint32_t span_len = (min(b0 + SB, nblk) - b0) * D::BLOCK;
+      const uint64_t first = (uint64_t)(uintptr_t)W_ + (uint64_t)min(row0, last) * row_bytes_ + span_at;
+      w_low = (uint32_t)first & 15u;
+      const uint32_t covered = run_rows ? (w_low + (run_rows - 1u) * row_bytes_ + span_len + 15u) & ~15u : 0u;
+      w_rs = make_rsrc((const void*)(uintptr_t)(first & ~15ull), covered);
+      w_none = make_rsrc((const void*)(uintptr_t)(first & ~15ull), 0u);
+      wbuf = (uint8_t*)(smem + a.w_off) + wave * (NR * WL * 1024u);
+    }
+    // request row j of the run into slot s (past the end of the run: zeros, no memory access)
+    auto request = [&](int s, uint32_t j) {
+      typedef __attribute__((address_space(3))) void* lds_ptr_t;
+      const uint32_t so = w_low + j * row_bytes_;                   // bytes from the descriptor's base to the slice
+      const uint32_t top = ((so & 15u) + wspan_len<D>(units_, ks) - 1u) & ~15u;  // offset of the slice's last piece
+      asm volatile("" ::: "memory");  // behind the reads of the slot's previous row
+#pragma unroll
+      for (int k = 0; k < WL; k++)  // lane l's piece lands at the given LDS address + 16 l
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(j < run_rows ? w_rs : w_none, (lds_ptr_t)(wbuf + (s * WL + k) * 1024u), 16,
+                                                 (int)min(16u * lane + 1024u * k, top), (int)(so & ~15u), 0, 0);
+    };
+    auto take = [&](int s, uint32_t j) {  // the lane's block bytes of row j, which slot s holds
+      return D::load(LdsRow::of(wbuf + s * WL * 1024u, ((w_low + j * row_bytes_) & 15u) - span_at), unit[0]);
+    };
     const uint8_t* run_base = W_ + (size_t)min(row0, last) * row_bytes_;
     auto fetch = [&](typename D::Raw (&slot)[ITERS], uint32_t j) {  // row j of the wave's run; past its end: zeros, no memory access
       const BufRow wr = {make_rsrc(run_base, j < run_rows ? run_rows * row_bytes_ : 0u), j * row_bytes_, 0u};
 #pragma unroll
       for (int i = 0; i < ITERS; i++) slot[i] = D::load(wr, unit[i]);
     };
+    // Half of the ring is requested ahead of the activations, the other half behind them: loads return in order, so with
+    // the whole ring ahead the activations of a small matrix wait for four rows.
+    constexpr int AHEAD = NR / 2;
 #pragma unroll
-    for (int s = 0; s < NR; s++) fetch(ring[s], s);
+    for (int s = 0; s < AHEAD; s++) {
+      if constexpr (STAGE_W) request(s, s);
+      else fetch(ring[s], s);
+    }
     if (group != cur_group) {
       // tokens past the last repeat it; their results are never stored
       auto x_of = [&](int t) { return x_ + (size_t)min(t0 + t, ta.n - 1) * ta.x_stride + (size_t)group * a.x_group_stride; };
@@ -458,10 +561,21 @@ __global__ __launch_bounds__(512) void mv_tok_kernel(const uint8_t* W_, uint32_t
       }
       cur_group = group;
     }
+#pragma unroll
+    for (int s = AHEAD; s < NR; s++) {
+      if constexpr (STAGE_W) request(s, s);
+      else fetch(ring[s], s);
+    }
     // RF rows' results are folded over the lanes together (a fold takes up to eight values): afterwards lane l holds
     // value k = group8_sel(l), row k / T of the group and token k % T, summed over l's 16-lane row
     constexpr int RF = NR * T <= 8 ? NR : 2 * T <= 8 ? 2 : 1;
-    for (uint32_t j0 = 0; j0 < rpw_; j0 += NR) {
+    if constexpr (STAGE_W) {  // row 0 to registers
+      wait_rows<(NR - 1) * WL>();
+      raw[0] = take(0, 0);
+    }
+    // A round = the NR rows the ring holds. Rounds with more rows behind them refill every slot (with an empty descriptor
+    // past the end of the run); the last round requests nothing, so a short run pays for no loads it does not need.
+    auto round = [&]<bool REFILL>(uint32_t j0) {
 #pragma unroll
       for (int f = 0; f < NR; f += RF) {
         float acc[RF * T];
@@ -470,23 +584,40 @@ __global__ __launch_bounds__(512) void mv_tok_kernel(const uint8_t* W_, uint32_t
           const int s = f + q;
 #pragma unroll
           for (int t = 0; t < T; t++) acc[q * T + t] = 0.f;
-          if (j0 + s < rpw_) {  // wave-uniform; no load inside (a row past the run is not decoded)
+          if constexpr (STAGE_W) {
+            // the next row moves to the other register set while this one is multiplied; this row's slot, whose bytes
+            // the multiplication has consumed, is then requested again
+            if (REFILL || s + 1 < NR) {  // (a constant: the loops are unrolled)
+              wait_rows_n((REFILL ? NR - 2 : NR - 2 - s) * WL);  // row requests behind the next row's
+              raw[(s + 1) & 1] = take((s + 1) % NR, j0 + s + 1);
+            }
+            if (j0 + s < rpw_) {
+              const float v = dec_dot<D>(raw[s & 1], xr[0][0], tbl, unit[0]);
+              acc[q] = valid[0] ? v : 0.f;
+            }
+            if constexpr (REFILL) request(s, j0 + s + NR);
+          } else {
+            if (j0 + s < rpw_) {  // wave-uniform; no load inside (a row past the run is not decoded)
 #pragma unroll
-            for (int t = 0; t < T; t++) {
+              for (int t = 0; t < T; t++) {
 #pragma unroll
-              for (int i = 0; i < ITERS; i++) {
-                const float v = dec_dot<D>(ring[s][i], xr[t][i], tbl, unit[i]);
-                acc[q * T + t] += valid[i] ? v : 0.f;
+                for (int i = 0; i < ITERS; i++) {
+                  const float v = dec_dot<D>(ring[s][i], xr[t][i], tbl, unit[i]);
+                  acc[q * T + t] += valid[i] ? v : 0.f;
+                }
               }
             }
+            if constexpr (REFILL) fetch(ring[s], j0 + s + NR);
           }
-          fetch(ring[s], j0 + s + NR);
         }
         row16_fold<RF * T>(acc, lane);
         const uint32_t k = group8_sel<RF * T>(lane), j = j0 + f + k / T;
         if (!(lane & 8u) && j < rpw_) part[(((rw * rpw_ + j) * KS + ks) * 4 + (lane >> 4)) * T + k % T] = acc[0];
       }
-    }
+    };
+    uint32_t j0 = 0;
+    for (; j0 + NR < rpw_; j0 += NR) round.template operator()<true>(j0);
+    round.template operator()<false>(j0);
     __syncthreads();
     for (uint32_t idx = tid; idx < tile_rows * T; idx += blockDim.x) {
       const uint32_t r = idx % tile_rows, t = idx / tile_rows, row = tile_row0 + r;  // consecutive lanes: consecutive rows

@@ -56,6 +56,7 @@ __device__ __attribute__((aligned(16))) const TblIQ1S8g g_tbl_iq1s8g = make_iq1s
 
 struct DecIQ1SM {
   static constexpr int UNIT = 32, GRID_WORDS = MSQ_IQ1S_GRID_N * 4, LDS_WORDS = GRID_WORDS + 32;
+  static constexpr uint32_t BLOCK = 50, UPB = 8;
   static constexpr bool STAGE_X = true;
   static constexpr int STAGES = 1;
   struct X { uint32_t lo[8], hi[8]; float xs, sx; };  // sx = xs * sum n: the sum of the unit's (rounded) activations
@@ -160,6 +161,7 @@ struct DecIQ2XXSM : DecIQ2XXSQ {
 // 6-bit scale and min: sum w x = d sc xs_run sum q n - dmin m xs_run sum n, q = nibble | high bit << 4 in 0..31.
 struct DecQ5KQ {
   static constexpr int UNIT = 32, LDS_WORDS = 0;
+  static constexpr uint32_t BLOCK = 176, UPB = 8;
   static constexpr bool STAGE_X = false;
   struct X { uint32_t lo[8], hi[8]; float xs[2], sx[2]; };
   typedef DecQ5K::Raw Raw;
@@ -223,6 +225,7 @@ __device__ __attribute__((aligned(16))) const TblIQ4NL16 g_tbl_iq4nl16 = make_iq
 
 struct DecIQ4NLQ {
   static constexpr int UNIT = 32, LDS_WORDS = 256;
+  static constexpr uint32_t BLOCK = 18, UPB = 1;
   static constexpr bool STAGE_X = true;
   struct X { uint32_t v[16]; float xs; };  // pair j = (n[j], n[j + 16]) as int16
   typedef DecIQ4NL::Raw Raw;

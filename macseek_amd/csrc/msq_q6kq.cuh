@@ -18,6 +18,7 @@ namespace msq {
 
 struct DecQ6KQ {
   static constexpr int UNIT = 32, LDS_WORDS = 0;
+  static constexpr uint32_t BLOCK = 210, UPB = 8;
   static constexpr bool STAGE_X = false, QUANT_X = true;  // (STAGE_X: the decode matvec reads its short runs directly, as DecQ6K)
   // per run k: two words of low bytes, two of high bytes, the scale, and -32 * sum n
   struct X { uint32_t lo[8], hi[8]; float xs[4]; int m32sn[4]; };
