@@ -272,7 +272,7 @@ def bench_moe_decode(torch, args):
                                "top-6 of a seeded softmax router + 1 shared IQ2_XXS expert, SwiGLU; fresh top-6 per step",
                    "bytes_per_step": step_bytes, "experts": NE, "top_k": TOPK, "dim": DIM, "inter": INTER},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBPS,
-                     "traffic": profile_traffic("moe_hbm_traffic_fetch_write.txt", "moe_gu_kernel<"), "traffic_source": "profiles/moe_hbm_traffic_fetch_write.txt", "kernel": "moe_gu_kernel<DecIQ1SQ,DecIQ2XXS>", "bytes_per_launch": gu_bytes,
+                     "traffic": profile_traffic("moe_hbm_traffic_fetch_write.txt", "moe_gu_kernel<"), "traffic_source": "profiles/moe_hbm_traffic_fetch_write.txt", "kernel": "moe_gu_kernel<DecIQ1SQ,DecIQ2XXSQ>", "bytes_per_launch": gu_bytes,
                      "avg_launch_us": gu_graph * 1e3,
                      "timing": "HIP event pair around one graph replay of %d back-to-back launches of this kernel" % n_ev,
                      "eager_event_pair_us": {"mean": gu_mean * 1e3, "median": gu_med * 1e3, "min": gu_min * 1e3},
