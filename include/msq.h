@@ -105,11 +105,14 @@ int msq_rmsnorm(void* stream, const MsqBuffer* x, const MsqBuffer* w, const MsqB
  * cols * groups, Y row stride is rows. n == 1 is exactly msq_matvec. For n >= 2, rows of up to 16384 columns (dense
  * types: 8192) run in a dot-product kernel that stages activations as fp16 pairs for the K / IQ formats (the
  * reference's numerics from two tokens on), fp32 for Q8_0 and the dense types, and decodes each weight once for up to
- * eight tokens. Wider rows, and
+ * eight tokens. From nine tokens on (groups == 1, X 16-byte aligned) Q5_K, Q6_K, IQ1_S and IQ2_XXS, and Q6_K matrices
+ * of 5 to 12 MB at eight tokens, run in msq_matmul's fused matrix-core kernel (activations rounded to fp16, exact
+ * payloads, scales in fp32); like msq_matmul these calls sum K slices through a buffer inside the library and must be
+ * enqueued on one stream at a time (MSQ_MVN_MM=0 keeps them in the dot-product kernel). The reference hands n >= 8 to
+ * its matmul kernel the same way (quant.mm:133-137). Wider rows, and
  * more than eight tokens over a large IQ4_NL / Q8_0 / F16 / BF16 matrix, run on the matrix cores with activations
- * rounded to fp16 (BF16 weights: split into two bf16 terms) and exact weights; the reference rounds activations to
- * fp16 the same way and, from n >= 8, weights too (quant.mm:133-137). Wide F32 matrices, and wide block-diagonal
- * calls whose group size is not a multiple of 16 rows, are served as n decode matvecs. */
+ * rounded to fp16 (BF16 weights: split into two bf16 terms) and exact weights. Wide F32 matrices, and wide
+ * block-diagonal calls whose group size is not a multiple of 16 rows, are served as n decode matvecs. */
 int msq_matvec_n(void* stream, int qtype, const MsqBuffer* W, int rows, int cols, const MsqBuffer* X,
                  const MsqBuffer* Y, int n, int accumulate, int groups);
 

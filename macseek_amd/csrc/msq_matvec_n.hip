@@ -1,5 +1,6 @@
 // C ABI: small-N matvec (see include/msq.h; reference host code src/kernels/quant.mm:129-156).
 #include <algorithm>
+#include <cstdlib>
 
 #include "msq_host.h"
 #include "msq_mvn.cuh"
@@ -43,7 +44,19 @@ extern "C" int msq_matvec_n(void* stream, int t, const MsqBuffer* W, int rows, i
                 msq_type_name_of(t), rows, cols, n);
   const int rpg = rows / groups;
   const double mb = (double)rb * rows / 1e6;
-  // Two kernels serve n > 1. The dot-product kernel (weights fetched in contiguous runs, decoded once for up to eight
+  // From nine tokens on (two passes of the dot-product kernel below) the K-quant and codebook formats go through the
+  // fused matrix-core kernel of msq_matmul, as the reference's small-N operator hands its larger n to its matmul kernel
+  // (quant.mm:133): Q6_K 2304x5120 at 12 tokens 17.3 -> 11.1 us, IQ1_S 4096x7168 at 16 tokens 24.9 -> 16.7, Q5_K
+  // 1280x5120 at 16 tokens 13.7 -> 9.7; at eight tokens only Q6_K matrices of 5 to 12 MB gain (1536x7168: 11.3 -> 10.8).
+  // IQ4_NL, Q8_0 and the dense types stay below (IQ4_NL 7168x4096 at 16 tokens: 20.6 us here, 26.4 there). That route
+  // sums its K slices through a buffer inside the library: such calls must be enqueued on one stream at a time.
+  {
+    const bool kq = t == MSQ_Q6_K || t == MSQ_Q5_K || t == MSQ_IQ1_S || t == MSQ_IQ2_XXS;
+    const bool mm = groups == 1 && cols % 128 == 0 && ((kq && n >= 9) || (t == MSQ_Q6_K && n == 8 && mb >= 5.0 && mb <= 12.0));
+    static const bool off = [] { const char* e = getenv("MSQ_MVN_MM"); return e && *e == '0'; }();
+    if (mm && !off && !((uintptr_t)bptr(X) & 15)) return msq_matmul(stream, t, W, rows, cols, X, Y, n, accumulate);
+  }
+  // Two kernels serve 2 <= n <= 8 (and what the rule above leaves). The dot-product kernel (weights fetched in contiguous runs, decoded once for up to eight
   // tokens, dot2 chains per token) wins wherever its shape fits: measured on MI355X at n = 16, IQ4_NL 7168x4096 takes
   // 20.7 us there and 25.4 us through the MFMA kernel, Q8_0 4096x7168 28.8 and 29.6 us, Q6_K 1536x7168 14.4 and 42.9 us.
   {

@@ -80,13 +80,15 @@ def test_matvec_n_vs_oracle(dev, t, rows, cols, groups, n, acc):
     print(f"  {O.TYPE_NAMES[t]:8s} [{cols:5d} -> {rows:5d}] g{groups} n={n:<2d} {'acc' if acc else '   '} "
           f"err(x staged) {err_h:.2e}  err(vs F32) {err_f:.2e}  north-star {err_ns:.2e}")
     # reference bounds: 2e-6 against the half-x reference for its F32-FMA kernel (n < 8), 1e-4 on its tile path (n >= 8),
-    # 2e-4 against the F32 reference (tests/test_quant_matvec_n.mm:45-46). Here the tighter one is held at every n
-    # (measured: at most 7.8e-7, Q5_K 37 x 256).
+    # 2e-4 against the F32 reference (tests/test_quant_matvec_n.mm:45-46): the same two here. The dot-product kernels
+    # stay below 1e-6 at every n; from nine tokens on the library hands the K-quant and codebook formats to its fused
+    # matrix-core kernel, whose codebook fragments carry the scale in the fp16 payload like the reference's tiles
+    # (measured there: 4e-5 for IQ2_XXS, below 2e-6 for Q5_K / Q6_K).
     # One token is the decode matvec: F32-activation arithmetic to the reference's 2e-5 (tests/test_quant_matvec.mm:42).
     if n == 1:
         assert err_f <= 2e-5 and err_ns <= TOL_NORTH_STAR
     else:
-        assert err_h <= 2e-6 and err_f <= 2e-4 and err_ns <= TOL_NORTH_STAR
+        assert err_h <= (2e-6 if n < 8 else 1e-4) and err_f <= 2e-4 and err_ns <= TOL_NORTH_STAR
 
 
 def test_matvec_n_misuse_and_untouched_rows(dev):
