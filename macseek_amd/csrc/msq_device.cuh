@@ -354,6 +354,31 @@ __device__ __forceinline__ void copy_jobs(uint32_t* smem, const CopyJob (&jobs)[
   }
 }
 
+// Waits until at most N of the wave's vector memory operations are outstanding, and keeps the compiler from moving memory
+// accesses across the wait (s_waitcnt: the count's low four bits in bits 0-3, its high two in bits 14-15; the other
+// counters at their maxima, i.e. not waited for). For loads whose destination is LDS, which the compiler does not track.
+template <int N>
+__device__ __forceinline__ void wait_vm() {
+  static_assert(N >= 0 && N < 64, "s_waitcnt holds six bits of vmcnt");
+  asm volatile("" ::: "memory");
+  __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
+  asm volatile("" ::: "memory");
+}
+// A piece of a prologue copy by loads that write LDS themselves (no registers in between, so the requests can be issued
+// ahead of everything else a kernel asks memory for and cost nothing until the data is needed): the whole groups of 64
+// items of the piece, dealt over the waves; item `slot` of the LDS region comes from src[perm(slot)] (a wave's load
+// writes 64 consecutive 16-byte slots, lane l the l-th; where the data is read in another order the source index is
+// permuted instead). Returns the number of items covered; the caller copies the rest, waits (wait_vm) and synchronises.
+typedef __attribute__((address_space(3))) void* lds_ptr_t;
+template <class PERM>
+__device__ __forceinline__ uint32_t lds_dma_groups(uint32_t* dst, const uint4* src, uint32_t n16, uint32_t wave, uint32_t nwaves,
+                                                   uint32_t lane, PERM perm) {
+  const uint32_t groups = n16 >> 6;
+  for (uint32_t g = wave; g < groups; g += nwaves)
+    __builtin_amdgcn_global_load_lds((const MSQ_GLOBAL void*)(src + perm(64u * g + lane)), (lds_ptr_t)(dst + 256u * g), 16, 0, 0);
+  return groups << 6;
+}
+
 // table piece k of decoder D for copy_jobs (an empty piece when D stages no such table or is not in use)
 template <class D>
 __device__ __forceinline__ CopyJob tbl_job_of(int k, uint32_t at, bool live) {
@@ -429,11 +454,28 @@ __device__ __forceinline__ float sum_h2(const uint32_t* v, int n) {
 // 32-value slice is 16 words, read as it is. Staged in LDS, four words of padding follow every slice (20 words apart:
 // 16 consecutive lanes hit 16 different bank quads, as with XLds).
 __host__ __device__ constexpr uint32_t xhalf_words(uint32_t cols) { return (cols >> 5) * 20u; }
+// The same slices without padding, for copies that cannot pad (loads that write LDS directly): slice u takes 16 words and
+// its four 16-byte items are rotated by u / 2, item c at word 16 u + 4 ((c + (u >> 1)) & 3) -- sixteen consecutive lanes
+// reading their item c then touch every group of four banks exactly twice, the least a 16-byte read of sixteen lanes can.
+__device__ __forceinline__ uint32_t xhalf_rot_src(uint32_t slot) {  // the source item that belongs in 16-byte slot `slot`
+  const uint32_t u = slot >> 2;
+  return 4u * u + ((slot - (u >> 1)) & 3u);
+}
 __device__ __forceinline__ X32 load_x32_half(const uint32_t* p) {
   X32 r;
 #pragma unroll
   for (int i = 0; i < 4; i++) {
     const u32x4 q = ((const u32x4*)p)[i];
+    r.v[4 * i] = q.x; r.v[4 * i + 1] = q.y; r.v[4 * i + 2] = q.z; r.v[4 * i + 3] = q.w;
+  }
+  r.sx = sum_h2(r.v, 16);
+  return r;
+}
+__device__ __forceinline__ X32 load_x32_half_rot(const uint32_t* region, uint32_t u) {  // slice u of a region in the rotated layout
+  X32 r;
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    const u32x4 q = *(const u32x4*)(region + 16u * u + 4u * ((i + (u >> 1)) & 3u));
     r.v[4 * i] = q.x; r.v[4 * i + 1] = q.y; r.v[4 * i + 2] = q.z; r.v[4 * i + 3] = q.w;
   }
   r.sx = sum_h2(r.v, 16);
@@ -486,6 +528,7 @@ struct DecIQ1S {
   }
   // the same bytes through a buffer descriptor: Off holds the lane's byte offsets inside a row, soff the row's offset
   struct Off { uint32_t qs, qh, d; };
+  static constexpr int FETCH_LOADS = 3;  // loads of one fetch()
   __device__ static Off offsets(uint32_t u) {
     const uint32_t b = (u >> 3) * 50u, ib = u & 7u;
     return {b + 2 + 4 * ib, b + 34 + 2 * ib, b};
@@ -571,6 +614,7 @@ struct DecIQ2XXS {
     return {a.x, a.y, ld16(b)};
   }
   struct Off { uint32_t a, d; };
+  static constexpr int FETCH_LOADS = 2;  // loads of one fetch()
   __device__ static Off offsets(uint32_t u) {
     const uint32_t b = (u >> 3) * 66u;
     return {b + 2 + 8 * (u & 7u), b};

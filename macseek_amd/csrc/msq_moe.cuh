@@ -72,9 +72,10 @@ __device__ __forceinline__ void store_h(const MoeArgs& a, size_t i, float v) {
 template <class DR, class DS>
 constexpr bool kHalfH = std::is_same_v<typename DR::X, X32> && std::is_same_v<typename DS::X, X32>;
 // the lane's slice (unit u) of the h row that starts at column col0 of the staged rows hs / of the rows in device memory
-template <class D, bool HALF>
+template <class D, bool HALF, bool ROT = false>
 __device__ __forceinline__ typename D::X load_h_staged(const uint32_t* hs, uint32_t col0, uint32_t u) {
-  if constexpr (HALF) return load_x32_half(hs + xhalf_words(col0) + 20u * u);
+  if constexpr (HALF && ROT) return load_x32_half_rot(hs, (col0 >> 5) + u);
+  else if constexpr (HALF) return load_x32_half(hs + xhalf_words(col0) + 20u * u);
   else return D::load_x(XLds{(const float*)hs + xlds_words(col0)}, u, kHScale);
 }
 template <class D, bool HALF>
@@ -544,9 +545,35 @@ __global__ __launch_bounds__(MAXT) void moe_down_kernel(const uint64_t* table, c
     const uint32_t run = uniform(small_div(n + RW - 1, RW));
     const uint32_t w0 = uniform(min(c0 + rg * run, c1)), w1 = uniform(min(w0 + run, c1));
 
+    // Codebook pairs that take h as fp16: tables and h rows come by loads that write LDS themselves, requested ahead of
+    // everything else (no registers are held for them, and they return -- loads return in order -- ahead of the first
+    // weight rows' trip to HBM instead of behind it); what does not fill a group of 64 items goes through one register.
+    constexpr bool DMA = RING_R && RING_S && HALF && MAXT <= 768;  // (the 1024-thread instantiations have no registers to spare)
+    [[maybe_unused]] u32x4 rest[4];
+    [[maybe_unused]] uint32_t rest_at[4] = {0u, 0u, 0u, 0u};  // LDS word offset + 1 of the thread's leftover item, 0: none
+    if constexpr (DMA) {
+      if (first && a.stage_x) {
+        const uint32_t lo = NE ? 0u : a.n_routed * a.inter;
+        const uint32_t hi = (a.run_shared ? a.n_routed + 1u : a.n_routed) * a.inter;
+        const CopyJob jobs[5] = {tbl_job_of<DR>(0, 0u, NE), tbl_job_of<DR>(1, 0u, NE), tbl_job_of<DS>(0, DR::LDS_WORDS, a.run_shared),
+                                 tbl_job_of<DS>(1, DR::LDS_WORDS, a.run_shared),
+                                 {(const uint4*)(a.h16 + lo), (uint32_t)(smem - tbl) + a.xs_off, (hi - lo) / 8u, 0u}};
+        auto same = [](uint32_t i) { return i; };
+#pragma unroll
+        for (int j = 0; j < 5; j++) {
+          if (jobs[j].n16 == 0) continue;
+          const uint32_t done = j == 4 ? lds_dma_groups(tbl + jobs[j].dst, jobs[j].src, jobs[j].n16, wave, nwaves, lane, xhalf_rot_src)
+                                       : lds_dma_groups(tbl + jobs[j].dst, jobs[j].src, jobs[j].n16, wave, nwaves, lane, same);
+          if (j < 4 && done + tid < jobs[j].n16) {  // (the h rows are whole groups: inter is a multiple of 256)
+            rest[j] = *(const u32x4*)(jobs[j].src + done + tid);
+            rest_at[j] = jobs[j].dst + 4u * (done + tid) + 1u;
+          }
+        }
+      }
+    }
     // the value of y that this thread adds to in the epilogue, requested ahead of the rows (14.3 -> 14.15 us)
     float yq = 0.f;
-    if (tid < n) yq = a.y[c0 + tid];
+    if (!DMA && tid < n) yq = a.y[c0 + tid];
     // ---- request the first rows of both matrices
     typename DR::Raw cur[RING_R ? 1 : RPW], nxt[RING_R ? 1 : RPW];
     uint32_t pv = w0;  // routed ring cursor
@@ -571,6 +598,21 @@ __global__ __launch_bounds__(MAXT) void moe_down_kernel(const uint64_t* table, c
     } else if (NE && w0 < w1) {
 #pragma unroll
       for (int j = 0; j < RPW; j++) cur[j] = DR::load(Dr + (size_t)min(w0 + j, w1 - 1) * a.rb_d_r, unit_r);
+    }
+    if constexpr (DMA) yq = a.y[c0 + min(tid, n - 1u)];  // (every wave: the wait below counts the loads behind the copy)
+    if (DMA && first && a.stage_x) {
+      wait_vm<NR * DR::FETCH_LOADS + 1>();  // everything older than the routed ring and y: the copy
+#pragma unroll
+      for (int j = 0; j < 4; j++)
+        if (rest_at[j]) *(u32x4*)(tbl + rest_at[j] - 1u) = rest[j];
+      const uint32_t lo = NE ? 0u : a.n_routed * a.inter;
+      const uint32_t* hs = smem + a.xs_off;
+      __syncthreads();
+      if (NE) xr = load_h_staged<DR, HALF, true>(hs, e * a.inter, unit_r);
+      if (a.run_shared) xs = load_h_staged<DS, HALF, true>(hs, a.n_routed * a.inter - lo, unit_s);
+      if (!valid_r) xr = typename DR::X{};
+      if (!valid_s) xs = typename DS::X{};
+      first = false;
     }
     if (first) {
       // h rows this launch reads: the routed ones [0, NE), then the shared one at n_routed (NE is 0 or n_routed)

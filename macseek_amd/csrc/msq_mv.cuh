@@ -357,17 +357,8 @@ __device__ __forceinline__ uint32_t wspan_len(uint32_t units, uint32_t ks) {
   } else return 0u;
 }
 
-// Waits until at most N of the wave's vector memory operations are outstanding, and keeps the compiler from moving memory
-// accesses across the wait (s_waitcnt: the count's low four bits in bits 0-3, its high two in bits 14-15; the other
-// counters at their maxima, i.e. not waited for).
 template <int N>
-__device__ __forceinline__ void wait_rows() {
-  static_assert(N >= 0 && N < 64, "s_waitcnt holds six bits of vmcnt");
-  asm volatile("" ::: "memory");
-  __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
-  asm volatile("" ::: "memory");
-}
-
+__device__ __forceinline__ void wait_rows() { wait_vm<N>(); }
 // the same for a count that is a constant only after unrolling (0 .. 9)
 __device__ __forceinline__ void wait_rows_n(int n) {
   switch (n) {
