@@ -373,9 +373,12 @@ typedef __attribute__((address_space(3))) void* lds_ptr_t;
 template <class PERM>
 __device__ __forceinline__ uint32_t lds_dma_groups(uint32_t* dst, const uint4* src, uint32_t n16, uint32_t wave, uint32_t nwaves,
                                                    uint32_t lane, PERM perm) {
+  // (the buffer form of the load: the compiler orders later LDS reads behind the global form with waits for every
+  // outstanding load, which would serialise a kernel's weight-row pipeline; callers wait explicitly instead)
   const uint32_t groups = n16 >> 6;
+  const rsrc_t rs = make_rsrc(src, n16 * 16u);
   for (uint32_t g = wave; g < groups; g += nwaves)
-    __builtin_amdgcn_global_load_lds((const MSQ_GLOBAL void*)(src + perm(64u * g + lane)), (lds_ptr_t)(dst + 256u * g), 16, 0, 0);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lds_ptr_t)(dst + 256u * g), 16, (int)(16u * perm(64u * g + lane)), 0, 0, 0);
   return groups << 6;
 }
 
