@@ -74,6 +74,9 @@ CASES = [
     (O.Q8_0, 1024, 2048, 2, False, "staged x, groups"), (O.IQ2_XXS, 2048, 1024, 8, False, "staged x, groups"),
     (O.IQ2_XXS, 16, 36864, 1, False, "row too long for LDS"), (O.Q8_0, 8, 16384, 1, True, "row too long for LDS acc"),
     (O.IQ1_S, 600, 12288, 1, False, "long staged row"),
+    # weight rows through LDS (large Q6_K / Q8_0 matrices): ragged row counts, a row that ends in a short wave slice
+    (O.Q6_K, 4099, 4096, 1, False, "large q6_k, ragged rows"), (O.Q6_K, 3001, 5376, 1, True, "large q6_k, 21 blocks per row acc"),
+    (O.Q8_0, 8201, 5120, 1, True, "large q8_0 acc"), (O.Q8_0, 16400, 2592, 1, False, "large q8_0, 81 blocks per row"),
 ]
 
 
