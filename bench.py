@@ -836,8 +836,9 @@ def bench_matmul(torch, args):
     from macseek_amd import quant as q
     dev = torch.device("cuda:0")
     rows_out = []
-    # n = 2048 and 512: dequantize-then-GEMM; n <= 128 (<= 256 on matrices of at most 2048 rows): the fused kernel
-    # (mm_fused_kernel); "route" names which one served the case
+    # n = 2048 and 512: dequantize-then-GEMM; n <= 128 (<= 256 on matrices of at most 2048 rows and on K-quants): the fused
+    # kernel (mm_fused_kernel); 65..256 tokens on large IQ4_NL / Q8_0 / codebook matrices: mm_tile_kernel; "route" names
+    # which one served the case
     cases = [(2048, q.QType.Q6_K, "Q6_K", 1536, 7168), (2048, q.QType.Q5_K, "Q5_K", 512, 7168),
              (2048, q.QType.IQ4_NL, "IQ4_NL", 7168, 4096), (2048, q.QType.BF16, "BF16", 384, 7168)]
     for n in (512, 256, 128, 64, 16):
@@ -863,9 +864,10 @@ def bench_matmul(torch, args):
         torch.cuda.synchronize()
         ms = a.elapsed_time(b) / reps
         flops = 2.0 * n * rows * cols
-        fused = n <= 128 or (n <= 256 and rows <= 2048)
+        tile = name in ("IQ4_NL", "Q8_0", "IQ1_S", "IQ2_XXS") and 65 <= n <= 256 and rows * cols >= 12000000
+        fused = n <= 128 or (n <= 256 and (rows <= 2048 or name in ("Q6_K", "Q5_K")))
         rows_out.append({"type": name, "rows": rows, "cols": cols, "n": n, "us_per_call": ms * 1e3, "TFLOPs": flops / (ms * 1e-3) / 1e12,
-                         "route": "mm_fused_kernel" if fused else "dequant + rocBLAS"})
+                         "route": "mm_tile_kernel" if tile else "mm_fused_kernel" if fused else "dequant + rocBLAS"})
     head = rows_out[0]
     n = 2048
     cpu = None

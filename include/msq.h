@@ -122,17 +122,22 @@ int msq_f32_to_f16(void* stream, const MsqBuffer* X, const MsqBuffer* X16, size_
 /* reference: ms::q::encode_matmul_h (quant.hpp:43-45, quant.mm:193-238). Prefill matmul
  * Y[n x rows] (+)= X16[n x x_stride] . W^T, X16 fp16 (x_stride = cols if 0), Y F32, any n >= 1, cols % 128 == 0.
  * Weights are rounded to fp16 and products accumulate in fp32, the reference's numerics (quant.hpp:36-39).
- * Up to 128 tokens (256 on matrices of at most 2048 rows; MSQ_MM_FUSED_MAX=N in the environment: up to N) a fused
- * kernel serves the call: nothing is allocated and the call only enqueues. When the matrix has few tiles K is cut into
- * slices whose partial sums pass through a 32 MB buffer inside the library and are added in order (results repeat bit for
- * bit; calls on this route share the buffer: one stream at a time). Above, an fp16 copy of W goes to scratch that the library owns (reference: quant.mm:176-184): that
+ * Up to 128 tokens (256 on matrices of at most 2048 rows and on Q6_K / Q5_K; MSQ_MM_FUSED_MAX=N in the environment: up
+ * to N) a fused kernel serves the call: nothing is allocated and the call only enqueues. When the matrix has few tiles K
+ * is cut into slices whose partial sums pass through a 32 MB buffer inside the library and are added in order (results
+ * repeat bit for bit; calls on this route share the buffer: one stream at a time). IQ1_S, IQ2_XXS, IQ4_NL and Q8_0
+ * matrices of 12 million weights and more take a second fused kernel from 65 to 256 tokens, which stages both operands
+ * through LDS (same numerics, same buffers; it wants activation rows on 16-byte boundaries, other strides stay with the
+ * first kernel). Above, an fp16 copy of W goes to scratch that the library owns (reference: quant.mm:176-184): that
  * scratch only grows (a larger shape allocates a new block, never waits for the stream; inside a stream capture a call
  * that would have to grow it fails with MSQ_ERR_SCRATCH), and calls sharing it must be enqueued on one stream at a time. */
 int msq_matmul_h(void* stream, int qtype, const MsqBuffer* W, int rows, int cols, const MsqBuffer* X16, const MsqBuffer* Y,
                  int n, int accumulate, int x_stride);
 
 /* reference: ms::q::encode_matmul (quant.hpp:40-41, quant.mm:240-248): converts X (F32 [n x cols], 16-byte aligned)
- * into library-owned fp16 scratch, then msq_matmul_h; the fused kernel reads the F32 activations as they are. */
+ * into library-owned fp16 scratch, then msq_matmul_h; the first fused kernel reads the F32 activations as they are, the
+ * second one an fp16 copy in a 16 MB buffer inside the library (shared like the partial sums; larger copies go to the
+ * growing scratch). */
 int msq_matmul(void* stream, int qtype, const MsqBuffer* W, int rows, int cols, const MsqBuffer* X, const MsqBuffer* Y, int n,
                int accumulate);
 

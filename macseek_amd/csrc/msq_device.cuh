@@ -170,6 +170,7 @@ struct LdsRow {
     return {base, at + (t & ~3u), t & 3u};
   }
 };
+__device__ __forceinline__ uint32_t ld8(const LdsRow& p) { return *(p.base + p.at + p.sh); }
 __device__ __forceinline__ uint32_t ld16(const LdsRow& p) { return *(const uint16_t*)(p.base + p.at + p.sh); }
 __device__ __forceinline__ uint32_t ld32(const LdsRow& p) {
   const uint32_t* q = (const uint32_t*)(p.base + p.at);
@@ -187,6 +188,36 @@ __device__ __forceinline__ u128_a2 ld128(const LdsRow& p) {
           __builtin_amdgcn_alignbyte(d4, d3, p.sh)};
 }
 
+// Loads in two parts, for kernels that request bytes ahead of the arithmetic on them: ldN_raw(p) only issues the
+// loads, fix() puts the bytes in place. For memory pointers the first part does everything; for LDS rows the aligned
+// words are read first and shifted when they are used (a shift right behind its read would wait for the read).
+struct Lds32Raw { uint32_t d0, d1, sh; };
+struct Lds64Raw { uint32_t d0, d1, d2, sh; };
+struct Lds128Raw { uint32_t d0, d1, d2, d3, d4, sh; };
+__device__ __forceinline__ Lds32Raw ld32_raw(const LdsRow& p) {
+  const uint32_t* q = (const uint32_t*)(p.base + p.at);
+  return {q[0], q[1], p.sh};
+}
+__device__ __forceinline__ Lds64Raw ld64_raw(const LdsRow& p) {
+  const uint32_t* q = (const uint32_t*)(p.base + p.at);
+  return {q[0], q[1], q[2], p.sh};
+}
+__device__ __forceinline__ Lds128Raw ld128_raw(const LdsRow& p) {
+  const uint32_t* q = (const uint32_t*)(p.base + p.at);
+  return {q[0], q[1], q[2], q[3], q[4], p.sh};
+}
+__device__ __forceinline__ uint32_t fix(const Lds32Raw& r) { return __builtin_amdgcn_alignbyte(r.d1, r.d0, r.sh); }
+__device__ __forceinline__ u64_a2 fix(const Lds64Raw& r) {
+  return {__builtin_amdgcn_alignbyte(r.d1, r.d0, r.sh), __builtin_amdgcn_alignbyte(r.d2, r.d1, r.sh)};
+}
+__device__ __forceinline__ u128_a2 fix(const Lds128Raw& r) {
+  return {__builtin_amdgcn_alignbyte(r.d1, r.d0, r.sh), __builtin_amdgcn_alignbyte(r.d2, r.d1, r.sh),
+          __builtin_amdgcn_alignbyte(r.d3, r.d2, r.sh), __builtin_amdgcn_alignbyte(r.d4, r.d3, r.sh)};
+}
+__device__ __forceinline__ uint32_t fix(uint32_t v) { return v; }
+__device__ __forceinline__ u64_a2 fix(const u64_a2& v) { return v; }
+__device__ __forceinline__ u128_a2 fix(const u128_a2& v) { return v; }
+
 #define MSQ_LOADERS(AS)                                                                                               \
   __device__ __forceinline__ uint32_t ld8(const AS uint8_t* p) { return *p; }                                         \
   __device__ __forceinline__ uint32_t ld16(const AS uint8_t* p) { return *(const AS uint16_t*)p; }                    \
@@ -198,7 +229,10 @@ __device__ __forceinline__ u128_a2 ld128(const LdsRow& p) {
   __device__ __forceinline__ u128_a2 ld128(const AS uint8_t* p) {                                                     \
     const u32x4_a2 v = *(const AS u32x4_a2*)p;                                                                        \
     return {v.x, v.y, v.z, v.w};                                                                                      \
-  }
+  }                                                                                                                   \
+  __device__ __forceinline__ uint32_t ld32_raw(const AS uint8_t* p) { return ld32(p); }                               \
+  __device__ __forceinline__ u64_a2 ld64_raw(const AS uint8_t* p) { return ld64(p); }                                 \
+  __device__ __forceinline__ u128_a2 ld128_raw(const AS uint8_t* p) { return ld128(p); }
 MSQ_LOADERS()
 MSQ_LOADERS(MSQ_GLOBAL)
 #undef MSQ_LOADERS
@@ -370,6 +404,16 @@ __device__ __forceinline__ void wait_vm() {
 // writes 64 consecutive 16-byte slots, lane l the l-th; where the data is read in another order the source index is
 // permuted instead). Returns the number of items covered; the caller copies the rest, waits (wait_vm) and synchronises.
 typedef __attribute__((address_space(3))) void* lds_ptr_t;
+// The same load, hidden from the compiler: it follows the builtin's LDS writes and puts a wait for every outstanding
+// load in front of each LDS read it cannot prove disjoint from them (a read of one half of a double buffer while the
+// other half is being filled), which would expose a full trip to memory per stage. Lane l's 16 bytes from byte
+// offset voff + soff of the descriptor land at dst + 16 l (dst wave-uniform). Callers wait with wait_vm and must not
+// use the builtin forms of LDS-direct loads, movrel or other users of M0 in the same kernel: M0 is not restored.
+__device__ __forceinline__ void lds_dma16(rsrc_t rs, const void* dst, uint32_t voff, uint32_t soff) {
+  const uint32_t at = (uint32_t)(uintptr_t)(lds_ptr_t)dst;
+  // (a scalar write of M0 wants one wait state before an instruction that reads it as the LDS address)
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds" : : "s"(at), "v"(voff), "s"(rs), "s"(soff) : "memory");
+}
 template <class PERM>
 __device__ __forceinline__ uint32_t lds_dma_groups(uint32_t* dst, const uint4* src, uint32_t n16, uint32_t wave, uint32_t nwaves,
                                                    uint32_t lane, PERM perm) {

@@ -3,9 +3,11 @@
 //
 // The reference multiplies fp16 activations by weight tiles dequantized to fp16 inside its GEMM kernel and, from
 // n >= 512, dequantizes the whole matrix to fp16 once and runs a dense GEMM (quant.mm:204-221). The same two routes
-// exist here; the switch between them sits where they were measured to cross (use_fused below). Fused route:
+// exist here; the switch between them sits where they were measured to cross (use_fused, tile_ok below). Fused route:
 // mm_fused_kernel (msq_mm.cuh) decodes each weight tile straight into matrix-core fragments -- no fp16 copy of W or X,
-// nothing allocated, the call only enqueues; when the tiles alone would not fill the device K is cut into slices whose
+// nothing allocated, the call only enqueues; for large matrices of four formats at 65 to 256 tokens mm_tile_kernel
+// does the same with both operands staged through LDS (F32 activations are first rounded to fp16 rows in a
+// file-scope device buffer, which calls share like the partial sums); when the tiles alone would not fill the device K is cut into slices whose
 // partial sums go to a file-scope device buffer and are added in order by a second launch (no floating-point atomics:
 // results repeat bit for bit; calls on this route share the buffer and must be enqueued on one stream at a time).
 // Materialising route: the bit-exact dequantizer writes
@@ -46,12 +48,17 @@ rocblas_handle g_blas = nullptr;
 // Which calls the fused kernel serves. The reference switches to dequantize-then-GEMM at 512 tokens (quant.mm:204); here
 // the switch sits where the two routes were measured to cross on MI355X: the fused kernel wins up to 128 tokens on every
 // matrix tried (Q6_K 1536x7168 at 128 tokens: 22.5 us against 36 us; 16 tokens: 11 against 30) and up to 256 tokens on
-// matrices of at most 2048 rows; above, the materialising route is ahead (IQ4_NL 7168x4096 at 512 tokens: 63 us against
-// 124). MSQ_MM_FUSED_MAX = N makes the switch "up to N tokens" for every matrix (0: never fused).
-bool use_fused(int n, int rows) {
+// matrices of at most 2048 rows and on every Q6_K / Q5_K matrix (4096x4096 at 192 tokens: 32 us against 44); above, the
+// materialising route is ahead (IQ4_NL 7168x4096 at 512 tokens: 63 us against 124). MSQ_MM_FUSED_MAX = N makes the
+// switch "up to N tokens" for every matrix (0: never fused).
+int fused_forced() {
   static const int forced = [] { const char* e = getenv("MSQ_MM_FUSED_MAX"); return e && *e ? atoi(e) : -1; }();
+  return forced;
+}
+bool use_fused(int t, int n, int rows) {
+  const int forced = fused_forced();
   if (forced >= 0) return n <= forced;
-  return n <= 128 || (n <= 256 && rows <= 2048);
+  return n <= 128 || (n <= 256 && (rows <= 2048 || t == MSQ_Q6_K || t == MSQ_Q5_K));
 }
 
 // at least `bytes` of device memory in s (>= 64 MiB like the reference's, quant.mm:176-183)
@@ -147,6 +154,16 @@ int splitk_limit() {
   return v;
 }
 
+// token counts that take the tile kernel (MSQ_MM_TILE_MIN / MSQ_MM_TILE_MAX: experiments; a huge minimum switches it off)
+long tile_min_tokens() {
+  static const long v = [] { const char* e = getenv("MSQ_MM_TILE_MIN"); return e && *e ? atol(e) : 65L; }();
+  return v;
+}
+long tile_max_tokens() {
+  static const long v = [] { const char* e = getenv("MSQ_MM_TILE_MAX"); return e && *e ? atol(e) : 256L; }();
+  return v;
+}
+
 template <class F, bool X_F32>
 int launch_mm_t(hipStream_t st, MmArgs a) {
   const long cus = device_info().cus;
@@ -203,6 +220,88 @@ int launch_mm(hipStream_t st, int t, const MmArgs& a) {
   return unsupported("matmul", t, (int)a.rows, (int)a.cols);
 }
 
+// The tile kernel (fp16 activations in memory): eight waves of one row tile each, 128 rows x 128 or 256 tokens per
+// workgroup (256 when the call has the tokens: a decoded fragment then feeds sixteen matrix instructions), one
+// workgroup per CU, K cut into slices of whole weight stages until every CU has one.
+template <class F, int TM, int XK>
+int launch_tile_c(hipStream_t st, MmArgs a) {
+  constexpr int WV = 8, RT = 1;
+  constexpr int P = ((F::WS_BYTES + 14 + 15) / 16) | 1, NPI = (16 * WV * RT * P + 64 * WV - 1) / (64 * WV);
+  const long cus = device_info().cus;
+  const uint32_t nstages = a.cols / XK, xpw = 256 / XK;
+  const size_t lds = (size_t)F::LDS_WORDS * 4 + 2 * (size_t)16 * TM * XK * 2 + 2 * (size_t)NPI * 64 * WV * 16 +
+                     (NPI * 64 * WV > 16 * WV * RT * P ? 0 : 16);  // (a fragment read may end a few bytes past its row's pieces)
+  const int rc = allow_large_lds(mm_tile_kernel<F, WV, RT, TM, XK>, lds);
+  if (rc != MSQ_OK) return rc;
+  const long gx = (a.rows + 16 * WV * RT - 1) / (16 * WV * RT), gy = (a.n + 16 * TM - 1) / (16 * TM);
+  const size_t cnt = (size_t)a.n * a.rows;
+  const long wstages = (nstages + xpw - 1) / xpw;  // weight stages (256 columns) of a row
+  long kz = std::min<long>(std::max<long>(1, cus / (gx * gy)), std::max<long>(1, wstages / 2));
+  kz = std::min<long>(kz, std::max<long>(1, (long)(kMmPartialBytes / (cnt * 4))));
+  if (splitk_limit() > 0) kz = std::min<long>(kz, splitk_limit());
+  float* partials = kz > 1 ? mm_partials() : nullptr;
+  if (!partials) kz = 1;
+  const long per = (wstages + kz - 1) / kz;
+  a.slice_stages = (uint32_t)(per * xpw);
+  kz = (wstages + per - 1) / per;
+  a.partials = kz > 1 ? partials : nullptr;
+  hipLaunchKernelGGL((mm_tile_kernel<F, WV, RT, TM, XK>), dim3((unsigned)gx, (unsigned)gy, (unsigned)kz), dim3(64 * WV), lds, st, a.X, a.W, a.Y,
+                     a.n, a.rows, a.cols, a.x_stride, a.row_bytes, a.accumulate, a.slice_stages, a.partials);
+  if (a.partials)
+    hipLaunchKernelGGL(mm_reduce_kernel, dim3((unsigned)((cnt + 255) / 256)), dim3(256), 0, st, (const float*)a.partials, a.Y, cnt, (uint32_t)kz,
+                       a.accumulate);
+  MSQ_HIP(hipGetLastError());
+  return MSQ_OK;
+}
+template <class F>
+int launch_tile_t(hipStream_t st, const MmArgs& a) {
+  return a.n >= 192 ? launch_tile_c<F, 16, 64>(st, a) : launch_tile_c<F, 8, 128>(st, a);
+}
+int launch_tile(hipStream_t st, int t, const MmArgs& a) {
+  switch (t) {
+    case MSQ_Q8_0: return launch_tile_t<FragQ8_0>(st, a);
+    case MSQ_IQ4_NL: return launch_tile_t<FragIQ4NL>(st, a);
+    case MSQ_IQ1_S: return launch_tile_t<FragIQ1S>(st, a);
+    case MSQ_IQ2_XXS: return launch_tile_t<FragIQ2XXS>(st, a);
+  }
+  return unsupported("matmul", t, (int)a.rows, (int)a.cols);
+}
+// Which calls take it, from what was measured against the two other routes on MI355X: the codebook formats, Q8_0 and
+// IQ4_NL, matrices of twelve million weights and more, 65 to 256 tokens (IQ2_XXS 4096x7168 at 128 tokens: 30 us against
+// 35 fused / 53 materialised; Q8_0 4096x4096 at 256: 33 against 45 / 34; beyond 256 tokens the dense GEMM on the
+// materialised matrix is ahead, and on smaller matrices the kernel above; Q6_K and Q5_K gain 6 % at best and stay
+// with the two other routes). MSQ_MM_TILE_MIN / _MAX / _ELEMS move the bounds. Also required: the matrix and the
+// activations each below 4 GiB (a buffer descriptor spans them), activation rows on 16-byte boundaries.
+bool tile_ok(int t, int n, int rows, int cols, size_t x_stride, const void* X16) {
+  switch (t) {
+    case MSQ_Q8_0: case MSQ_IQ4_NL: case MSQ_IQ1_S: case MSQ_IQ2_XXS: break;
+    default: return false;
+  }
+  static const long min_elems = [] { const char* e = getenv("MSQ_MM_TILE_ELEMS"); return e && *e ? atol(e) : 12000000L; }();
+  const size_t lim = ((size_t)1 << 32) - 64;
+  if (fused_forced() >= 0 && n > fused_forced()) return false;
+  return n >= tile_min_tokens() && n <= tile_max_tokens() && (long)rows * cols >= min_elems &&
+         (size_t)rows * msq_type_row_bytes(t, cols) < lim && ((size_t)(n - 1) * x_stride + cols) * 2 < lim && x_stride % 8 == 0 &&
+         ((uintptr_t)X16 & 15) == 0;
+}
+
+// fp16 copy of the activations for the tile kernel: a file-scope device array (nothing allocated, capturable) while
+// it is large enough, the growing scratch above otherwise. Like the partial sums it is shared by the calls of a device.
+constexpr size_t kMmX16Bytes = (size_t)16 << 20;
+__device__ __align__(256) uint16_t g_mm_x16[kMmX16Bytes / 2];
+uint16_t* g_mm_x16_ptr[16] = {};
+uint16_t* mm_x16() {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 16) return nullptr;
+  std::lock_guard<std::mutex> lock(g_mu);
+  if (!g_mm_x16_ptr[dev]) {
+    void* p = nullptr;
+    if (hipGetSymbolAddress(&p, HIP_SYMBOL(g_mm_x16)) != hipSuccess) { (void)hipGetLastError(); return nullptr; }
+    g_mm_x16_ptr[dev] = (uint16_t*)p;
+  }
+  return g_mm_x16_ptr[dev];
+}
+
 // more tokens than the fused kernel takes: W as fp16 in scratch (F16 weights are the GEMM operand as they are), then the dense GEMM
 int matmul_big(hipStream_t st, int t, const MsqBuffer* W, int rows, int cols, const uint16_t* X16, float* Y, int n, bool accumulate,
                int x_stride) {
@@ -219,7 +318,7 @@ int matmul_big(hipStream_t st, int t, const MsqBuffer* W, int rows, int cols, co
 
 }  // namespace
 
-void matmul_partials_setup() { (void)mm_partials(); }
+void matmul_partials_setup() { (void)mm_partials(); (void)mm_x16(); }
 
 }  // namespace msq
 
@@ -246,7 +345,12 @@ int msq_matmul_h(void* stream, int t, const MsqBuffer* W, int rows, int cols, co
     return fail(MSQ_ERR_ARGUMENT, "macseek quant: matmul: buffer missing, too small or misaligned (type %s rows %d cols %d n %d)",
                 msq_type_name_of(t), rows, cols, n);
   hipStream_t st = (hipStream_t)stream;
-  if (use_fused(n, rows)) {
+  if (tile_ok(t, n, rows, cols, (size_t)xs, bptr(X16))) {
+    const MmArgs a{bptr(X16), bptr(W), (float*)bptr_mut(Y), (uint32_t)n, (uint32_t)rows, (uint32_t)cols, (uint32_t)xs,
+                   (uint32_t)msq_type_row_bytes(t, cols), accumulate ? 1u : 0u};
+    return launch_tile(st, t, a);
+  }
+  if (use_fused(t, n, rows)) {
     const MmArgs a{bptr(X16), bptr(W), (float*)bptr_mut(Y), (uint32_t)n, (uint32_t)rows, (uint32_t)cols, (uint32_t)xs,
                    (uint32_t)msq_type_row_bytes(t, cols), accumulate ? 1u : 0u};
     return launch_mm<false>(st, t, a);
@@ -263,7 +367,24 @@ int msq_matmul(void* stream, int t, const MsqBuffer* W, int rows, int cols, cons
     return fail(MSQ_ERR_ARGUMENT, "macseek quant: matmul: buffer missing, too small or misaligned (type %s rows %d cols %d n %d)",
                 msq_type_name_of(t), rows, cols, n);
   hipStream_t st = (hipStream_t)stream;
-  if (use_fused(n, rows)) {
+  if (tile_ok(t, n, rows, cols, (size_t)cols, nullptr)) {
+    // the activations as fp16 rows first (one pass over X; every workgroup of the tile kernel then fetches half the bytes)
+    const size_t xbytes = (size_t)n * cols * 2;
+    uint16_t* x16 = xbytes <= kMmX16Bytes ? mm_x16() : nullptr;
+    std::unique_lock<std::mutex> lock(g_mu, std::defer_lock);
+    if (!x16) {
+      lock.lock();
+      const int rc = reserve(g_x16, xbytes, st);
+      if (rc != MSQ_OK) return rc;
+      x16 = (uint16_t*)g_x16.p;
+    }
+    const int rx = launch_f32_to_f16(st, (const float*)bptr(X), x16, (size_t)n * cols);
+    if (rx != MSQ_OK) return rx;
+    const MmArgs a{x16, bptr(W), (float*)bptr_mut(Y), (uint32_t)n, (uint32_t)rows, (uint32_t)cols, (uint32_t)cols,
+                   (uint32_t)msq_type_row_bytes(t, cols), accumulate ? 1u : 0u};
+    return launch_tile(st, t, a);
+  }
+  if (use_fused(t, n, rows)) {
     const MmArgs a{bptr(X), bptr(W), (float*)bptr_mut(Y), (uint32_t)n, (uint32_t)rows, (uint32_t)cols, (uint32_t)cols,
                    (uint32_t)msq_type_row_bytes(t, cols), accumulate ? 1u : 0u};
     return launch_mm<true>(st, t, a);  // X is rounded to fp16 on its way into LDS

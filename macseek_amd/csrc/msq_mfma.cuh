@@ -47,7 +47,9 @@ __device__ __forceinline__ uint32_t bf16_rne(float f) {
 //   HAS_ADD            weight = scale * payload + add
 //   LDS_WORDS, fill_lds
 //   col_of(q, p)       column (0..31 inside the step) that position p of chunk q stands for
-//   get(row, step, q, tbl, h, scale, add)   payloads of the 8 weights of weight row `row` (pointer to its first byte)
+//   get(row, step, q, tbl)   payloads of the 8 weights of weight row `row` (pointer to its first byte); the block
+//                            formats split it into load_raw (the lane's bytes: loads only) and finish (table lookups
+//                            and arithmetic), so that a kernel can request a step's bytes ahead of its arithmetic
 struct FragOut {
   uint32_t h[4];
   float scale, add;
@@ -55,61 +57,86 @@ struct FragOut {
 
 struct FragIQ1S {
   static constexpr bool BF16_MATH = false, HAS_ADD = false;
+  static constexpr int WS_BYTES = 50;  // bytes of a row per 256 columns
   static constexpr int LDS_WORDS = MSQ_IQ1S_GRID_N * 4;
   __device__ static void fill_lds(uint32_t* lds, int tid, int nt) { copy_words16(lds, g_tbl_iq1s.w, LDS_WORDS, tid, nt); }
   __device__ static uint32_t col_of(uint32_t q, uint32_t p) { return 8u * q + p; }
+  struct Raw { uint32_t qh, qs, d; };
   template <class P>
-  __device__ static FragOut get(P row, uint32_t step, uint32_t q, const uint32_t* tbl) {
+  __device__ static Raw load_raw(P row, uint32_t step, uint32_t q) {
     const P b = row + (step >> 3) * 50u;
     const uint32_t ib = step & 7u;
-    const uint32_t qh = ld16(b + 34 + 2 * ib);
-    const uint32_t idx = ld8(b + 2 + 4 * ib + q) | (((qh >> (3 * q)) & 7u) << 8);
+    return {ld16(b + 34 + 2 * ib), ld8(b + 2 + 4 * ib + q), ld16(b)};
+  }
+  __device__ static FragOut finish(const Raw& r, uint32_t, uint32_t q, const uint32_t* tbl) {
+    const uint32_t qh = r.qh;
+    const uint32_t idx = r.qs | (((qh >> (3 * q)) & 7u) << 8);
     const uint4 g = ((const uint4*)tbl)[idx];
     const uint32_t delta2 = (qh & 0x8000u) ? 0xB000B000u : 0x30003000u;  // -0.125 / +0.125 in both halves
     FragOut o;
     o.h[0] = pk_add_f16(g.x, delta2); o.h[1] = pk_add_f16(g.y, delta2);  // grid + delta is exact in fp16
     o.h[2] = pk_add_f16(g.z, delta2); o.h[3] = pk_add_f16(g.w, delta2);
-    o.scale = half_bits_to_float(ld16(b)) * (float)(2u * ((qh >> 12) & 7u) + 1u);
+    o.scale = half_bits_to_float(r.d) * (float)(2u * ((qh >> 12) & 7u) + 1u);
     o.add = 0.f;
     return o;
   }
+  template <class P>
+  __device__ static FragOut get(P row, uint32_t step, uint32_t q, const uint32_t* tbl) { return finish(load_raw(row, step, q), step, q, tbl); }
 };
 
 struct FragIQ2XXS {
   static constexpr bool BF16_MATH = false, HAS_ADD = false;
+  static constexpr int WS_BYTES = 66;  // bytes of a row per 256 columns
   static constexpr int LDS_WORDS = MSQ_IQ2XXS_GRID_N * 4 + 128 * 4;
   __device__ static void fill_lds(uint32_t* lds, int tid, int nt) { DecIQ2XXS::fill_lds(lds, tid, nt); }
   __device__ static uint32_t col_of(uint32_t q, uint32_t p) { return 8u * q + p; }
+  template <class W32>
+  struct Raw { W32 a1; uint32_t gi, d; };
   template <class P>
-  __device__ static FragOut get(P row, uint32_t step, uint32_t q, const uint32_t* tbl) {
+  __device__ static auto load_raw(P row, uint32_t step, uint32_t q) {
     const P b = row + (step >> 3) * 66u;
     const P a8 = b + 2 + 8 * (step & 7u);
-    const uint32_t a1 = ld32(a8 + 4);
-    const uint4 g = ((const uint4*)tbl)[ld8(a8 + q)];
+    return Raw<decltype(ld32_raw(a8))>{ld32_raw(a8 + 4), ld8(a8 + q), ld16(b)};
+  }
+  template <class R>
+  __device__ static FragOut finish(const R& r, uint32_t, uint32_t q, const uint32_t* tbl) {
+    const uint32_t a1 = fix(r.a1);
+    const uint4 g = ((const uint4*)tbl)[r.gi];
     const uint4 s = ((const uint4*)(tbl + MSQ_IQ2XXS_GRID_N * 4))[(a1 >> (7 * q)) & 127u];
     FragOut o;
     o.h[0] = g.x ^ s.x; o.h[1] = g.y ^ s.y; o.h[2] = g.z ^ s.z; o.h[3] = g.w ^ s.w;
-    o.scale = half_bits_to_float(ld16(b)) * (0.5f + (float)(a1 >> 28)) * 0.25f;
+    o.scale = half_bits_to_float(r.d) * (0.5f + (float)(a1 >> 28)) * 0.25f;
     o.add = 0.f;
     return o;
   }
+  template <class P>
+  __device__ static FragOut get(P row, uint32_t step, uint32_t q, const uint32_t* tbl) { return finish(load_raw(row, step, q), step, q, tbl); }
 };
 
 struct FragQ8_0 {
   static constexpr bool BF16_MATH = false, HAS_ADD = false;
+  static constexpr int WS_BYTES = 272;  // bytes of a row per 256 columns
   static constexpr int LDS_WORDS = 0;
   __device__ static void fill_lds(uint32_t*, int, int) {}
   __device__ static uint32_t col_of(uint32_t q, uint32_t p) { return 8u * q + p; }
+  template <class W64>
+  struct Raw { W64 v; uint32_t d; };
   template <class P>
-  __device__ static FragOut get(P row, uint32_t step, uint32_t q, const uint32_t*) {
+  __device__ static auto load_raw(P row, uint32_t step, uint32_t q) {
     const P b = row + step * 34u;
-    const u64_a2 v = ld64(b + 2 + 8 * q);
+    return Raw<decltype(ld64_raw(b))>{ld64_raw(b + 2 + 8 * q), ld16(b)};
+  }
+  template <class P>
+  __device__ static FragOut get(P row, uint32_t step, uint32_t q, const uint32_t* tbl) { return finish(load_raw(row, step, q), step, q, tbl); }
+  template <class R>
+  __device__ static FragOut finish(const R& r, uint32_t, uint32_t, const uint32_t*) {
+    const u64_a2 v = fix(r.v);
     const uint32_t lo = v.x ^ 0x80808080u, hi = v.y ^ 0x80808080u;  // bytes become q + 128
     const uint32_t bias = 0xE480E480u;                              // -1152 in both halves
     FragOut o;
     o.h[0] = pk_add_f16(bytes01_to_h2_1024(lo), bias); o.h[1] = pk_add_f16(bytes23_to_h2_1024(lo), bias);
     o.h[2] = pk_add_f16(bytes01_to_h2_1024(hi), bias); o.h[3] = pk_add_f16(bytes23_to_h2_1024(hi), bias);
-    o.scale = half_bits_to_float(ld16(b));
+    o.scale = half_bits_to_float(r.d);
     o.add = 0.f;
     return o;
   }
@@ -119,26 +146,36 @@ struct FragQ8_0 {
 // its positions (2i, 2i + 1) stand for columns (4q + i, 4q + i + 16) and one table lookup per byte yields both.
 struct FragIQ4NL {
   static constexpr bool BF16_MATH = false, HAS_ADD = false;
+  static constexpr int WS_BYTES = 144;  // bytes of a row per 256 columns
   static constexpr int LDS_WORDS = 256;
   __device__ static void fill_lds(uint32_t* lds, int tid, int nt) { copy_words16(lds, g_tbl_iq4nl.w, 256, tid, nt); }
   __device__ static uint32_t col_of(uint32_t q, uint32_t p) { return 4u * q + (p >> 1) + 16u * (p & 1u); }
   __device__ static uint32_t pos_of(uint32_t c) { return 8u * ((c & 15u) >> 2) + 2u * (c & 3u) + (c >> 4); }  // inverse of col_of
+  template <class W32>
+  struct Raw { W32 v; uint32_t d; };
   template <class P>
-  __device__ static FragOut get(P row, uint32_t step, uint32_t q, const uint32_t* tbl) {
+  __device__ static auto load_raw(P row, uint32_t step, uint32_t q) {
     const P b = row + step * 18u;
-    const uint32_t v = ld32(b + 2 + 4 * q);
+    return Raw<decltype(ld32_raw(b))>{ld32_raw(b + 2 + 4 * q), ld16(b)};
+  }
+  template <class R>
+  __device__ static FragOut finish(const R& r, uint32_t, uint32_t, const uint32_t* tbl) {
+    const uint32_t v = fix(r.v);
     FragOut o;
     o.h[0] = tbl[v & 0xFFu]; o.h[1] = tbl[(v >> 8) & 0xFFu]; o.h[2] = tbl[(v >> 16) & 0xFFu]; o.h[3] = tbl[v >> 24];
-    o.scale = half_bits_to_float(ld16(b));
+    o.scale = half_bits_to_float(r.d);
     o.add = 0.f;
     return o;
   }
+  template <class P>
+  __device__ static FragOut get(P row, uint32_t step, uint32_t q, const uint32_t* tbl) { return finish(load_raw(row, step, q), step, q, tbl); }
 };
 
 // Q6_K: the 16-column scale groups are half a K step wide, so a step is issued as two MFMAs (chunks 0-1, chunks 2-3);
 // get() returns the scale of the lane's own half and get_scales() both halves' scales of the lane's row.
 struct FragQ6K {
   static constexpr bool BF16_MATH = false, HAS_ADD = false;
+  static constexpr int WS_BYTES = 210;  // bytes of a row per 256 columns
   static constexpr int LDS_WORDS = 0;
   __device__ static void fill_lds(uint32_t*, int, int) {}
   __device__ static uint32_t col_of(uint32_t q, uint32_t p) { return 8u * q + p; }
@@ -158,6 +195,31 @@ struct FragQ6K {
     o.add = 0.f;
     return o;
   }
+  template <class W64>
+  struct Raw { W64 ql, qh; uint32_t sc, d; };
+  template <class P>
+  __device__ static auto load_raw(P row, uint32_t step, uint32_t q) {
+    const P b = row + (step >> 3) * 210u;
+    const uint32_t e0 = 32u * (step & 7u) + 8u * q, h = e0 >> 7, k = (e0 & 127u) >> 5, l0 = e0 & 31u;
+    return Raw<decltype(ld64_raw(b))>{ld64_raw(b + 64 * h + 32 * (k & 1u) + l0), ld64_raw(b + 128 + 32 * h + l0),
+                                      ld16(b + 192 + 8 * h + 2 * k), ld16(b + 208)};
+  }
+  // (the scale of the lane's own half of the step: chunks 0-1 the first 16 columns, chunks 2-3 the second)
+  template <class R>
+  __device__ static FragOut finish(const R& r, uint32_t step, uint32_t q, const uint32_t*) {
+    const uint32_t k = step & 3u;
+    const uint32_t sh4 = 4u * (k >> 1), sh2 = 2u * k;
+    const u64_a2 ql = fix(r.ql), qh = fix(r.qh);
+    const uint32_t q0 = ((ql.x >> sh4) & 0x0F0F0F0Fu) | (((qh.x >> sh2) & 0x03030303u) << 4);
+    const uint32_t q1 = ((ql.y >> sh4) & 0x0F0F0F0Fu) | (((qh.y >> sh2) & 0x03030303u) << 4);
+    const uint32_t bias = 0xE420E420u;  // -1056 = -(1024 + 32) in both halves
+    FragOut o;
+    o.h[0] = pk_add_f16(bytes01_to_h2_1024(q0), bias); o.h[1] = pk_add_f16(bytes23_to_h2_1024(q0), bias);
+    o.h[2] = pk_add_f16(bytes01_to_h2_1024(q1), bias); o.h[3] = pk_add_f16(bytes23_to_h2_1024(q1), bias);
+    o.scale = half_bits_to_float(r.d) * (float)(int)(int8_t)(q < 2 ? r.sc & 0xFFu : r.sc >> 8);
+    o.add = 0.f;
+    return o;
+  }
   template <class P>
   __device__ static void get_scales(P row, uint32_t step, float& sa, float& sb) {
     const P b = row + (step >> 3) * 210u;
@@ -171,24 +233,35 @@ struct FragQ6K {
 
 struct FragQ5K {
   static constexpr bool BF16_MATH = false, HAS_ADD = true;
+  static constexpr int WS_BYTES = 176;  // bytes of a row per 256 columns
   static constexpr int LDS_WORDS = 0;
   __device__ static void fill_lds(uint32_t*, int, int) {}
   __device__ static uint32_t col_of(uint32_t q, uint32_t p) { return 8u * q + p; }
+  template <class W64, class W128>
+  struct Raw { W64 ql, qh; W128 hdr; };  // hdr: d | dmin, then the 12 scale bytes
   template <class P>
-  __device__ static FragOut get(P row, uint32_t step, uint32_t q, const uint32_t*) {
+  __device__ static auto load_raw(P row, uint32_t step, uint32_t q) {
     const P b = row + (step >> 3) * 176u;
-    const uint32_t is = step & 7u, g = is >> 1, run = is & 1u, l0 = 8u * q;
-    const u64_a2 ql = ld64(b + 48 + 32 * g + l0), qh = ld64(b + 16 + l0);
+    const uint32_t g = (step & 7u) >> 1, l0 = 8u * q;
+    return Raw<decltype(ld64_raw(b)), decltype(ld128_raw(b))>{ld64_raw(b + 48 + 32 * g + l0), ld64_raw(b + 16 + l0), ld128_raw(b)};
+  }
+  template <class P>
+  __device__ static FragOut get(P row, uint32_t step, uint32_t q, const uint32_t* tbl) { return finish(load_raw(row, step, q), step, q, tbl); }
+  template <class R>
+  __device__ static FragOut finish(const R& r, uint32_t step, uint32_t, const uint32_t*) {
+    const uint32_t is = step & 7u, run = is & 1u;
+    const u64_a2 ql = fix(r.ql), qh = fix(r.qh);
+    const u128_a2 hdr = fix(r.hdr);
     const uint32_t q0 = ((ql.x >> (4 * run)) & 0x0F0F0F0Fu) | (((qh.x >> is) & 0x01010101u) << 4);
     const uint32_t q1 = ((ql.y >> (4 * run)) & 0x0F0F0F0Fu) | (((qh.y >> is) & 0x01010101u) << 4);
     const uint32_t bias = 0xE400E400u;  // -1024 in both halves
-    // the 12 scale bytes, fetched unconditionally (a load inside a branch makes the waits that follow conservative)
-    const uint32_t s0 = ld32(b + 4), s1 = ld32(b + 8), s2 = ld32(b + 12);
+    // (all 12 scale bytes were fetched: a load inside a branch makes the waits that follow conservative)
+    const uint32_t s0 = hdr.y, s1 = hdr.z, s2 = hdr.w;
     auto byte = [&](uint32_t i) { const uint32_t w = i < 4 ? s0 : i < 8 ? s1 : s2; return (w >> (8 * (i & 3u))) & 0xFFu; };
     uint32_t sc, mn;
     if (is < 4) { sc = byte(is) & 63u; mn = byte(is + 4) & 63u; }
     else { sc = (byte(is + 4) & 0xFu) | ((byte(is - 4) >> 6) << 4); mn = (byte(is + 4) >> 4) | ((byte(is) >> 6) << 4); }
-    const uint32_t dd = ld32(b);
+    const uint32_t dd = hdr.x;
     FragOut o;
     o.h[0] = pk_add_f16(bytes01_to_h2_1024(q0), bias); o.h[1] = pk_add_f16(bytes23_to_h2_1024(q0), bias);
     o.h[2] = pk_add_f16(bytes01_to_h2_1024(q1), bias); o.h[3] = pk_add_f16(bytes23_to_h2_1024(q1), bias);

@@ -219,6 +219,216 @@ __global__ __launch_bounds__(64 * WV) void mm_fused_kernel(const void* X_, const
   }
 }
 
+// The same product for more tokens, block formats only, activations as fp16 rows in memory. The kernel above fetches a
+// lane's weight bytes straight from memory: sixteen rows per load instruction, a row per lane, so every load asks the
+// vector cache for sixteen or more lines, and its waves wait for every LDS read in front of the matrix instruction that
+// uses it. Here
+//  * weights and activations both come by loads that write LDS directly (no registers, no conversion, no address
+//    arithmetic per stage for the activations): the weight bytes of a weight stage (256 columns of the workgroup's
+//    16 WV RT rows) as consecutive aligned 16-byte pieces over consecutive lanes, every cache line asked for once; the
+//    activations of a stage ([16 TM tokens][XK columns]) one stage ahead, the 16-byte chunks of a token's row stored
+//    at slot (chunk ^ f(token)), so that the sixteen tokens of a fragment read hit sixteen different bank groups
+//    without padding;
+//  * the fragment decoders read the weight bytes from LDS (load_raw / finish); a decoded fragment feeds TM matrix
+//    instructions -- decoding costs about 37 vector instructions per fragment, a matrix instruction takes the time of
+//    3.5, so TM = 16 where the call has the tokens. Measured with TM = 16: the LDS is busy 88 % of the time (one
+//    16-byte-per-lane activation read per matrix instruction), the matrix cores about half of it;
+//  * the K loop is pipelined by hand: the bytes of step j + 2 and the activation fragments of the next half step are
+//    read from LDS and the weights of step j + 1 decoded while the matrix cores work on step j; scheduling barriers
+//    keep the compiler from moving the reads back next to their use; the requests to memory are dealt over the steps
+//    (the load unit takes one every sixteen cycles or so: a wave that issues them in one go waits there).
+// The loads that write LDS are hidden from the compiler (lds_dma16): the waits for them are explicit (wait_vm).
+template <class F, int WV, int RT, int TM, int XK>
+__global__ __launch_bounds__(64 * WV) void mm_tile_kernel(const void* X_, const uint8_t* W_, float* Y_, uint32_t n_, uint32_t rows_,
+                                                          uint32_t cols_, uint32_t x_stride_, uint32_t row_bytes_, uint32_t accumulate_,
+                                                          uint32_t slice_stages_, float* partials_) {
+  const MmArgs a{X_, W_, Y_, n_, rows_, cols_, x_stride_, row_bytes_, accumulate_, slice_stages_, partials_};
+  constexpr int NT = 64 * WV, TOK = 16 * TM, ROWS = 16 * WV * RT;
+  constexpr int CPT = XK / 8;                 // 16-byte chunks per token and stage
+  constexpr int XBUF = TOK * XK * 2;
+  constexpr int NS = XK / 32;                 // K steps per stage
+  constexpr int XPW = 256 / XK;               // stages per weight stage
+  constexpr int TH = TM < 8 ? TM : 8, UPS = TM / TH;  // token tiles per unit of the pipeline, units per K step
+  static_assert((XK == 64 || XK == 128) && TM % TH == 0, "");
+  // 16-byte pieces per row and weight stage: the stage's bytes at any 2-byte alignment inside their first piece; an odd
+  // count, so that the sixteen rows of a tile start in sixteen different groups of four banks
+  constexpr int P = ((F::WS_BYTES + 14 + 15) / 16) | 1;
+  constexpr int NPI = (ROWS * P + NT - 1) / NT;  // weight pieces per thread and weight stage
+  constexpr int WBUF = NPI * NT * 16;
+  constexpr int XPI = TOK * CPT / NT;            // activation pieces per thread and stage
+  static_assert(TOK * CPT % NT == 0, "every thread requests the same number of pieces");
+  constexpr bool PAIR = requires { F::pos_of(0u); };
+  extern __shared__ __attribute__((aligned(16))) uint32_t smem[];
+  uint32_t* tbl = smem;
+  uint8_t* abuf = (uint8_t*)(smem + F::LDS_WORDS);
+  uint8_t* wbuf = abuf + 2 * XBUF;
+  const uint32_t tid = threadIdx.x, lane = tid & 63u;
+  const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
+  const uint32_t n16 = lane & 15u, q = lane >> 4;
+  const uint32_t row0 = blockIdx.x * ROWS, m0 = blockIdx.y * TOK;
+  const uint32_t nstages = a.cols / XK;
+  const uint32_t st0 = blockIdx.z * a.slice_stages, st1 = min(st0 + a.slice_stages, nstages);  // st0: a whole number of weight stages
+  // slot of chunk c in the row of token t: the LDS has 32 banks of four bytes, rows are one or two times 128 bytes
+  // apart, so all rows start in the same bank; eight consecutive lanes (tokens) of a 16-byte read are served together and
+  // have to hit eight different 16-byte groups: the token's low three bits go into the slot
+  auto swz = [](uint32_t t) { return CPT == 16 ? (t & 15u) : (t & 7u); };
+
+  // ---- activations: piece i = k NT + tid is slot i % CPT of token i / CPT (host: rows 16-byte aligned, below 4 GiB)
+  const rsrc_t xrs = make_rsrc(a.X, ((a.n - 1) * a.x_stride + a.cols) * 2u);
+  uint32_t xoff[XPI];
+#pragma unroll
+  for (int k = 0; k < XPI; k++) {
+    const uint32_t i = (uint32_t)k * NT + tid, t = i / CPT;
+    xoff[k] = min(m0 + t, a.n - 1) * a.x_stride * 2u + 16u * ((i % CPT) ^ swz(t));  // tokens past n repeat the last one
+  }
+  auto x_request = [&](uint32_t st, uint32_t buf, int k0, int k1) {
+#pragma unroll
+    for (int k = k0; k < k1; k++)
+      lds_dma16(xrs, abuf + buf * XBUF + ((uint32_t)k * NT + wave * 64u) * 16u, xoff[k], st * (XK * 2u));
+  };
+  // ---- weights: piece i = k NT + tid is 16-byte piece i % P of row i / P
+  const uintptr_t wa = (uintptr_t)a.W;
+  const uint32_t wmis = (uint32_t)wa & 15u;
+  const uint32_t wbytes = (wmis + a.rows * a.row_bytes + 15u) & ~15u;  // (below 4 GiB: the host sends larger matrices elsewhere)
+  const rsrc_t wrs = make_rsrc((const void*)(wa - wmis), wbytes);      // whole aligned pieces: no piece straddles the end
+  uint32_t woff[NPI], wpc[NPI];
+#pragma unroll
+  for (int k = 0; k < NPI; k++) {
+    const uint32_t i = (uint32_t)k * NT + tid, rl = i / P, r = row0 + rl;
+    woff[k] = rl < (uint32_t)ROWS && r < a.rows ? wmis + r * a.row_bytes : ~0u;  // rows past the end: zeros, no traffic
+    wpc[k] = (i % P) * 16u;
+  }
+  auto w_request = [&](uint32_t ws, uint32_t buf) {  // (past a row's last block this fetches bytes nobody reads)
+#pragma unroll
+    for (int k = 0; k < NPI; k++) {
+      const uint32_t v = woff[k] + ws * (uint32_t)F::WS_BYTES;
+      lds_dma16(wrs, wbuf + buf * WBUF + ((uint32_t)k * NT + wave * 64u) * 16u, woff[k] == ~0u ? wbytes : (v & ~15u) + wpc[k], 0u);
+    }
+  };
+  uint32_t myoff[RT];
+  const uint8_t* lbase[RT];
+#pragma unroll
+  for (int rt = 0; rt < RT; rt++) {
+    const uint32_t rl = (wave * RT + rt) * 16u + n16;
+    myoff[rt] = wmis + min(row0 + rl, a.rows - 1) * a.row_bytes;
+    lbase[rt] = wbuf + rl * (uint32_t)(P * 16);
+  }
+
+  x_request(st0, 0, 0, XPI);
+  w_request(st0 / XPW, 0);
+  F::fill_lds(tbl, (int)tid, NT);
+  wait_vm<0>();
+  __syncthreads();
+
+  f4_t acc[RT][TM];
+#pragma unroll
+  for (int rt = 0; rt < RT; rt++)
+#pragma unroll
+    for (int t = 0; t < TM; t++) acc[rt][t] = f4_t{0.f, 0.f, 0.f, 0.f};
+
+  for (uint32_t st = st0; st < st1; st++) {
+    const uint32_t rel = st - st0, buf = rel & 1u, ws = st / XPW, sub = st % XPW, wb = (rel / XPW) & 1u;
+    // the targets of this stage's requests were last read before the barrier that ended the previous stage (the
+    // weight buffer before the one that ended the previous weight stage)
+    const uint32_t stn = st + 1 < st1 ? st + 1 : st;  // (the last stage fetches itself again: the waits stay the same)
+    const uint8_t* arow = abuf + buf * XBUF + n16 * (XK * 2u);
+    LdsRow lrow[RT];
+#pragma unroll
+    for (int rt = 0; rt < RT; rt++) lrow[rt] = LdsRow::of(lbase[rt] + wb * WBUF, (myoff[rt] + ws * (uint32_t)F::WS_BYTES) & 15u);
+    const uint32_t sl0 = sub * NS;  // first K step of this stage inside the weight stage
+    decltype(F::load_raw(lrow[0], 0u, 0u)) raw[2][RT];
+    uint4 bx[2][TH];
+    uint32_t h[2][RT][4];
+    auto fetch_w = [&](int slot, int js) {
+#pragma unroll
+      for (int rt = 0; rt < RT; rt++) raw[slot][rt] = F::load_raw(lrow[rt], sl0 + js, q);
+    };
+    auto fetch_x = [&](int slot, int js, int u) {
+#pragma unroll
+      for (int t = 0; t < TH; t++) {
+        const uint8_t* tr = arow + (u * TH + t) * 16 * (XK * 2);
+        if constexpr (PAIR) {
+          // positions (2 i, 2 i + 1) of chunk q stand for columns (4 q + i, 16 + 4 q + i) of the step: two 8-byte reads,
+          // interleaved when they are used
+          const uint32_t c1 = 4u * js + (q >> 1), at = 8u * (q & 1u);
+          const uint2 lo = *(const uint2*)(tr + 16u * (c1 ^ swz(n16)) + at), hi = *(const uint2*)(tr + 16u * ((c1 + 2u) ^ swz(n16)) + at);
+          bx[slot][t] = uint4{lo.x, lo.y, hi.x, hi.y};
+        } else {
+          bx[slot][t] = *(const uint4*)(tr + 16u * ((4u * js + q) ^ swz(n16)));
+        }
+      }
+    };
+    auto decode = [&](int hs, int slot, int js) {
+#pragma unroll
+      for (int rt = 0; rt < RT; rt++) {
+        const FragOut f = F::finish(raw[slot][rt], sl0 + js, q, tbl);
+#pragma unroll
+        for (int p = 0; p < 4; p++) h[hs][rt][p] = scale_round_h2(f.h[p], f.scale, F::HAS_ADD ? f.add : 0.f);
+      }
+    };
+    fetch_w(0, 0);
+    fetch_x(0, 0, 0);
+    if (NS > 1) fetch_w(1, 1);
+    __builtin_amdgcn_sched_barrier(0);
+    decode(0, 0, 0);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int g = 0; g < NS * UPS; g++) {  // unit g: token tiles u TH .. of K step js
+      const int js = g / UPS, u = g % UPS;
+      if (u == 0 && js + 2 < NS) fetch_w(js & 1, js + 2);
+      if (g + 1 < NS * UPS) fetch_x((g + 1) & 1, (g + 1) / UPS, (g + 1) % UPS);
+      if (u == 0) {
+        constexpr int XA = NS > 1 ? (XPI + NS - 2) / (NS - 1) : XPI;  // activations over the first steps, weights with the last
+        if (js < NS - 1 || NS == 1) x_request(stn, buf ^ 1u, js * XA, (js + 1) * XA < XPI ? (js + 1) * XA : XPI);
+        if (js == NS - 1 && sub == 0) w_request(ws + 1, wb ^ 1u);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      if (u == 0 && js + 1 < NS) decode((js + 1) & 1, (js + 1) & 1, js + 1);
+#pragma unroll
+      for (int t = 0; t < TH; t++) {
+        const uint4 av = bx[g & 1][t];
+        uint32_t x[4] = {av.x, av.y, av.z, av.w};
+        if constexpr (PAIR) {
+          x[0] = __builtin_amdgcn_perm(av.z, av.x, 0x05040100u); x[1] = __builtin_amdgcn_perm(av.z, av.x, 0x07060302u);
+          x[2] = __builtin_amdgcn_perm(av.w, av.y, 0x05040100u); x[3] = __builtin_amdgcn_perm(av.w, av.y, 0x07060302u);
+        }
+#pragma unroll
+        for (int rt = 0; rt < RT; rt++) acc[rt][u * TH + t] = mfma_f16(x, h[js & 1][rt], acc[rt][u * TH + t]);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    // the next stage's activations have to be there; the weight stage requested behind them in the first stage of a
+    // weight stage may stay in flight over the next stage
+    if (sub == 0) wait_vm<NPI>();
+    else wait_vm<0>();
+    __syncthreads();
+  }
+  wait_vm<0>();  // a weight stage may still be on its way into this workgroup's LDS: not past the end of the kernel
+
+  // D: lane holds weight row n16 of its tile (column of D), tokens 4 q + i of every token tile
+#pragma unroll
+  for (int rt = 0; rt < RT; rt++) {
+    const uint32_t row = row0 + (wave * RT + rt) * 16u + n16;
+    if (row >= a.rows) continue;
+    float* out = a.partials ? a.partials + (size_t)blockIdx.z * a.n * a.rows : a.Y;
+    const bool add = !a.partials && a.accumulate;
+#pragma unroll
+    for (int t = 0; t < TM; t++) {
+      float old[4];
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+        const uint32_t tok = m0 + 16u * t + 4u * q + i;
+        old[i] = add && tok < a.n ? out[(size_t)tok * a.rows + row] : 0.f;
+      }
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+        const uint32_t tok = m0 + 16u * t + 4u * q + i;
+        if (tok < a.n) out[(size_t)tok * a.rows + row] = old[i] + acc[rt][t][i];
+      }
+    }
+  }
+}
+
 // Y (+)= partials[0] + partials[1] + ... in that order, element by element
 __global__ __launch_bounds__(256) void mm_reduce_kernel(const float* __restrict__ partials, float* __restrict__ Y, size_t count,
                                                         uint32_t slices, uint32_t accumulate) {

@@ -19,7 +19,7 @@ NO_SCRATCH = [
     "15moe_down_kernelINS_7DecIQ1SENS_9DecIQ2XXSELi768",
     "13moe_gu_kernelINS_10DecIQ2XXSQES1_",                            # IQ2_XXS routed + IQ2_XXS shared
     "19moe_pf_block_kernel",                                        # prefill grouped GEMM, BASELINE configs[3]
-    "15mm_fused_kernel", "16mm_reduce_kernel",                      # fused prefill matmul
+    "15mm_fused_kernel", "14mm_tile_kernel", "16mm_reduce_kernel",  # fused prefill matmul
     "19router_fused_kernel",
 ]
 

@@ -27,6 +27,13 @@ CASES = [  # (type, rows, cols, n, accumulate): tests/test_quant_matmul.mm:18-25
     (O.Q5_K, 272, 1024, 257, True), (O.Q6_K, 384, 1024, 512, False), (O.IQ4_NL, 96, 512, 700, False),
     # the fused kernel with one K slice per tile (two stages of K: nothing to cut) and with many (the cases above)
     (O.Q8_0, 16384, 256, 100, True),
+    (O.IQ4_NL, 200, 640, 90, False), (O.Q8_0, 130, 384, 70, True), (O.IQ2_XXS, 144, 1024, 100, False),
+    (O.Q5_K, 130, 2304, 66, True), (O.Q6_K, 1536, 7168, 128, False),
+    # the tile kernel (IQ1_S, IQ2_XXS, IQ4_NL, Q8_0 matrices of 12 M weights and more, 65 to 256 tokens; 128-token tiles
+    # below 192 tokens, 256-token tiles from there): ragged row and token counts, an odd number of 128-column stages
+    # (half a weight stage at the end of a row), accumulate, both sides of its upper token bound
+    (O.IQ2_XXS, 4096, 4096, 100, False), (O.Q8_0, 3200, 3968, 70, True), (O.IQ4_NL, 4104, 3072, 129, False),
+    (O.IQ1_S, 2048, 6144, 256, True), (O.IQ4_NL, 3104, 4224, 200, True), (O.IQ2_XXS, 3000, 4096, 257, False),
 ]
 
 
@@ -79,6 +86,55 @@ def test_f32_to_f16_and_strided_matmul_h(dev):
     got = Y.cpu().numpy()
     assert (got[n * rows:] == 3.0).all()
     assert float(np.max(np.abs(got[: n * rows].reshape(n, rows) - sh) / (mag + 1e-12))) <= 1e-5
+
+
+@pytest.mark.parametrize("xs", [3976, 3970])
+def test_tile_matmul_h_strided(dev, xs):
+    """fp16 activations with a row stride, a large Q8_0 matrix at 96 tokens: rows on 16-byte boundaries go to the tile
+    kernel as they are, any other stride to the kernel that fetches lane by lane; both give the half-exact product."""
+    t, rows, cols, n = O.Q8_0, 3200, 3968, 96
+    Wb = O.random_blocks(t, rows * cols, 5)
+    X = O.randn(n * xs, 6)
+    X16 = up(X.astype(np.float16))
+    Y = torch.full((n * rows + 4,), 3.0, dtype=torch.float32, device=dev)
+    e = q.Enc()
+    q.encode_matmul_h(e, t, q.Buffer.of(up(Wb)), rows, cols, q.Buffer.of(X16), q.Buffer.of(Y), n, False, xs)
+    e.wait()
+    Xs = X.reshape(n, xs)[:, :cols].copy()
+    sh, _, mag, _ = reference(t, Wb, rows, cols, Xs, n)
+    got = Y.cpu().numpy()
+    assert (got[n * rows:] == 3.0).all()
+    assert float(np.max(np.abs(got[: n * rows].reshape(n, rows) - sh) / (mag + 1e-12))) <= 1e-5
+
+
+def test_tile_matmul_in_a_captured_graph(dev):
+    """The tile route allocates nothing either (the fp16 copy of the activations and the partial sums live in
+    file-scope device arrays): captured, every replay repeats the eager result bit for bit."""
+    t, rows, cols, n = O.IQ2_XXS, 3072, 4096, 130
+    Wb = O.random_blocks(t, rows * cols, 31)
+    X = O.randn(n * cols, 32)
+    sh, _, mag, _ = reference(t, Wb, rows, cols, X, n)
+    Wd, Xd = up(Wb), up(X)
+    Yd = torch.zeros(n * rows, dtype=torch.float32, device=dev)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        q.encode_matmul(q.Enc(side), t, q.Buffer.of(Wd), rows, cols, q.Buffer.of(Xd), q.Buffer.of(Yd), n)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    eager = Yd.clone()
+    got = eager.cpu().numpy().astype(np.float64).reshape(n, rows)
+    assert float(np.max(np.abs(got - sh) / (mag + 1e-12))) <= 1e-5
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        q.encode_matmul(q.Enc(torch.cuda.current_stream()), t, q.Buffer.of(Wd), rows, cols, q.Buffer.of(Xd), q.Buffer.of(Yd), n)
+    for rep in range(3):
+        Yd.fill_(7.0)
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(Yd, eager), f"replay {rep} differs from the eager result"
+        _ = (Xd * 2).sum().item()
 
 
 def test_fused_matmul_in_a_captured_graph(dev):
