@@ -577,6 +577,51 @@ def bench_issue_probe(torch, args):
             "roofline": None, "cpu_baseline": None, "pct_of_hbm_peak": None}
 
 
+def bench_lds_bank_probe(torch, args):
+    """Which lanes of a wave the LDS serves in the same pass (libmsq_probe.so: lds_bank_probe_kernel). Lane l reads at
+    256 l + 16 slot(l): two lanes collide exactly when their slots are equal, so a slot pattern that runs at the rate of
+    distinct slots names lanes that never share a pass. The last rows check the resulting model for 16-byte reads --
+    groups {0-7, 24-31}, {8-15, 16-23}, {32-39, 56-63}, {40-47, 48-55} -- against the activation layouts of the prefill
+    kernels before and after they were changed to it."""
+    from macseek_amd import build as B
+    if not os.path.exists(B.PROBE_OUT):
+        raise RuntimeError("bench.py: %s is missing; build it with `python -m macseek_amd.build`" % B.PROBE_OUT)
+    P = C.CDLL(B.PROBE_OUT)
+    P.msq_probe_lds_bank.restype = C.c_int
+    P.msq_probe_lds_bank.argtypes = [C.c_void_p, C.c_int, C.c_void_p, C.c_void_p, C.c_int]
+    dev = torch.device("cuda:0")
+    out = torch.zeros(2, dtype=torch.int64, device=dev)
+    lane = lambda f: [256 * l + 16 * f(l) for l in range(64)]
+    frag = lambda f: [f(l & 15, l >> 4) for l in range(64)]  # lane = 16 chunk + token, as the matrix fragments are read
+    pats = [("distinct slots in every 16 lanes (l % 16)", lane(lambda l: l % 16)),
+            ("all lanes one slot", lane(lambda l: 0)),
+            ("aligned quads share (l / 4)", lane(lambda l: l // 4)),
+            ("l, l+8 share and l, l+32 share (l % 8 + 8 (l / 16 % 2))", lane(lambda l: l % 8 + 8 * (l // 16 % 2))),
+            ("l, l+8, l+16, l+24 share (l % 8 + 8 (l / 32 % 2))", lane(lambda l: l % 8 + 8 * (l // 32 % 2))),
+            ("l, l+4, l+8, l+12 share (l % 4 + 4 (l / 16))", lane(lambda l: l % 4 + 4 * (l // 16))),
+            ("neighbours share (l % 32 / 2)", lane(lambda l: l % 32 // 2)),
+            ("fragment rows 528 B apart, chunks 128 B apart (prefill GEMM, old)", frag(lambda n, q: n * 528 + 128 * q)),
+            ("fragment rows 528 B apart, chunks at 0, 256, 128, 384 (prefill GEMM, now)", frag(lambda n, q: n * 528 + 256 * (q & 1) + 128 * (q >> 1))),
+            ("fragment rows 272 B apart, chunks 16 B apart (fused matmul)", frag(lambda n, q: n * 272 + 16 * q)),
+            ("fragment rows 256 B apart, slot = chunk ^ token (tile matmul)", frag(lambda n, q: n * 256 + 16 * (q ^ n)))]
+    iters, rows = 400, []
+    for width in (16, 8, 4):
+        for name, addr in pats:
+            a = torch.tensor(addr, dtype=torch.int32, device=dev)
+            for _ in range(2):
+                rc = P.msq_probe_lds_bank(C.c_void_p(torch.cuda.current_stream().cuda_stream), width, C.c_void_p(a.data_ptr()),
+                                          C.c_void_p(out.data_ptr()), iters)
+                if rc != 0:
+                    raise RuntimeError("msq_probe_lds_bank failed: %d" % rc)
+                torch.cuda.synchronize()
+            rows.append({"bytes_per_lane": width, "pattern": name, "cycles_per_wave_read": round(float(out[0].item()) / (iters * 16 * 8), 2)})
+    for r in rows:
+        sys.stderr.write("%2d B  %-78s %6.2f\n" % (r["bytes_per_lane"], r["pattern"], r["cycles_per_wave_read"]))
+    return {"value": 0.0, "ms_per_step": 0.0, "dtype": "LDS reads",
+            "config": {"workload": "LDS bank probe: cycles per wave-wide read with the LDS saturated by eight waves, by lane -> address pattern", "rows": rows},
+            "roofline": None, "cpu_baseline": None, "pct_of_hbm_peak": None}
+
+
 def bench_handover_probe(torch, args):
     """What a device-wide hand-over inside one launch costs (libmsq_probe.so: handover_probe_kernel), the step a
     single-launch MoE layer needs between gate/up and down: per workgroup, microseconds from its start until its h
@@ -896,7 +941,7 @@ def main():
     ap.add_argument("--steps", type=int, default=500)
     ap.add_argument("--warmup", type=int, default=100)
     ap.add_argument("--workload", default="moe_decode",
-                    choices=["moe_decode", "moe_prefill", "matvec_iq1s", "matvec_iq2xxs", "q8_0", "matvec_n", "router", "matmul", "stream", "copy_calibration", "issue_probe", "handover_probe", "table"])
+                    choices=["moe_decode", "moe_prefill", "matvec_iq1s", "matvec_iq2xxs", "q8_0", "matvec_n", "router", "matmul", "stream", "copy_calibration", "issue_probe", "handover_probe", "lds_bank_probe", "table"])
     ap.add_argument("--one-stream", action="store_true",
                     help="profiling runs: msq_moe_prefill keeps its launches on one stream (MSQ_MOEP_ONE_STREAM=1), so that "
                          "per-kernel durations and counters are not those of two kernels sharing the device")
@@ -945,6 +990,8 @@ def main():
         r = bench_issue_probe(torch, args)
     elif args.workload == "handover_probe":
         r = bench_handover_probe(torch, args)
+    elif args.workload == "lds_bank_probe":
+        r = bench_lds_bank_probe(torch, args)
     elif args.workload == "router":
         r = bench_router(torch, args)
     elif args.workload == "table":

@@ -10,7 +10,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OUT = os.path.join(HERE, "libmsq.so")
 # the benchmark's instruction-issue probe: a shared object of its own, no part of the library
-PROBE_SRC = [os.path.join(CSRC, "probe", "issue_probe.hip"), os.path.join(CSRC, "probe", "handover_probe.hip")]
+PROBE_SRC = [os.path.join(CSRC, "probe", f) for f in ("issue_probe.hip", "handover_probe.hip", "lds_bank_probe.hip")]
 PROBE_OUT = os.path.join(HERE, "libmsq_probe.so")
 OBJDIR = os.path.join(HERE, "csrc", "build")
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")

@@ -209,6 +209,14 @@ constexpr int pf_blk_rows(bool gu, int T) { return pf_blk_waves(T) * pf_blk_rt(g
 template <class B>
 constexpr size_t pf_blk_lds(int T) { return (size_t)B::LDS_WORDS * 4 + (T > 3 ? 1 : 2) * (size_t)(T > 3 ? kPfBigTokens : kPfBlkTokens) * kPfBlkPitch; }
 
+// Where the 16 bytes of step j of chunk q (columns blk_col_of(q, j) .. + 7 of a block) sit in a token's staged row: the
+// chunks in the order 0, 2, 1, 3. A 16-byte LDS read serves the lanes in four groups of sixteen -- {0-7, 24-31},
+// {8-15, 16-23}, {32-39, 56-63}, {40-47, 48-55}, measured -- so a group holds tokens 0-7 of one chunk and tokens 8-15 of
+// its neighbour (lane = 16 q + token); rows are 33 sixteen-byte units apart, token n starts in bank group n mod 16, and the
+// two halves of a group only miss each other when the neighbouring chunks are a multiple of 256 bytes apart (in column
+// order they are 128 apart and every read took two passes).
+__device__ __forceinline__ uint32_t pf_lds_at(uint32_t q, uint32_t j) { return 16u * (16u * (q & 1u) + 8u * (q >> 1) + j); }
+
 template <class B, bool GU, int T>
 __device__ __forceinline__ void pf_block_body(const PfBlkArgs& a) {
   constexpr int WAVES = pf_blk_waves(T), NT = 64 * WAVES;
@@ -261,7 +269,7 @@ __device__ __forceinline__ void pf_block_body(const PfBlkArgs& a) {
 #pragma unroll
     for (int i = 0; i < AG; i++) {
       const uint32_t g = tid + i * NT;
-      if (g < T * 512u) *(u32x4*)(abuf + buf * ABUF + (g >> 5) * PITCH + (g & 31u) * 16u) = pa[i];
+      if (g < T * 512u) *(u32x4*)(abuf + buf * ABUF + (g >> 5) * PITCH + pf_lds_at((g >> 3) & 3u, g & 7u)) = pa[i];
     }
   };
 
@@ -305,7 +313,7 @@ __device__ __forceinline__ void pf_block_body(const PfBlkArgs& a) {
         for (int r = 0; r < R; r++) lk[r] = B::lookup(cur[r], j, tbl, n16);
 #pragma unroll
         for (int u = 0; u < 2; u++) {
-          const uint4 av = *(const uint4*)(arow + u * 16 * PITCH + 2u * blk_col_of(q, j));
+          const uint4 av = *(const uint4*)(arow + u * 16 * PITCH + pf_lds_at(q, j));
           af[u][0] = av.x; af[u][1] = av.y; af[u][2] = av.z; af[u][3] = av.w;
         }
         uint32_t h[R][4];
@@ -315,7 +323,7 @@ __device__ __forceinline__ void pf_block_body(const PfBlkArgs& a) {
         for (int t = 0; t < T; t++) {
           const uint32_t(&x)[4] = af[t % 3];
           if (t + 2 < T) {
-            const uint4 av = *(const uint4*)(arow + (t + 2) * 16 * PITCH + 2u * blk_col_of(q, j));
+            const uint4 av = *(const uint4*)(arow + (t + 2) * 16 * PITCH + pf_lds_at(q, j));
             uint32_t(&y)[4] = af[(t + 2) % 3];
             y[0] = av.x; y[1] = av.y; y[2] = av.z; y[3] = av.w;
           }
@@ -354,7 +362,7 @@ __device__ __forceinline__ void pf_block_body(const PfBlkArgs& a) {
       if (p % PPS == 0) {  // activations of step j, read with the fragments' column mapping
 #pragma unroll
         for (int t = 0; t < T; t++) {
-          const uint4 av = *(const uint4*)(arow + t * 16 * PITCH + 2u * blk_col_of(q, j));
+          const uint4 av = *(const uint4*)(arow + t * 16 * PITCH + pf_lds_at(q, j));
           af[t][0] = av.x; af[t][1] = av.y; af[t][2] = av.z; af[t][3] = av.w;
         }
       }
