@@ -56,7 +56,7 @@ __global__ __launch_bounds__(1024) void bw_probe_kernel(const uint4* __restrict_
 namespace {
 
 // Launch shape of the decode matvec. units = cols / UNIT columns-slices per row; a wave covers 64 * iters of them.
-struct MvShape { int iters, ks, rw, rpw, unit; int per_cu = 1; bool stage_w = false; };  // per_cu: persistent workgroups per CU, stage_w: weight rows through LDS (mv_tok_kernel)
+struct MvShape { int iters, ks, rw, rpw, unit; int per_cu = 1; bool stage_w = false, free_shape = false; };  // per_cu: persistent workgroups per CU, stage_w: weight rows through LDS (mv_tok_kernel), free_shape: no part of the shape was imposed by the caller
 
 int mv_unit(int t) { return msq_type_block_elems(t) == 1 ? 8 : 32; }
 
@@ -203,7 +203,7 @@ bool mv_tok_shape(int t, int rows, int cols, int groups, int n, int token_groups
   static const int env_sw = env_knob_early("MSQ_MV_STAGEW", -1);
   const bool stage_w = n == 1 && free_shape &&
                        (env_sw >= 0 ? env_sw > 0 : (t == MSQ_Q6_K && bytes >= 12e6) || (t == MSQ_Q8_0 && bytes >= 40e6));
-  *s = {iters, ks, rw, rpw, unit, per_cu, stage_w};
+  *s = {iters, ks, rw, rpw, unit, per_cu, stage_w, free_shape};
   return true;
 }
 
@@ -219,11 +219,35 @@ bool tok_serves_single(int t, int rows, int cols, const MvShape& s, const MsqMvC
 }
 
 template <class D, int T>
-int launch_mv_tok(hipStream_t st, const MvShape& s, MvTokArgs& ta) {
+int launch_mv_tok(hipStream_t st, const MvShape& s_, const MvTokArgs& ta_) {
+  MvTokArgs ta = ta_;  // (the launch may reshape rows into pairs: the caller's arguments stay as they are)
   MvArgs& a = ta.m;
+  MvShape s = s_;
+  // One token, rows whose units fill a whole number of waves and at most half of another (5120 or 7168 columns of a
+  // block format: 2.5 and 3.5 waves): two rows are launched as one of twice the units, which leaves no lane idle
+  // (mv_tok_kernel, PAIR). One group, an even number of rows, a row's units a multiple of 16. Measured, rows one by
+  // one / in pairs: Q6_K 129280x5120 113.2 / 99.8 us, 1536x7168 6.41 / 6.10, 2304x5120 6.61 / 6.29, Q8_0 2304x5120
+  // 6.67 / 6.52; the codebook formats, bound by their lookups, lose 1 % and keep the one-row form. MSQ_MV_PAIR = 0 / 2:
+  // never / every format.
+  bool pair = false;
+  if constexpr (T == 1) {
+    static const int env_pair = env_knob_early("MSQ_MV_PAIR", -1);
+    const int u = (int)(a.cols / D::UNIT), k1 = (u + 63) / 64, k2 = (2 * u + 63) / 64;
+    pair = s.iters == 1 && s.free_shape && (D::LDS_WORDS == 0 || env_pair == 2) && !a.norm_w && env_pair != 0 && a.rows % 2 == 0 && a.rows_per_group >= a.rows && u % 16 == 0 &&
+           k2 < 2 * k1 && k2 <= 8;
+    if (pair) {
+      a.rows /= 2;
+      a.rows_per_group = a.rows;
+      a.row_bytes *= 2;
+      s.ks = k2;
+      s.rw = std::max(1, 8 / k2);
+      const long wgs = std::max(1, s.per_cu * device_info().cus);
+      s.rpw = (int)std::min<long>(32, std::max<long>(1, (a.rows + wgs * s.rw - 1) / (wgs * s.rw)));
+    }
+  }
   const int threads = 64 * s.rw * s.ks;
   const int tile_rows = s.rw * s.rpw;
-  a.units = a.cols / D::UNIT;
+  a.units = (pair ? 2 : 1) * (a.cols / D::UNIT);
   a.ks = s.ks;
   a.rpw = s.rpw;
   a.ntiles = (a.rows + tile_rows - 1) / tile_rows;
@@ -259,9 +283,15 @@ int launch_mv_tok(hipStream_t st, const MvShape& s, MvTokArgs& ta) {
   const int gx = (int)std::min<long>(a.ntiles, std::max(1, per_cu * device_info().cus / gy));
   const dim3 grid((unsigned)gx, (unsigned)gy);
   if (sw) {
-    if constexpr (tok_stages_w<D, 1, T>()) launch(mv_tok_kernel<D, 1, T, false, true>, grid);
-  } else if (s.iters == 1) launch(mv_tok_kernel<D, 1, T>, grid);
-  else if constexpr (D::UNIT == 8) launch(mv_tok_kernel<D, 2, T>, grid);
+    if constexpr (tok_stages_w<D, 1, T>()) {
+      if (pair) launch(mv_tok_kernel<D, 1, T, false, true, true>, grid);
+      else launch(mv_tok_kernel<D, 1, T, false, true>, grid);
+    }
+  } else if (s.iters == 1) {
+    if (pair) {
+      if constexpr (T == 1) launch(mv_tok_kernel<D, 1, T, false, false, true>, grid);
+    } else launch(mv_tok_kernel<D, 1, T>, grid);
+  } else if constexpr (D::UNIT == 8) launch(mv_tok_kernel<D, 2, T>, grid);
   else return MSQ_ERR_UNSUPPORTED;  // two block-format units per lane and T activation slices do not fit the registers
   MSQ_HIP(hipGetLastError());
   return MSQ_OK;

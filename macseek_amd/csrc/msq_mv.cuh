@@ -378,7 +378,12 @@ __device__ __forceinline__ void wait_rows_n(int n) {
 
 // Decoders with STAGE_X take the activations through LDS (contiguous loads, tok_round() tokens per round); with the
 // others every lane reads its slices from device memory, all T tokens' loads in flight at once.
-template <class D, int ITERS, int T, bool NORM = false, bool SW = false>
+// PAIR (with SW): the launch treats two consecutive rows as one row of twice the units -- rows are contiguous in memory,
+// so a wave's slice of 64 units may run from the end of one row into the next -- which leaves no lane idle when a row's
+// units fill a whole number of waves and a half (5120 columns: five waves per row pair instead of twice three). rows_,
+// row_bytes_, units_, ks_ and the tile shape then describe the pairs; the two rows' 16-lane sums are told apart when
+// the partial sums are added (a row's units must be a multiple of 16 for that).
+template <class D, int ITERS, int T, bool NORM = false, bool SW = false, bool PAIR = false>
 __global__ __launch_bounds__(512) void mv_tok_kernel(const uint8_t* W_, uint32_t rows_, uint32_t row_bytes_, uint32_t units_, uint32_t ks_,
                                                      uint32_t rpw_, uint32_t ntiles_, uint32_t rows_per_group_, const float* x_,
                                                      uint32_t cols_, const MvTokArgs ta) {
@@ -427,6 +432,9 @@ __global__ __launch_bounds__(512) void mv_tok_kernel(const uint8_t* W_, uint32_t
     valid[i] = u < units_;
     unit[i] = valid[i] ? u : units_ - 1;  // idle lanes shadow the last unit; their result is dropped
   }
+  uint32_t xu[ITERS];  // the unit of the activations that goes with unit[i] (second row of a pair: the same columns again)
+#pragma unroll
+  for (int i = 0; i < ITERS; i++) xu[i] = PAIR && unit[i] >= (units_ >> 1) ? unit[i] - (units_ >> 1) : unit[i];
   typename D::X xr[T][ITERS];
   uint32_t cur_group = 0xFFFFFFFFu;
   float* xs = (float*)(smem + a.xs_off);
@@ -520,7 +528,7 @@ __global__ __launch_bounds__(512) void mv_tok_kernel(const uint8_t* W_, uint32_t
           }
           __syncthreads();
 #pragma unroll
-          for (int i = 0; i < ITERS; i++) xr[0][i] = D::load_x(XLds{xs}, unit[i]);
+          for (int i = 0; i < ITERS; i++) xr[0][i] = D::load_x(XLds{xs}, xu[i]);
           staged = true;
         }
       }
@@ -529,13 +537,13 @@ __global__ __launch_bounds__(512) void mv_tok_kernel(const uint8_t* W_, uint32_t
       for (int t = 0; t < T; t++) {
         if constexpr (NORM) {
 #pragma unroll
-          for (int i = 0; i < ITERS; i++) xr[t][i] = D::load_x(XLds{xs}, unit[i]);
+          for (int i = 0; i < ITERS; i++) xr[t][i] = D::load_x(XLds{xs}, xu[i]);
         } else if constexpr (!STAGE) {
 #pragma unroll
-          for (int i = 0; i < ITERS; i++) xr[t][i] = D::load_x(x_of(t), unit[i]);
+          for (int i = 0; i < ITERS; i++) xr[t][i] = D::load_x(x_of(t), xu[i]);
         } else if (!D::STAGE_X && !a.stage_x) {  // (rows too long for a round of G in LDS: read directly, as for few tokens)
 #pragma unroll
-          for (int i = 0; i < ITERS; i++) xr[t][i] = D::load_x(x_of(t), unit[i]);
+          for (int i = 0; i < ITERS; i++) xr[t][i] = D::load_x(x_of(t), xu[i]);
         } else {
           if (t % G == 0) {
             __syncthreads();  // readers of the previous round are done
@@ -546,7 +554,7 @@ __global__ __launch_bounds__(512) void mv_tok_kernel(const uint8_t* W_, uint32_t
             __syncthreads();
           }
 #pragma unroll
-          for (int i = 0; i < ITERS; i++) xr[t][i] = D::load_x(XLds{xs + (t % G) * roww}, unit[i]);
+          for (int i = 0; i < ITERS; i++) xr[t][i] = D::load_x(XLds{xs + (t % G) * roww}, xu[i]);
         }
       }
       }
@@ -610,6 +618,17 @@ __global__ __launch_bounds__(512) void mv_tok_kernel(const uint8_t* W_, uint32_t
     for (; j0 + NR < rpw_; j0 += NR) round.template operator()<true>(j0);
     round.template operator()<false>(j0);
     __syncthreads();
+    if constexpr (PAIR) {  // (one token) pair r / 2, its first or second units / 32 sixteen-lane sums
+      const uint32_t G = units_ >> 5;
+      for (uint32_t r = tid; r < 2u * tile_rows; r += blockDim.x) {
+        const uint32_t row = 2u * tile_row0 + r;
+        if (row < 2u * rows_) {
+          const float s = sum_in_order(part + (r >> 1) * 4 * KS + (r & 1u) * G, G, 1);
+          float* y = a.y + row;
+          *y = a.accumulate ? *y + s : s;
+        }
+      }
+    } else
     for (uint32_t idx = tid; idx < tile_rows * T; idx += blockDim.x) {
       const uint32_t r = idx % tile_rows, t = idx / tile_rows, row = tile_row0 + r;  // consecutive lanes: consecutive rows
       if (row < rows_ && t0 + t < ta.n) {

@@ -77,6 +77,10 @@ CASES = [
     # weight rows through LDS (large Q6_K / Q8_0 matrices): ragged row counts, a row that ends in a short wave slice
     (O.Q6_K, 4099, 4096, 1, False, "large q6_k, ragged rows"), (O.Q6_K, 3001, 5376, 1, True, "large q6_k, 21 blocks per row acc"),
     (O.Q8_0, 8201, 5120, 1, True, "large q8_0 acc"), (O.Q8_0, 16400, 2592, 1, False, "large q8_0, 81 blocks per row"),
+    # ... and with rows of two and a half / three and a half waves of units, which go two rows at a time when the row
+    # count is even (the last pair ragged against the tile; an odd count keeps the one-row form)
+    (O.Q6_K, 3002, 5120, 1, True, "large q6_k, row pairs acc"), (O.Q6_K, 2100, 7168, 1, False, "large q6_k, row pairs of 7 waves"),
+    (O.Q8_0, 7990, 5120, 1, False, "large q8_0, row pairs"), (O.Q6_K, 3003, 5120, 1, False, "large q6_k, odd rows"),
 ]
 
 
