@@ -230,7 +230,7 @@ int launch_mv_tok(hipStream_t st, const MvShape& s_, const MvTokArgs& ta_) {
   // 6.67 / 6.52; the codebook formats, bound by their lookups, lose 1 % and keep the one-row form. MSQ_MV_PAIR = 0 / 2:
   // never / every format.
   bool pair = false;
-  if constexpr (T == 1) {
+  {
     static const int env_pair = env_knob_early("MSQ_MV_PAIR", -1);
     const int u = (int)(a.cols / D::UNIT), k1 = (u + 63) / 64, k2 = (2 * u + 63) / 64;
     pair = s.iters == 1 && s.free_shape && (D::LDS_WORDS == 0 || env_pair == 2) && !a.norm_w && env_pair != 0 && a.rows % 2 == 0 && a.rows_per_group >= a.rows && u % 16 == 0 &&
@@ -241,7 +241,7 @@ int launch_mv_tok(hipStream_t st, const MvShape& s_, const MvTokArgs& ta_) {
       a.row_bytes *= 2;
       s.ks = k2;
       s.rw = std::max(1, 8 / k2);
-      const long wgs = std::max(1, s.per_cu * device_info().cus);
+      const long wgs = std::max<long>(1, s.per_cu * device_info().cus / (((long)ta.n + T - 1) / T));
       s.rpw = (int)std::min<long>(32, std::max<long>(1, (a.rows + wgs * s.rw - 1) / (wgs * s.rw)));
     }
   }
@@ -288,9 +288,8 @@ int launch_mv_tok(hipStream_t st, const MvShape& s_, const MvTokArgs& ta_) {
       else launch(mv_tok_kernel<D, 1, T, false, true>, grid);
     }
   } else if (s.iters == 1) {
-    if (pair) {
-      if constexpr (T == 1) launch(mv_tok_kernel<D, 1, T, false, false, true>, grid);
-    } else launch(mv_tok_kernel<D, 1, T>, grid);
+    if (pair) launch(mv_tok_kernel<D, 1, T, false, false, true>, grid);
+    else launch(mv_tok_kernel<D, 1, T>, grid);
   } else if constexpr (D::UNIT == 8) launch(mv_tok_kernel<D, 2, T>, grid);
   else return MSQ_ERR_UNSUPPORTED;  // two block-format units per lane and T activation slices do not fit the registers
   MSQ_HIP(hipGetLastError());

@@ -618,13 +618,13 @@ __global__ __launch_bounds__(512) void mv_tok_kernel(const uint8_t* W_, uint32_t
     for (; j0 + NR < rpw_; j0 += NR) round.template operator()<true>(j0);
     round.template operator()<false>(j0);
     __syncthreads();
-    if constexpr (PAIR) {  // (one token) pair r / 2, its first or second units / 32 sixteen-lane sums
+    if constexpr (PAIR) {  // pair r / 2, its first or second units / 32 sixteen-lane sums
       const uint32_t G = units_ >> 5;
-      for (uint32_t r = tid; r < 2u * tile_rows; r += blockDim.x) {
-        const uint32_t row = 2u * tile_row0 + r;
-        if (row < 2u * rows_) {
-          const float s = sum_in_order(part + (r >> 1) * 4 * KS + (r & 1u) * G, G, 1);
-          float* y = a.y + row;
+      for (uint32_t idx = tid; idx < 2u * tile_rows * T; idx += blockDim.x) {
+        const uint32_t r = idx % (2u * tile_rows), t = idx / (2u * tile_rows), row = 2u * tile_row0 + r;
+        if (row < 2u * rows_ && t0 + t < ta.n) {
+          const float s = sum_in_order(part + ((r >> 1) * 4 * KS + (r & 1u) * G) * T + t, G, T);
+          float* y = a.y + (size_t)(t0 + t) * ta.y_stride + row;
           *y = a.accumulate ? *y + s : s;
         }
       }
