@@ -196,6 +196,8 @@ struct PfBlkArgs {
   uint32_t nitems, total;
   uint32_t K, N, row_bytes, nblocks;
   uint32_t row_chunks;      // chunks of pf_blk_rows() weight rows
+  uint32_t chunks_per_wg;   // consecutive row chunks one workgroup takes, one after the other
+  uint32_t row_groups;      // workgroups per item: row_chunks / chunks_per_wg, rounded up
 };
 
 constexpr int kPfBlkTokens = 48, kPfBigTokens = 112, kPfBigTiles = kPfBigTokens / 16, kPfBlkPitch = 256 * 2 + 16;
@@ -236,21 +238,29 @@ __device__ __forceinline__ void pf_block_body(const PfBlkArgs& a) {
   // consecutive workgroups land on different XCDs: the row chunks of one item stay on one XCD (shared L2 for its
   // activations), and items are dealt round-robin over the XCDs
   const uint32_t xcd = blockIdx.x & 7u, slot = blockIdx.x >> 3;
-  const uint32_t item = (slot / a.row_chunks) * 8u + xcd, rc = slot % a.row_chunks;
+  const uint32_t item = (slot / a.row_groups) * 8u + xcd, rc0 = (slot % a.row_groups) * a.chunks_per_wg;
   if (item >= a.nitems) return;
   const uint32_t e = a.items[3 * item], t0 = a.items[3 * item + 1], cnt = a.items[3 * item + 2];
   const uint32_t base = a.offs[e] + t0;
+  // A workgroup takes chunks_per_wg consecutive row chunks of its item, one after the other: the first trip to memory
+  // (about 4.5 us before the first block can be multiplied, 17 % of a down-projection workgroup's life) is paid once, and
+  // the next chunk's first block is requested during the last block of the one before, where a single chunk would
+  // fetch its last block again
+  // (built into the down projection of the small items only: the other variants have no registers to spare for it)
+  constexpr bool MULTI = !GU && T <= 3;
+  const uint32_t nch = MULTI ? min(a.chunks_per_wg, a.row_chunks - rc0) : 1u;
 
-  gptr_t wrow[R];
-  uint32_t row_of[RT];
+  // a weight row = the expert's matrix (a scalar address) + the lane's row offset (32 bits: a matrix is far below 4 GiB)
+  gptr_t wbase[NM];
+  uint32_t woff[RT], row_of[RT];
+#pragma unroll
+  for (int m = 0; m < NM; m++) wbase[m] = as_global((const void*)a.ptrs[3 * e + (GU ? m : 2)]);
 #pragma unroll
   for (int jt = 0; jt < RT; jt++) {
-    row_of[jt] = ((rc * WAVES + wave) * RT + jt) * 16u + n16;
-    const uint32_t row = min(row_of[jt], a.N - 1);
-#pragma unroll
-    for (int m = 0; m < NM; m++)
-      wrow[jt * NM + m] = as_global((const void*)a.ptrs[3 * e + (GU ? m : 2)]) + (size_t)row * a.row_bytes;
+    row_of[jt] = ((rc0 * WAVES + wave) * RT + jt) * 16u + n16;
+    woff[jt] = min(row_of[jt], a.N - 1) * a.row_bytes;
   }
+  auto wrow = [&](int r, uint32_t off) { return wbase[r % NM] + (size_t)(woff[r / NM] + off); };
 
   // activation chunk loader: T * 512 granules of 16 bytes (token g / 32, column g % 32) over the workgroup's threads
   constexpr int AG = (T * 512 + NT - 1) / NT;
@@ -275,21 +285,30 @@ __device__ __forceinline__ void pf_block_body(const PfBlkArgs& a) {
 
   typename B::Raw cur[R], nxt[R];
 #pragma unroll
-  for (int r = 0; r < R; r++) cur[r] = B::load(wrow[r], q);
+  for (int r = 0; r < R; r++) cur[r] = B::load(wrow(r, 0u), q);
   a_issue(0);
   B::fill_lds(tbl, (int)tid, NT);
   a_store(0);
   __syncthreads();
 
+  uint32_t kb = 0;  // blocks done so far (double buffering: block kb sits in buffer kb % 2)
+  for (uint32_t c = 0; c < nch; c++) {
+  const bool more = c + 1 < nch;
   f4_t acc[T][R];
 #pragma unroll
   for (int t = 0; t < T; t++)
 #pragma unroll
     for (int r = 0; r < R; r++) acc[t][r] = f4_t{0.f, 0.f, 0.f, 0.f};
 
-  for (uint32_t kc = 0; kc < a.nblocks; kc++) {
-    const uint32_t kn = kc + 1 < a.nblocks ? kc + 1 : kc;  // the last block fetches itself again: no branch around the loads
-    const uint8_t* arow = abuf + (DB ? (kc & 1u) * ABUF : 0u) + n16 * PITCH;
+  for (uint32_t kc = 0; kc < a.nblocks; kc++, kb++) {
+    // the block requested during this one: the chunk's next, or the first of the workgroup's next chunk, or (nothing left)
+    // this one again: no branch around the loads
+    const bool lastb = kc + 1 == a.nblocks;
+    const uint32_t kn = !lastb ? kc + 1 : more ? 0u : kc;
+    // (the host lets a workgroup take several chunks only when all chunks are whole: the next chunk's rows are then the
+    // same number of bytes further for every lane)
+    const uint32_t wn = kn * (uint32_t)B::BLOCK_BYTES + (c + (lastb && more ? 1u : 0u)) * ((uint32_t)(WAVES * RT * 16) * a.row_bytes);
+    const uint8_t* arow = abuf + (DB ? (kb & 1u) * ABUF : 0u) + n16 * PITCH;
     if constexpr (T > 3) {
       // many token tiles: a step's fragments are all decoded first, then every tile's activation fragment (read from
       // LDS two tiles ahead of its use) feeds one matrix instruction per fragment
@@ -305,7 +324,7 @@ __device__ __forceinline__ void pf_block_body(const PfBlkArgs& a) {
         }
         if (j >= 2 && j - 2 < R) {
           __builtin_amdgcn_sched_barrier(0);
-          nxt[j - 2] = B::load(wrow[j - 2] + (size_t)kn * B::BLOCK_BYTES, q);
+          nxt[j - 2] = B::load(wrow(j - 2, wn), q);
           __builtin_amdgcn_sched_barrier(0);
         }
         typename B::Look lk[R];
@@ -356,7 +375,7 @@ __device__ __forceinline__ void pf_block_body(const PfBlkArgs& a) {
       }
       if (p % 2 == 0 && p >= 2 && p / 2 - 1 < R) {
         __builtin_amdgcn_sched_barrier(0);
-        nxt[p / 2 - 1] = B::load(wrow[p / 2 - 1] + (size_t)kn * B::BLOCK_BYTES, q);
+        nxt[p / 2 - 1] = B::load(wrow(p / 2 - 1, wn), q);
         __builtin_amdgcn_sched_barrier(0);
       }
       if (p % PPS == 0) {  // activations of step j, read with the fragments' column mapping
@@ -388,7 +407,7 @@ __device__ __forceinline__ void pf_block_body(const PfBlkArgs& a) {
     // the other activation buffer was last read one block ago, before the previous barrier: free to refill (with a
     // single buffer every wave has to be done with the block first)
     if (!DB) __syncthreads();
-    a_store(DB ? (kc & 1u) ^ 1u : 0u);
+    a_store(DB ? (kb & 1u) ^ 1u : 0u);
 #pragma unroll
     for (int r = 0; r < R; r++) cur[r] = nxt[r];
     __syncthreads();
@@ -423,6 +442,10 @@ __device__ __forceinline__ void pf_block_body(const PfBlkArgs& a) {
       }
     }
   }
+  // the next chunk: its first block is in `cur` and in LDS already
+#pragma unroll
+  for (int jt = 0; jt < RT; jt++) row_of[jt] += WAVES * RT * 16;
+  }
 }
 
 // Kernel variants: T = 3 takes the items of up to three token tiles in one launch, largest first (each runs the body
@@ -433,7 +456,7 @@ __global__ __launch_bounds__(64 * pf_blk_waves(T)) void moe_pf_block_kernel(cons
   if constexpr (T > 3) {
     pf_block_body<B, GU, T>(a);
   } else {
-    const uint32_t item = ((blockIdx.x >> 3) / a.row_chunks) * 8u + (blockIdx.x & 7u);
+    const uint32_t item = ((blockIdx.x >> 3) / a.row_groups) * 8u + (blockIdx.x & 7u);
     if (item >= a.nitems) return;
     const uint32_t cnt = a.items[3 * item + 2];
     if (cnt > 32) pf_block_body<B, GU, 3>(a);

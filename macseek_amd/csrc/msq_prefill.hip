@@ -68,7 +68,15 @@ int launch_block_tt(hipStream_t st, PfBlkArgs a) {
     MSQ_HIP(hipFuncSetAttribute((const void*)moe_pf_block_kernel<B, GU, T>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
     attr_set = true;
   }
-  const uint32_t grid = ((a.nitems + 7) / 8) * 8 * a.row_chunks;
+  // two row chunks per workgroup while that leaves three workgroups and more per CU (MSQ_MOEP_CHUNKS imposes a count)
+  static const int env_ch = [] { const char* e = getenv("MSQ_MOEP_CHUNKS"); return e && *e ? atoi(e) : 0; }();
+  const uint32_t items8 = ((a.nitems + 7) / 8) * 8;
+  uint32_t ch = env_ch > 0 ? (uint32_t)env_ch : ((size_t)items8 * ((a.row_chunks + 1) / 2) >= (size_t)3 * device_info().cus ? 2u : 1u);
+  ch = std::max(1u, std::min(ch, a.row_chunks));
+  if (a.N % rows_per_item || GU || T > 3) ch = 1;  // (a ragged last chunk clamps its rows: the chunks are then not a fixed stride apart)
+  a.chunks_per_wg = ch;
+  a.row_groups = (a.row_chunks + ch - 1) / ch;
+  const uint32_t grid = items8 * a.row_groups;
   hipLaunchKernelGGL((moe_pf_block_kernel<B, GU, T>), dim3(grid), dim3(64 * pf_blk_waves(T)), pf_blk_lds<B>(T), st, a);
   MSQ_HIP(hipGetLastError());
   return MSQ_OK;
